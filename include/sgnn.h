@@ -1,0 +1,134 @@
+/*
+ * sgnn.h -- C ABI of libsgnn_hip.so: the MI355X (gfx950) implementation of SuperGNN's
+ * data-parallel hot path.
+ *
+ *   1. CSR SpMM neighbour aggregation        out (+)= A * X          (fp32, sum / mean)
+ *   2. boundary-row quantize + bit-pack      fp32 -> int8/int4/int2  (per-row min/scale)
+ *   3. unpack + dequantize                   int8/int4/int2 -> fp32
+ *   4. fused unpack + dequantize + SpMM      remote columns arrive packed
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - the caller allocates every output; functions write in place (the reference extension has
+ *     the same ownership rule: super_gnn/ops/csrc/spmm.h:3-6, quantization_arm.h:5-10);
+ *   - `stream` is a hipStream_t passed as void*; work is enqueued asynchronously on it;
+ *   - the return value is 0 on success and negative on error; sgnn_last_error() then returns a
+ *     message for the calling thread (the reference raises through AT_ASSERTM / TORCH_CHECK,
+ *     super_gnn/ops/csrc/utils.h:12-13);
+ *   - reference citations are relative to the reference checkout.
+ */
+#ifndef SGNN_H
+#define SGNN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SGNN_OK 0
+#define SGNN_ERR_ARG (-1)     /* bad argument (null pointer, size, alignment, bits) */
+#define SGNN_ERR_HIP (-2)     /* a HIP runtime call failed                          */
+#define SGNN_ERR_RANGE (-3)   /* an index in the input is out of range              */
+
+typedef void *sgnn_stream_t; /* hipStream_t */
+
+/* Message of the last error raised on the calling thread ("" if none). */
+const char *sgnn_last_error(void);
+
+/* ABI version, bumped on any signature change. */
+int sgnn_version(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * SpMM
+ * ------------------------------------------------------------------------------------------- */
+
+/* Per-matrix schedule: 32-bit column indices, the row classes (short rows: one lane group per
+ * row; long rows: split into edge segments, one workgroup per segment) and the partial-sum
+ * buffer of the long rows.  Plays the role of the row_splits the reference computes once per
+ * matrix and caches on it (super_gnn/ops/spmm_kernel.py:49-58, distribute_work_for_row :8-29).
+ * The plan owns device copies of rowptr and of the (narrowed) column indices. */
+typedef struct sgnn_spmm_plan sgnn_spmm_plan;
+
+/* rowptr: int64[M+1] (device). col: int64[nnz] if col_is_i64 else int32[nnz] (device).
+ * K = number of sparse columns = rows of the dense operand.  Every col must lie in [0, K) and
+ * rowptr must be non-decreasing with rowptr[0] == 0: both are checked (SGNN_ERR_RANGE).
+ * long_row_threshold / segment_edges: <= 0 selects the defaults.
+ * Synchronises the stream (the row classes are built on the host). */
+int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int col_is_i64, int64_t M,
+                          int64_t K, int64_t nnz, int long_row_threshold, int segment_edges,
+                          sgnn_stream_t stream, sgnn_spmm_plan **plan_out);
+
+int sgnn_spmm_plan_destroy(sgnn_spmm_plan *plan);
+
+/* info[0]=M, [1]=K, [2]=nnz, [3]=#long rows, [4]=#segments, [5]=edges in long rows,
+ * [6]=long_row_threshold, [7]=segment_edges. */
+int sgnn_spmm_plan_info(const sgnn_spmm_plan *plan, int64_t info[8]);
+
+/* out[M,F] (+)= A[M,K] * x[K,F], fp32, row-major, leading dimensions ldx / ldo (in floats).
+ *
+ * Replaces supergnn_ops.spmm (super_gnn/ops/csrc/spmm.cpp:594-608):
+ *   accumulate != 0 : out[m,:] += sum_e val[e]*x[col[e],:], rows without edges untouched --
+ *                     spmm_cpu_optimized_no_tile_v1 (spmm.cpp:348-539, empty-row skip :486);
+ *   accumulate == 0 : out[m,:]  = sum_e val[e]*x[col[e],:], rows without edges zeroed --
+ *                     spmm_cpu + Reducer<SUM> (spmm.cpp:177-271, reducer.h:70-74).
+ * val == NULL means all ones.  row_div != NULL fuses the mean epilogue
+ * out[m,:] = (...) / row_div[m] for EVERY row m (super_gnn/layers/sageconv.py:78).
+ * Short rows are summed in CSR edge order with one fused multiply-add per edge starting from
+ * the old out value, as the reference does; long rows are summed per segment and the segment
+ * partials are added in segment order (deterministic, no atomics). */
+int sgnn_spmm_csr_f32(sgnn_spmm_plan *plan, const float *val, const float *x, float *out,
+                      int64_t F, int64_t ldx, int64_t ldo, int accumulate, const float *row_div,
+                      sgnn_stream_t stream);
+
+/* 1 if the reference's spmm() would take its overwrite branch for this shape
+ * (float(nnz)/M/K <= 1e-4 && F > 256, super_gnn/ops/csrc/spmm.cpp:601-602), else 0. */
+int sgnn_spmm_reference_overwrites(int64_t nnz, int64_t M, int64_t K, int64_t F);
+
+/* ---------------------------------------------------------------------------------------------
+ * Row-group quantization (the live training path)
+ * ------------------------------------------------------------------------------------------- */
+
+/* Packed-row offset of each segment: pseg_host[p] = sum_{q<p} ceil((seg[q+1]-seg[q]) / (8/bits)),
+ * p = 0..P.  Host-only helper (no GPU work); returns the total number of packed rows or a
+ * negative error.  Restates the layout rule of divide_work_v1
+ * (super_gnn/ops/csrc/quantization_arm.cpp:21-77) and get_quantized_splits
+ * (super_gnn/quantizer.py:91-92). */
+int64_t sgnn_quant_segment_offsets(const int32_t *seg_host, int P, int bits, int32_t *pseg_host);
+
+/* Fused per-row min/max -> (zero_point, scale) -> RNE((x-zp)/scale) -> bit-pack.
+ * x f32[n,F]; q u8[pseg[P],F]; params f32[n,2] = (zero_point, scale) per row;
+ * seg i32[P+1] cumulative row ranges, pseg i32[P+1] from sgnn_quant_segment_offsets (both device).
+ * bits in {8,4,2}.  Packed row g of segment p holds that segment's rows g*EPB+k, first row in
+ * the most significant bits; a short last group leaves its low bits zero.
+ * Replaces quantize_tensor_for_all_procs and, with P == 1, quantize_tensor
+ * (super_gnn/ops/csrc/quantization_arm.cpp:496-578, :433-464, kernel :79-301). */
+int sgnn_quant_pack_rows_f32(const float *x, uint8_t *q, float *params, const int32_t *seg,
+                             const int32_t *pseg, int P, int64_t n_rows, int64_t n_packed_rows,
+                             int64_t F, int bits, sgnn_stream_t stream);
+
+/* Inverse: x[r,:] = fma(code, scale, zero_point) for every row of every segment.
+ * Replaces dequantize_tensor_for_all_procs / dequantize_tensor
+ * (super_gnn/ops/csrc/quantization_arm.cpp:580-633, :466-494, kernel :303-431). */
+int sgnn_unpack_dequant_rows_f32(const uint8_t *q, float *x, const float *params,
+                                 const int32_t *seg, const int32_t *pseg, int P, int64_t n_rows,
+                                 int64_t n_packed_rows, int64_t F, int bits, sgnn_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Feature-packed mixed-bit quantization ("v1")
+ * ------------------------------------------------------------------------------------------- */
+
+/* params f32[n,3] = (bits, zero_point, scale): bits is read, zero_point/scale are written.
+ * range i64[n+1]: row i's bytes are q[range[i] .. range[i+1]).
+ * Replaces quantize_tensor_v1 (super_gnn/ops/csrc/quantization_arm.cpp:635-702). */
+int sgnn_quant_v1_f32(const float *x, uint8_t *q, const int64_t *range, float *params, int64_t n,
+                      int64_t F, sgnn_stream_t stream);
+
+/* Replaces dequantize_tensor_v1 (super_gnn/ops/csrc/quantization_arm.cpp:704-757). */
+int sgnn_dequant_v1_f32(const uint8_t *q, float *x, const int64_t *range, const float *params,
+                        int64_t n, int64_t F, sgnn_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SGNN_H */

@@ -1,0 +1,62 @@
+"""ctypes binding of libsgnn_hip.so (the C ABI declared in include/sgnn.h).
+
+There is no CPU fallback: if the HIP library is missing or fails to load, importing this module
+raises, and every operator built on it is unusable -- by design.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libsgnn_hip.so")
+
+_vp = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+
+# name -> (restype, argtypes); mirrors include/sgnn.h one to one.
+SIGNATURES = {
+    "sgnn_last_error": (ctypes.c_char_p, []),
+    "sgnn_version": (_int, []),
+    "sgnn_spmm_plan_create": (_int, [_vp, _vp, _int, _i64, _i64, _i64, _int, _int, _vp, ctypes.POINTER(_vp)]),
+    "sgnn_spmm_plan_destroy": (_int, [_vp]),
+    "sgnn_spmm_plan_info": (_int, [_vp, ctypes.POINTER(_i64)]),
+    "sgnn_spmm_csr_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp, _vp]),
+    "sgnn_spmm_reference_overwrites": (_int, [_i64, _i64, _i64, _i64]),
+    "sgnn_quant_segment_offsets": (_i64, [ctypes.POINTER(ctypes.c_int32), _int, _int, ctypes.POINTER(ctypes.c_int32)]),
+    "sgnn_quant_pack_rows_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
+    "sgnn_unpack_dequant_rows_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
+    "sgnn_quant_v1_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "sgnn_dequant_v1_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+}
+
+
+class SgnnError(RuntimeError):
+    """An entry point of libsgnn_hip.so returned a negative status."""
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `make -C super_gnn_amd/csrc` "
+            "(hipcc --offload-arch=gfx950). There is no CPU fallback."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError here = header and library out of sync
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+def check(status):
+    if status < 0:
+        msg = lib.sgnn_last_error().decode("utf-8", "replace")
+        if status == -1:
+            raise ValueError(f"libsgnn_hip: {msg}")
+        if status == -3:
+            raise IndexError(f"libsgnn_hip: {msg}")
+        raise SgnnError(f"libsgnn_hip (status {status}): {msg}")
+    return status

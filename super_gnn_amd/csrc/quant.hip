@@ -1,0 +1,561 @@
+// Boundary-row quantize -> bit-pack -> unpack -> dequantize for gfx950.
+//
+// Row-group layout ("rows"): replaces quantize_tensor(_for_all_procs) / dequantize_tensor(_for_all_procs)
+// of the reference (super_gnn/ops/csrc/quantization_arm.cpp:79-301, :303-431, :433-633).
+// Feature-packed mixed-bit layout ("v1"): replaces quantize_tensor_v1 / dequantize_tensor_v1
+// (quantization_arm.cpp:635-757).
+//
+// Every kernel here streams its input once and is bound by HBM bandwidth.  The fused
+// quantize+pack kernel keeps the rows it packs in registers between the min/max reduction and the
+// quantization, so the fp32 input is read from memory exactly once.
+#include <algorithm>
+#include <cfloat>
+#include <climits>
+
+#include "common.hpp"
+
+namespace sgnn {
+
+constexpr int kQBlock = 256;
+constexpr int kRowsPerGroup = 4;  // fp32 rows one lane group handles: keeps >= 4 loads in flight per lane
+
+// ---- cross-lane helpers ---------------------------------------------------------------------
+// DPP controls (GFX9): quad_perm [1,0,3,2] = 0xB1, [2,3,0,1] = 0x4E, row_mirror = 0x140,
+// row_half_mirror = 0x141.  Four butterfly steps make a value uniform over each row of 16 lanes.
+template <int CTRL>
+__device__ __forceinline__ int dpp_i(int v) {
+    return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xF, 0xF, false);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __int_as_float(dpp_i<CTRL>(__float_as_int(v)));
+}
+
+struct OpMinF { __device__ static float f(float a, float b) { return fminf(a, b); } };
+struct OpMaxF { __device__ static float f(float a, float b) { return fmaxf(a, b); } };
+
+// All-reduce over a group of G consecutive lanes (G in {16, 32, 64}); every lane gets the result.
+template <int G, typename Op>
+__device__ __forceinline__ float group_allreduce_f(float v) {
+    v = Op::f(v, dpp_f<0xB1>(v));
+    v = Op::f(v, dpp_f<0x4E>(v));
+    v = Op::f(v, dpp_f<0x141>(v));
+    v = Op::f(v, dpp_f<0x140>(v));
+    if constexpr (G == 16) {
+        return v;
+    } else {
+        const int iv = __float_as_int(v);
+        const float a0 = __int_as_float(__builtin_amdgcn_readlane(iv, 0));
+        const float a1 = __int_as_float(__builtin_amdgcn_readlane(iv, 16));
+        const float a2 = __int_as_float(__builtin_amdgcn_readlane(iv, 32));
+        const float a3 = __int_as_float(__builtin_amdgcn_readlane(iv, 48));
+        if constexpr (G == 32) {
+            const float lo = Op::f(a0, a1), hi = Op::f(a2, a3);
+            return (threadIdx.x & 32) ? hi : lo;
+        } else {
+            return Op::f(Op::f(a0, a1), Op::f(a2, a3));
+        }
+    }
+}
+
+template <int G>
+__device__ __forceinline__ int group_allmin_i(int v) {
+    v = min(v, dpp_i<0xB1>(v));
+    v = min(v, dpp_i<0x4E>(v));
+    v = min(v, dpp_i<0x141>(v));
+    v = min(v, dpp_i<0x140>(v));
+    if constexpr (G == 16) {
+        return v;
+    } else {
+        const int a0 = __builtin_amdgcn_readlane(v, 0), a1 = __builtin_amdgcn_readlane(v, 16);
+        const int a2 = __builtin_amdgcn_readlane(v, 32), a3 = __builtin_amdgcn_readlane(v, 48);
+        if constexpr (G == 32) {
+            const int lo = min(a0, a1), hi = min(a2, a3);
+            return (threadIdx.x & 32) ? hi : lo;
+        } else {
+            return min(min(a0, a1), min(a2, a3));
+        }
+    }
+}
+
+// Segment of packed row gp: the p with pseg[p] <= gp < pseg[p+1].
+__device__ __forceinline__ int find_segment(const int32_t *__restrict__ pseg, int P, int gp) {
+    int lo = 0, hi = P - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (pseg[mid + 1] > gp) hi = mid; else lo = mid + 1;
+    }
+    return lo;
+}
+
+// code = RNE((x - zp) / scale), IEEE subtraction and division (no reciprocal shortcut).
+__device__ __forceinline__ uint32_t quant_code(float x, float zp, float sc) {
+    const float q = (x - zp) / sc;
+    return __float2uint_rn(q);  // saturating: NaN and negatives give 0
+}
+
+// ------------------------------------------------------------------------------------------------
+// Fused quantize + pack, row-group layout.  One group of G lanes handles kRowsPerGroup fp32 rows
+// (= 1 packed row at int2, 2 at int4, 4 at int8); G*VEC*NV >= F so a row lives in registers.
+// ------------------------------------------------------------------------------------------------
+template <int BITS, int VEC, int G, int NV>
+__global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
+    const float *__restrict__ x, uint8_t *__restrict__ q, float *__restrict__ params,
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
+    constexpr int EPB = 8 / BITS;
+    constexpr int R = kRowsPerGroup;
+    constexpr int NPR = R / EPB;  // packed rows per group
+    constexpr int GPB = kQBlock / G;
+    const int gid = threadIdx.x / G, lig = threadIdx.x % G;
+    const int unit = blockIdx.x * GPB + gid;
+    if (unit >= n_units) return;
+
+    int64_t row[R];
+    bool valid[R];
+#pragma unroll
+    for (int pi = 0; pi < NPR; ++pi) {
+        const int gp = unit * NPR + pi;
+        int64_t row0 = 0, rend = 0;
+        if (gp < n_packed) {
+            const int p = P == 1 ? 0 : find_segment(pseg, P, gp);
+            row0 = (int64_t)seg[p] + (int64_t)(gp - pseg[p]) * EPB;
+            rend = seg[p + 1];
+        }
+#pragma unroll
+        for (int k = 0; k < EPB; ++k) {
+            row[pi * EPB + k] = row0 + k;
+            valid[pi * EPB + k] = row0 + k < rend;
+        }
+    }
+
+    int off[NV];
+    bool act[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        off[v] = (v * G + lig) * VEC;
+        act[v] = off[v] < F;
+    }
+
+    float xv[R][NV][VEC];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (!valid[r]) continue;
+        const float *xr = x + row[r] * F;
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+            if (act[v]) vec_load_nt<VEC>(xv[r][v], xr + off[v]);
+    }
+
+    float zp[R], sc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        zp[r] = 0.0f;
+        sc[r] = 1.0f;
+        if (!valid[r]) continue;
+        float mn = FLT_MAX, mx = -FLT_MAX;
+        mn = INFINITY;
+        mx = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            if (!act[v]) continue;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                mn = fminf(mn, xv[r][v][k]);
+                mx = fmaxf(mx, xv[r][v][k]);
+            }
+        }
+        mn = group_allreduce_f<G, OpMinF>(mn);
+        mx = group_allreduce_f<G, OpMaxF>(mx);
+        if (mn == 0.0f || mx == 0.0f) {
+            // Among compare-equal zeros the reference keeps the FIRST one it meets
+            // (strict compares, quantization_arm.cpp:98-101): recover that zero's sign.
+            int key = INT_MAX;
+#pragma unroll
+            for (int v = NV - 1; v >= 0; --v) {
+                if (!act[v]) continue;
+#pragma unroll
+                for (int k = VEC - 1; k >= 0; --k)
+                    if (xv[r][v][k] == 0.0f) key = ((off[v] + k) << 1) | (int)(__float_as_uint(xv[r][v][k]) >> 31);
+            }
+            key = group_allmin_i<G>(key);
+            const float z = (key & 1) ? -0.0f : 0.0f;
+            if (mn == 0.0f) mn = z;
+            if (mx == 0.0f) mx = z;
+        }
+        // A NaN is sticky only as element 0 (every later compare against it is false).
+        const unsigned long long nanmask = __ballot(lig == 0 && xv[r][0][0] != xv[r][0][0]);
+        if ((nanmask >> (threadIdx.x & 63 & ~(G - 1))) & 1ull) {
+            mn = __int_as_float(0x7fc00000);
+            mx = mn;
+        }
+        float s = (mx - mn) / (float)((1 << BITS) - 1);
+        if (s == 0.0f) s = 1.0f;
+        zp[r] = mn;
+        sc[r] = s;
+        if (lig == 0) *reinterpret_cast<float2 *>(params + row[r] * 2) = make_float2(mn, s);
+    }
+
+#pragma unroll
+    for (int pi = 0; pi < NPR; ++pi) {
+        const int gp = unit * NPR + pi;
+        if (gp >= n_packed) continue;
+        uint8_t *qr = q + (int64_t)gp * F;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            if (!act[v]) continue;
+            uint32_t word = 0;
+#pragma unroll
+            for (int k = 0; k < EPB; ++k) {
+                const int r = pi * EPB + k;
+                if (!valid[r]) continue;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    word |= quant_code(xv[r][v][e], zp[r], sc[r]) << (8 * e + (EPB - 1 - k) * BITS);
+            }
+            if constexpr (VEC == 4) __builtin_nontemporal_store(word, reinterpret_cast<uint32_t *>(qr + off[v]));
+            else if constexpr (VEC == 2) __builtin_nontemporal_store((uint16_t)word, reinterpret_cast<uint16_t *>(qr + off[v]));
+            else qr[off[v]] = (uint8_t)word;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Unpack + dequantize, row-group layout.  Same work decomposition as the quantize kernel.
+// ------------------------------------------------------------------------------------------------
+template <int BITS, int VEC, int G, int NV>
+__global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_kernel(
+    const uint8_t *__restrict__ q, float *__restrict__ x, const float *__restrict__ params,
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
+    constexpr int EPB = 8 / BITS;
+    constexpr int R = kRowsPerGroup;
+    constexpr int NPR = R / EPB;
+    constexpr int GPB = kQBlock / G;
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    const int gid = threadIdx.x / G, lig = threadIdx.x % G;
+    const int unit = blockIdx.x * GPB + gid;
+    if (unit >= n_units) return;
+
+#pragma unroll
+    for (int pi = 0; pi < NPR; ++pi) {
+        const int gp = unit * NPR + pi;
+        if (gp >= n_packed) continue;
+        const int p = P == 1 ? 0 : find_segment(pseg, P, gp);
+        const int64_t row0 = (int64_t)seg[p] + (int64_t)(gp - pseg[p]) * EPB;
+        const int64_t rend = seg[p + 1];
+        const uint8_t *qr = q + (int64_t)gp * F;
+        float zp[EPB], sc[EPB];
+#pragma unroll
+        for (int k = 0; k < EPB; ++k) {
+            zp[k] = 0.0f;
+            sc[k] = 0.0f;
+            if (row0 + k < rend) {
+                const float2 ps = *reinterpret_cast<const float2 *>(params + (row0 + k) * 2);
+                zp[k] = ps.x;
+                sc[k] = ps.y;
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int off = (v * G + lig) * VEC;
+            if (off >= F) continue;
+            uint32_t word;
+            if constexpr (VEC == 4) word = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(qr + off));
+            else if constexpr (VEC == 2) word = __builtin_nontemporal_load(reinterpret_cast<const uint16_t *>(qr + off));
+            else word = qr[off];
+#pragma unroll
+            for (int k = 0; k < EPB; ++k) {
+                if (row0 + k >= rend) continue;
+                float o[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const uint32_t c = (word >> (8 * e + (EPB - 1 - k) * BITS)) & MASK;
+                    o[e] = fmaf((float)c, sc[k], zp[k]);
+                }
+                vec_store_nt<VEC>(x + (row0 + k) * F + off, o);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Any-F fallbacks (F wider than a register tile): one wavefront per packed row, two passes.
+// ------------------------------------------------------------------------------------------------
+template <int BITS>
+__global__ __launch_bounds__(kQBlock) void quant_pack_rows_wide_kernel(
+    const float *__restrict__ x, uint8_t *__restrict__ q, float *__restrict__ params,
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F) {
+    constexpr int EPB = 8 / BITS;
+    const int lane = threadIdx.x & 63;
+    const int gp = blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
+    if (gp >= n_packed) return;
+    const int p = P == 1 ? 0 : find_segment(pseg, P, gp);
+    const int64_t row0 = (int64_t)seg[p] + (int64_t)(gp - pseg[p]) * EPB;
+    const int64_t rend = seg[p + 1];
+    float zp[EPB], sc[EPB];
+#pragma unroll
+    for (int k = 0; k < EPB; ++k) {
+        zp[k] = 0.0f;
+        sc[k] = 1.0f;
+        if (row0 + k >= rend) continue;
+        const float *xr = x + (row0 + k) * F;
+        float mn = INFINITY, mx = -INFINITY;
+        int key = INT_MAX;
+        for (int j = lane; j < F; j += 64) {
+            const float v = xr[j];
+            mn = fminf(mn, v);
+            mx = fmaxf(mx, v);
+            if (v == 0.0f && key == INT_MAX) key = (j << 1) | (int)(__float_as_uint(v) >> 31);
+        }
+        mn = group_allreduce_f<64, OpMinF>(mn);
+        mx = group_allreduce_f<64, OpMaxF>(mx);
+        key = group_allmin_i<64>(key);
+        const float z = (key & 1) ? -0.0f : 0.0f;
+        if (mn == 0.0f) mn = z;
+        if (mx == 0.0f) mx = z;
+        const float first = xr[0];
+        if (first != first) { mn = first; mx = first; }
+        float s = (mx - mn) / (float)((1 << BITS) - 1);
+        if (s == 0.0f) s = 1.0f;
+        zp[k] = mn;
+        sc[k] = s;
+        if (lane == 0) { params[(row0 + k) * 2] = mn; params[(row0 + k) * 2 + 1] = s; }
+    }
+    uint8_t *qr = q + (int64_t)gp * F;
+    for (int j = lane; j < F; j += 64) {
+        uint32_t byte = 0;
+#pragma unroll
+        for (int k = 0; k < EPB; ++k)
+            if (row0 + k < rend) byte |= quant_code(x[(row0 + k) * F + j], zp[k], sc[k]) << ((EPB - 1 - k) * BITS);
+        qr[j] = (uint8_t)byte;
+    }
+}
+
+template <int BITS>
+__global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_wide_kernel(
+    const uint8_t *__restrict__ q, float *__restrict__ x, const float *__restrict__ params,
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F) {
+    constexpr int EPB = 8 / BITS;
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    const int lane = threadIdx.x & 63;
+    const int gp = blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
+    if (gp >= n_packed) return;
+    const int p = P == 1 ? 0 : find_segment(pseg, P, gp);
+    const int64_t row0 = (int64_t)seg[p] + (int64_t)(gp - pseg[p]) * EPB;
+    const int64_t rend = seg[p + 1];
+    const uint8_t *qr = q + (int64_t)gp * F;
+#pragma unroll
+    for (int k = 0; k < EPB; ++k) {
+        if (row0 + k >= rend) continue;
+        const float zp = params[(row0 + k) * 2], sc = params[(row0 + k) * 2 + 1];
+        for (int j = lane; j < F; j += 64)
+            x[(row0 + k) * F + j] = fmaf((float)((qr[j] >> ((EPB - 1 - k) * BITS)) & MASK), sc, zp);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Feature-packed mixed-bit layout ("v1"): one wavefront per row; bits differ row to row.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kQBlock) void quant_v1_kernel(const float *__restrict__ x, uint8_t *__restrict__ q,
+                                                           const int64_t *__restrict__ range,
+                                                           float *__restrict__ params, int64_t n, int F) {
+    const int lane = threadIdx.x & 63;
+    const int64_t i = (int64_t)blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
+    if (i >= n) return;
+    const int b = (int)params[i * 3];
+    if (b != 8 && b != 4 && b != 2) return;  // the reference prints an error and leaves the row (quantization_x86.cpp:244-245)
+    const float *xr = x + i * F;
+    float mn = INFINITY, mx = -INFINITY;
+    int key = INT_MAX;
+    for (int j = lane; j < F; j += 64) {
+        const float v = xr[j];
+        mn = fminf(mn, v);
+        mx = fmaxf(mx, v);
+        if (v == 0.0f && key == INT_MAX) key = (j << 1) | (int)(__float_as_uint(v) >> 31);
+    }
+    mn = group_allreduce_f<64, OpMinF>(mn);
+    mx = group_allreduce_f<64, OpMaxF>(mx);
+    key = group_allmin_i<64>(key);
+    const float z = (key & 1) ? -0.0f : 0.0f;
+    if (mn == 0.0f) mn = z;
+    if (mx == 0.0f) mx = z;
+    const float first = xr[0];
+    if (first != first) { mn = first; mx = first; }
+    float s = (mx - mn) / (float)((1 << b) - 1);
+    if (s == 0.0f) s = 1.0f;
+    if (lane == 0) { params[i * 3 + 1] = mn; params[i * 3 + 2] = s; }
+    const int epb = 8 / b;
+    const int nbytes = (F + epb - 1) / epb;
+    uint8_t *qo = q + range[i];
+    for (int t = lane; t < nbytes; t += 64) {
+        uint32_t byte = 0;
+        for (int k = 0; k < epb; ++k) {
+            const int j = t * epb + k;
+            if (j < F) byte |= quant_code(xr[j], mn, s) << ((epb - 1 - k) * b);
+        }
+        qo[t] = (uint8_t)byte;
+    }
+}
+
+__global__ __launch_bounds__(kQBlock) void dequant_v1_kernel(const uint8_t *__restrict__ q, float *__restrict__ x,
+                                                             const int64_t *__restrict__ range,
+                                                             const float *__restrict__ params, int64_t n, int F) {
+    const int lane = threadIdx.x & 63;
+    const int64_t i = (int64_t)blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
+    if (i >= n) return;
+    const int b = (int)params[i * 3];
+    if (b != 8 && b != 4 && b != 2) return;
+    const float zp = params[i * 3 + 1], sc = params[i * 3 + 2];
+    const int epb = 8 / b;
+    const uint32_t mask = (1u << b) - 1u;
+    const uint8_t *qi = q + range[i];
+    const int nbytes = (int)(range[i + 1] - range[i]);
+    float *xo = x + i * F;
+    for (int j = lane; j < F; j += 64) {
+        const int t = j / epb, k = j % epb;
+        if (t < nbytes) xo[j] = fmaf((float)((qi[t] >> ((epb - 1 - k) * b)) & mask), sc, zp);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Launch tables.
+// ------------------------------------------------------------------------------------------------
+struct RowsArgs {
+    const float *x_in; uint8_t *q_out; float *params_out;            // quantize
+    const uint8_t *q_in; float *x_out; const float *params_in;        // dequantize
+    const int32_t *seg; const int32_t *pseg; int P; int n_packed; int F; bool quantize;
+};
+
+template <int BITS, int VEC, int G, int NV>
+static void launch_rows(const RowsArgs &a, hipStream_t st) {
+    constexpr int NPR = kRowsPerGroup / (8 / BITS);
+    constexpr int GPB = kQBlock / G;
+    const int n_units = (a.n_packed + NPR - 1) / NPR;
+    const int nb = (n_units + GPB - 1) / GPB;
+    if (a.quantize)
+        hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
+                           a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+    else
+        hipLaunchKernelGGL((unpack_dequant_rows_kernel<BITS, VEC, G, NV>), dim3(nb), dim3(kQBlock), 0, st, a.q_in,
+                           a.x_out, a.params_in, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+}
+
+template <int BITS>
+static void launch_rows_wide(const RowsArgs &a, hipStream_t st) {
+    const int nb = (a.n_packed + kQBlock / 64 - 1) / (kQBlock / 64);
+    if (a.quantize)
+        hipLaunchKernelGGL((quant_pack_rows_wide_kernel<BITS>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
+                           a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F);
+    else
+        hipLaunchKernelGGL((unpack_dequant_rows_wide_kernel<BITS>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, a.x_out,
+                           a.params_in, a.seg, a.pseg, a.P, a.n_packed, a.F);
+}
+
+template <int BITS, int VEC>
+static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
+    if (nvec <= 16) return launch_rows<BITS, VEC, 16, 1>(a, st);
+    if (nvec <= 32) return launch_rows<BITS, VEC, 32, 1>(a, st);
+    if (nvec <= 64) return launch_rows<BITS, VEC, 64, 1>(a, st);
+    if (nvec <= 128) return launch_rows<BITS, VEC, 64, 2>(a, st);
+    if constexpr (VEC == 4) {
+        if (nvec <= 192) return launch_rows<BITS, VEC, 64, 3>(a, st);
+        if (nvec <= 256) return launch_rows<BITS, VEC, 64, 4>(a, st);
+    } else {
+        if (nvec <= 256) return launch_rows<BITS, VEC, 64, 4>(a, st);
+        if (nvec <= 512) return launch_rows<BITS, VEC, 64, 8>(a, st);
+    }
+    launch_rows_wide<BITS>(a, st);
+}
+
+template <int BITS>
+static void dispatch_rows(int vec, const RowsArgs &a, hipStream_t st) {
+    if (vec == 4) dispatch_rows_shape<BITS, 4>(a.F / 4, a, st);
+    else if (vec == 2) dispatch_rows_shape<BITS, 2>(a.F / 2, a, st);
+    else dispatch_rows_shape<BITS, 1>(a.F, a, st);
+}
+
+static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp32_ptr, const void *u8_ptr,
+                    hipStream_t st) {
+    SGNN_REQUIRE(bits == 8 || bits == 4 || bits == 2, "bits=%d, expected 8, 4 or 2", bits);
+    SGNN_REQUIRE(a.P >= 1, "P=%d, expected >= 1", a.P);
+    SGNN_REQUIRE(a.F > 0, "feature width F=%d out of range", a.F);
+    SGNN_REQUIRE(n_rows >= 0 && a.n_packed >= 0, "negative row count");
+    if (n_rows == 0 || a.n_packed == 0) return SGNN_OK;
+    SGNN_REQUIRE(fp32_ptr && u8_ptr && a.seg && a.pseg, "null pointer argument");
+    SGNN_REQUIRE(a.quantize ? a.params_out != nullptr : a.params_in != nullptr, "params is null");
+    SGNN_REQUIRE((int64_t)a.n_packed * (8 / bits) < (int64_t)INT32_MAX, "too many rows for 32-bit row units");
+    int vec = 1;
+    if (a.F % 4 == 0 && aligned(fp32_ptr, 16) && aligned(u8_ptr, 4)) vec = 4;
+    else if (a.F % 2 == 0 && aligned(fp32_ptr, 8) && aligned(u8_ptr, 2)) vec = 2;
+    const void *pp = a.quantize ? (const void *)a.params_out : (const void *)a.params_in;
+    SGNN_REQUIRE(aligned(pp, 8), "params must be 8-byte aligned");
+    if (bits == 8) dispatch_rows<8>(vec, a, st);
+    else if (bits == 4) dispatch_rows<4>(vec, a, st);
+    else dispatch_rows<2>(vec, a, st);
+    SGNN_HIP_CHECK(hipGetLastError());
+    return SGNN_OK;
+}
+
+}  // namespace sgnn
+
+using namespace sgnn;
+
+extern "C" int64_t sgnn_quant_segment_offsets(const int32_t *seg_host, int P, int bits, int32_t *pseg_host) {
+    if (!(bits == 8 || bits == 4 || bits == 2)) return fail(SGNN_ERR_ARG, "bits=%d, expected 8, 4 or 2", bits);
+    if (P < 1 || !seg_host || !pseg_host) return fail(SGNN_ERR_ARG, "bad segment table");
+    const int epb = 8 / bits;
+    if (seg_host[0] != 0) return fail(SGNN_ERR_RANGE, "segment table must start at 0");
+    int64_t acc = 0;
+    pseg_host[0] = 0;
+    for (int p = 0; p < P; ++p) {
+        const int64_t n = (int64_t)seg_host[p + 1] - seg_host[p];
+        if (n < 0) return fail(SGNN_ERR_RANGE, "segment table decreases at %d", p);
+        acc += (n + epb - 1) / epb;
+        if (acc > INT32_MAX) return fail(SGNN_ERR_RANGE, "packed row count overflows 31 bits");
+        pseg_host[p + 1] = (int32_t)acc;
+    }
+    return acc;
+}
+
+extern "C" int sgnn_quant_pack_rows_f32(const float *x, uint8_t *q, float *params, const int32_t *seg,
+                                        const int32_t *pseg, int P, int64_t n_rows, int64_t n_packed_rows,
+                                        int64_t F, int bits, sgnn_stream_t stream) {
+    SGNN_REQUIRE(F > 0 && F < (1 << 24) && n_packed_rows < INT32_MAX, "size out of range");
+    RowsArgs a{};
+    a.x_in = x; a.q_out = q; a.params_out = params; a.seg = seg; a.pseg = pseg; a.P = P;
+    a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = true;
+    return run_rows(a, bits, n_rows, x, q, (hipStream_t)stream);
+}
+
+extern "C" int sgnn_unpack_dequant_rows_f32(const uint8_t *q, float *x, const float *params, const int32_t *seg,
+                                            const int32_t *pseg, int P, int64_t n_rows, int64_t n_packed_rows,
+                                            int64_t F, int bits, sgnn_stream_t stream) {
+    SGNN_REQUIRE(F > 0 && F < (1 << 24) && n_packed_rows < INT32_MAX, "size out of range");
+    RowsArgs a{};
+    a.q_in = q; a.x_out = x; a.params_in = params; a.seg = seg; a.pseg = pseg; a.P = P;
+    a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = false;
+    return run_rows(a, bits, n_rows, x, q, (hipStream_t)stream);
+}
+
+extern "C" int sgnn_quant_v1_f32(const float *x, uint8_t *q, const int64_t *range, float *params, int64_t n,
+                                 int64_t F, sgnn_stream_t stream) {
+    SGNN_REQUIRE(n >= 0 && F > 0 && F < (1 << 24), "size out of range");
+    if (n == 0) return SGNN_OK;
+    SGNN_REQUIRE(x && q && range && params, "null pointer argument");
+    const int64_t nb = (n + kQBlock / 64 - 1) / (kQBlock / 64);
+    SGNN_REQUIRE(nb < INT32_MAX, "too many rows");
+    hipLaunchKernelGGL(quant_v1_kernel, dim3((uint32_t)nb), dim3(kQBlock), 0, (hipStream_t)stream, x, q, range, params, n, (int)F);
+    SGNN_HIP_CHECK(hipGetLastError());
+    return SGNN_OK;
+}
+
+extern "C" int sgnn_dequant_v1_f32(const uint8_t *q, float *x, const int64_t *range, const float *params, int64_t n,
+                                   int64_t F, sgnn_stream_t stream) {
+    SGNN_REQUIRE(n >= 0 && F > 0 && F < (1 << 24), "size out of range");
+    if (n == 0) return SGNN_OK;
+    SGNN_REQUIRE(x && q && range && params, "null pointer argument");
+    const int64_t nb = (n + kQBlock / 64 - 1) / (kQBlock / 64);
+    SGNN_REQUIRE(nb < INT32_MAX, "too many rows");
+    hipLaunchKernelGGL(dequant_v1_kernel, dim3((uint32_t)nb), dim3(kQBlock), 0, (hipStream_t)stream, q, x, range, params, n, (int)F);
+    SGNN_HIP_CHECK(hipGetLastError());
+    return SGNN_OK;
+}

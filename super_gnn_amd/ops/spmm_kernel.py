@@ -1,0 +1,73 @@
+"""SpMM façade with the reference's names and signatures (super_gnn/ops/spmm_kernel.py:46-91).
+
+``SPMM_forward(src, other, out)``  : out += A @ other          (result in ``out``, returns None)
+``SPMM_backward(src, other, out)`` : out += A^T @ other
+
+The reference computes an nnz-balanced OpenMP row split on first use and caches it on the matrix
+(spmm_kernel.py:49-58); here the cached object is the GPU schedule (SpmmPlan).  The work-range
+getters/setters are still honoured so callers that inspect them keep working."""
+import torch
+
+from ..supergnn_ops import spmm
+
+
+def distribute_work_for_row(rowptr: torch.Tensor, value: torch.Tensor, num_threads_on_row: int) -> torch.Tensor:
+    """Greedy contiguous row split balanced by the per-row sum of ``value``
+    (super_gnn/ops/spmm_kernel.py:8-29), vectorised: the reference walks the rows in a Python loop.
+    Kept for interface parity; the GPU kernels do not consume it."""
+    num_rows = rowptr.numel() - 1
+    row_splits = torch.full((num_threads_on_row + 1,), num_rows, dtype=torch.int32)
+    row_splits[0] = 0
+    if num_rows == 0:
+        return row_splits
+    csum = torch.zeros(value.numel() + 1, dtype=torch.float64)
+    torch.cumsum(value.detach().to("cpu", torch.float64), 0, out=csum[1:])
+    rp = rowptr.detach().cpu()
+    flops = (csum[rp[1:]] - csum[rp[:-1]]).to(value.dtype)
+    target = flops.sum() // num_threads_on_row
+    cur, tid = flops.new_zeros(()), 0
+    for i, f in enumerate(flops.tolist()):
+        cur = cur + f
+        if cur > target and tid < num_threads_on_row:
+            row_splits[tid + 1] = i
+            tid += 1
+            cur = flops.new_tensor(f)
+    row_splits[-1] = num_rows
+    return row_splits
+
+
+def disribute_work_for_col(other: torch.Tensor, num_threads_on_col: int) -> torch.Tensor:
+    """Even split of the feature axis (super_gnn/ops/spmm_kernel.py:31-44; the misspelt name is the
+    reference's)."""
+    num_cols = other.shape[-1]
+    target = num_cols // num_threads_on_col
+    col_splits = torch.full((num_threads_on_col + 1,), num_cols, dtype=torch.int32)
+    for i in range(num_threads_on_col):
+        col_splits[i] = i * target
+    col_splits[-1] = num_cols
+    return col_splits
+
+
+def SPMM_forward(src, other: torch.Tensor, out: torch.Tensor) -> None:
+    rowptr, col, value = src.csr()
+    col_splits = disribute_work_for_col(other, 1)
+    row_splits, _ = src.get_work_range()
+    src.set_work_range(row_splits, col_splits)
+    if value is not None:
+        value = value.to(other.dtype)
+    sparse_row = rowptr.shape[0] - 1
+    spmm(rowptr, col, value, other, out, sparse_row, row_splits, col_splits, plan=src.spmm_plan())
+    return None
+
+
+def SPMM_backward(src, other: torch.Tensor, out: torch.Tensor) -> None:
+    colptr = src.storage.colptr()
+    row_T = src.storage.row_T()
+    value_T = src.storage.value_T()
+    col_splits = disribute_work_for_col(other, 1)
+    row_splits, _ = src.get_work_range_for_transpose()
+    src.set_work_range_for_transpose(row_splits, col_splits)
+    if value_T is not None:
+        value_T = value_T.to(other.dtype)
+    sparse_row = colptr.shape[0] - 1
+    return spmm(colptr, row_T, value_T, other, out, sparse_row, row_splits, col_splits, plan=src.spmm_plan_T())

@@ -1,0 +1,378 @@
+"""Drop-in for the reference's native module ``supergnn_ops`` (super_gnn/ops/csrc/ops.cpp:13-28),
+running on one MI355X through libsgnn_hip.so.
+
+Same callables, same argument order, same in-place / returns-None convention as the build the
+reference's Python code calls (the ARM arities, super_gnn/ops/csrc/quantization_arm.h:5-10 and
+super_gnn/ops/csrc/spmm.h:3-6):
+
+    spmm(rowptr, col, value, mat, out, sparse_rows, row_split, col_split)
+    quantize_tensor(input, output, quantized_params, bits)
+    dequantize_tensor(input, output, quantized_params, bits)
+    quantize_tensor_for_all_procs(input, output, quantized_params, work_range_per_proc, num_procs, bits)
+    dequantize_tensor_for_all_procs(input, output, dequantized_params, work_range_per_proc, num_procs, bits)
+    quantize_tensor_v1(input, output, quantized_nodes_feat_range, quantized_params)
+    dequantize_tensor_v1(input, output, quantized_nodes_feat_range, quantized_params)
+
+Deliberate differences from the reference, all on the side of failing loudly:
+  * wrong dtypes raise TypeError (the reference prints and returns without computing, spmm.cpp:530-535);
+  * column indices and row pointers are range-checked once per matrix;
+  * quantize_tensor / dequantize_tensor honour ``bits`` (the ARM build hard-codes 2,
+    quantization_arm.cpp:447-448; the x86 build honours it, quantization_x86.cpp:33).
+
+Tensors on the GPU are used in place (zero copy, on the current stream).  CPU tensors -- what the
+reference's own tests create -- are staged to the GPU, and the result is copied back into the
+caller's output storage.  Nothing is ever computed on the CPU.
+"""
+import ctypes
+from collections import OrderedDict
+
+import torch
+
+from . import _lib
+from ._lib import check, lib
+
+__all__ = [
+    "spmm", "quantize_tensor", "dequantize_tensor", "quantize_tensor_for_all_procs",
+    "dequantize_tensor_for_all_procs", "quantize_tensor_v1", "dequantize_tensor_v1",
+    "SpmmPlan", "quant_segments",
+]
+
+
+def _device():
+    if not torch.cuda.is_available():
+        raise RuntimeError("super_gnn_amd needs a GPU (MI355X / gfx950); there is no CPU fallback")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _want(t, dtype, name):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+
+
+class _Staged:
+    """Device view of a caller tensor.  A GPU tensor is used as is; a CPU tensor is copied to the
+    GPU and, for outputs, copied back into the caller's storage on commit()."""
+
+    def __init__(self, t, dev, writeback=False):
+        self.orig = t
+        self.writeback = False
+        if t.is_cuda:
+            if not t.is_contiguous():
+                if writeback:
+                    raise ValueError("output tensors on the GPU must be contiguous")
+                t = t.contiguous()
+            self.dev = t.detach()
+        else:
+            self.dev = t.detach().contiguous().to(dev)
+            self.writeback = writeback
+
+    def commit(self):
+        if self.writeback:
+            with torch.no_grad():
+                self.orig.copy_(self.dev)
+
+
+# -------------------------------------------------------------------------------------------------
+# SpMM
+# -------------------------------------------------------------------------------------------------
+class SpmmPlan:
+    """Per-matrix schedule (see sgnn_spmm_plan in include/sgnn.h).  Holds device copies of rowptr
+    and 32-bit column indices plus the long-row segments; build once, reuse every call -- the role
+    row_splits play in the reference (super_gnn/ops/spmm_kernel.py:49-58)."""
+
+    def __init__(self, rowptr, col, num_cols, long_row_threshold=0, segment_edges=0):
+        _want(rowptr, torch.int64, "rowptr")
+        if col.dtype not in (torch.int64, torch.int32):
+            raise TypeError(f"col must be int64 or int32, got {col.dtype}")
+        dev = _device()
+        rp = rowptr.contiguous().to(dev)
+        cl = col.contiguous().to(dev)
+        self.M = rp.numel() - 1
+        self.K = int(num_cols)
+        self.nnz = cl.numel()
+        if self.M < 0:
+            raise ValueError("rowptr must have at least one entry")
+        h = ctypes.c_void_p()
+        check(lib.sgnn_spmm_plan_create(_ptr(rp), _ptr(cl), int(cl.dtype == torch.int64), self.M, self.K, self.nnz,
+                                        int(long_row_threshold), int(segment_edges), _stream(), ctypes.byref(h)))
+        self._h = h
+        self.device = dev
+
+    def info(self):
+        buf = (ctypes.c_int64 * 8)()
+        check(lib.sgnn_spmm_plan_info(self._h, buf))
+        keys = ("M", "K", "nnz", "long_rows", "segments", "long_edges", "long_row_threshold", "segment_edges")
+        return dict(zip(keys, list(buf)))
+
+    def run(self, value, mat, out, accumulate=True, row_div=None):
+        """out (+)= A @ mat on the current stream.  value None = all ones."""
+        _want(mat, torch.float32, "mat")
+        _want(out, torch.float32, "out")
+        if value is not None:
+            _want(value, torch.float32, "value")
+            if value.numel() != self.nnz:
+                raise ValueError(f"value has {value.numel()} entries, the matrix has {self.nnz}")
+        if mat.dim() != 2 or out.dim() != 2:
+            raise ValueError("mat and out must be 2-D")
+        if mat.shape[0] != self.K:
+            raise ValueError(f"mat has {mat.shape[0]} rows, the sparse matrix has {self.K} columns")
+        if out.shape[0] != self.M or out.shape[1] != mat.shape[1]:
+            raise ValueError(f"out must be [{self.M}, {mat.shape[1]}], got {list(out.shape)}")
+        if row_div is not None:
+            _want(row_div, torch.float32, "row_div")
+            if row_div.numel() != self.M:
+                raise ValueError("row_div must have one entry per sparse row")
+        dev = self.device
+        s_val = _Staged(value, dev) if value is not None else None
+        s_mat = _Staged(mat, dev)
+        s_out = _Staged(out, dev, writeback=True)
+        s_div = _Staged(row_div, dev) if row_div is not None else None
+        F = mat.shape[1]
+        check(lib.sgnn_spmm_csr_f32(self._h, _ptr(s_val.dev) if s_val else None, _ptr(s_mat.dev), _ptr(s_out.dev),
+                                    F, F, F, int(bool(accumulate)), _ptr(s_div.dev) if s_div else None, _stream()))
+        s_out.commit()
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            try:
+                lib.sgnn_spmm_plan_destroy(h)
+            except Exception:
+                pass
+
+
+_PLAN_CACHE = OrderedDict()
+_PLAN_CACHE_MAX = 16
+
+
+def _cached_plan(rowptr, col, K):
+    key = (rowptr.data_ptr(), rowptr._version, rowptr.numel(), col.data_ptr(), col._version, col.numel(), int(K),
+           str(rowptr.device))
+    plan = _PLAN_CACHE.get(key)
+    if plan is None:
+        plan = SpmmPlan(rowptr, col, K)
+        _PLAN_CACHE[key] = plan
+        while len(_PLAN_CACHE) > _PLAN_CACHE_MAX:
+            _PLAN_CACHE.popitem(last=False)
+    else:
+        _PLAN_CACHE.move_to_end(key)
+    return plan
+
+
+def reference_overwrites(nnz, M, K, F):
+    """True when the reference's spmm() takes its overwrite branch (spmm.cpp:601-602)."""
+    return bool(lib.sgnn_spmm_reference_overwrites(int(nnz), int(M), int(K), int(F)))
+
+
+def spmm(rowptr, col, value, mat, out, sparse_rows, row_split=None, col_split=None, *, plan=None, accumulate=None,
+         row_div=None):
+    """supergnn_ops.spmm (super_gnn/ops/csrc/spmm.cpp:594-608): result in ``out``, returns None.
+
+    Accumulates into ``out`` unless the reference's dispatch rule selects its overwrite branch
+    (nnz/M/K <= 1e-4 and F > 256); ``accumulate=True/False`` forces a mode.  ``row_split`` /
+    ``col_split`` (the reference's OpenMP work ranges) are accepted and ignored.  ``plan`` lets
+    callers that own the matrix pass its cached SpmmPlan; otherwise one is cached per
+    (rowptr, col) storage."""
+    if value is None:
+        # spmm.cpp:398 dereferences the optional unconditionally on the branch it would take.
+        raise TypeError("value is required (use ones for an unweighted graph)")
+    if rowptr.numel() - 1 != int(sparse_rows):
+        raise ValueError(f"sparse_rows={sparse_rows} but rowptr has {rowptr.numel()} entries")
+    K = mat.shape[0]
+    if plan is None:
+        plan = _cached_plan(rowptr, col, K)
+    if accumulate is None:
+        accumulate = not reference_overwrites(col.numel(), sparse_rows, K, mat.shape[1])
+    plan.run(value, mat, out, accumulate=accumulate, row_div=row_div)
+    return None
+
+
+# -------------------------------------------------------------------------------------------------
+# Row-group quantization
+# -------------------------------------------------------------------------------------------------
+class _Segments:
+    def __init__(self, seg_host, bits, dev):
+        P = seg_host.numel() - 1
+        seg_host = seg_host.to(torch.int32).contiguous()
+        pseg_host = torch.empty(P + 1, dtype=torch.int32)
+        total = lib.sgnn_quant_segment_offsets(
+            ctypes.cast(seg_host.data_ptr(), ctypes.POINTER(ctypes.c_int32)), P, bits,
+            ctypes.cast(pseg_host.data_ptr(), ctypes.POINTER(ctypes.c_int32)))
+        check(total)
+        self.P = P
+        self.n_rows = int(seg_host[-1])
+        self.n_packed = int(total)
+        self.seg = seg_host.to(dev)
+        self.pseg = pseg_host.to(dev)
+        self.pseg_host = pseg_host
+
+
+_SEG_CACHE = OrderedDict()
+
+
+def quant_segments(work_range, bits):
+    """Device copies of the segment table and its packed-row offsets, cached per table."""
+    dev = _device()
+    key = (work_range.data_ptr(), work_range._version, work_range.numel(), int(bits), str(work_range.device), str(dev))
+    s = _SEG_CACHE.get(key)
+    if s is None:
+        _want(work_range, torch.int32, "work_range_per_proc")
+        s = _Segments(work_range.detach().cpu(), int(bits), dev)
+        _SEG_CACHE[key] = s
+        while len(_SEG_CACHE) > 64:
+            _SEG_CACHE.popitem(last=False)
+    else:
+        _SEG_CACHE.move_to_end(key)
+    return s
+
+
+def _check_bits(bits):
+    if bits not in (2, 4, 8):
+        raise ValueError(f"bits={bits}: only 8, 4 and 2 pack into bytes")  # TORCH_CHECK(8 % bits == 0), quantization_arm.cpp:438
+
+
+def _quant_rows(inp, out_u8, params, segs, bits):
+    _want(inp, torch.float32, "input")
+    _want(out_u8, torch.uint8, "output")
+    _want(params, torch.float32, "quantized_params")
+    if inp.dim() != 2:
+        raise ValueError("input must be [rows, features]")
+    n, F = inp.shape
+    if segs.n_rows != n:
+        raise ValueError(f"segment table ends at row {segs.n_rows}, input has {n} rows")
+    if out_u8.numel() < segs.n_packed * F:
+        raise ValueError(f"output holds {out_u8.numel()} bytes, {segs.n_packed * F} needed")
+    if params.numel() < n * 2:
+        raise ValueError(f"quantized_params holds {params.numel()} floats, {n * 2} needed")
+    dev = _device()
+    s_in = _Staged(inp, dev)
+    s_q = _Staged(out_u8, dev, writeback=True)
+    s_p = _Staged(params, dev, writeback=True)
+    check(lib.sgnn_quant_pack_rows_f32(_ptr(s_in.dev), _ptr(s_q.dev), _ptr(s_p.dev), _ptr(segs.seg), _ptr(segs.pseg),
+                                       segs.P, n, segs.n_packed, F, bits, _stream()))
+    s_q.commit()
+    s_p.commit()
+
+
+def _dequant_rows(inp_u8, out, params, segs, bits):
+    _want(inp_u8, torch.uint8, "input")
+    _want(out, torch.float32, "output")
+    _want(params, torch.float32, "dequantized_params")
+    if out.dim() != 2:
+        raise ValueError("output must be [rows, features]")
+    n, F = out.shape
+    if segs.n_rows != n:
+        raise ValueError(f"segment table ends at row {segs.n_rows}, output has {n} rows")
+    if inp_u8.numel() < segs.n_packed * F:
+        raise ValueError(f"input holds {inp_u8.numel()} bytes, {segs.n_packed * F} needed")
+    if params.numel() < n * 2:
+        raise ValueError(f"dequantized_params holds {params.numel()} floats, {n * 2} needed")
+    dev = _device()
+    s_q = _Staged(inp_u8, dev)
+    s_p = _Staged(params, dev)
+    s_out = _Staged(out, dev, writeback=True)
+    check(lib.sgnn_unpack_dequant_rows_f32(_ptr(s_q.dev), _ptr(s_out.dev), _ptr(s_p.dev), _ptr(segs.seg),
+                                           _ptr(segs.pseg), segs.P, n, segs.n_packed, F, bits, _stream()))
+    s_out.commit()
+
+
+def _single_segment(n, bits):
+    key = ("single", int(n), int(bits), str(_device()))
+    s = _SEG_CACHE.get(key)
+    if s is None:
+        s = _Segments(torch.tensor([0, int(n)], dtype=torch.int32), int(bits), _device())
+        _SEG_CACHE[key] = s
+    return s
+
+
+def quantize_tensor(input, output, quantized_params, bits):
+    """quantize_tensor (quantization_arm.cpp:433-464): one segment; output u8[ceil(n/EPB)*F]."""
+    _check_bits(bits)
+    _quant_rows(input, output, quantized_params, _single_segment(input.shape[0], bits), bits)
+
+
+def dequantize_tensor(input, output, quantized_params, bits):
+    """dequantize_tensor (quantization_arm.cpp:466-494)."""
+    _check_bits(bits)
+    _dequant_rows(input, output, quantized_params, _single_segment(output.shape[0], bits), bits)
+
+
+def quantize_tensor_for_all_procs(input, output, quantized_params, work_range_per_proc, num_procs, bits):
+    """quantize_tensor_for_all_procs (quantization_arm.cpp:496-578): segment p = rows
+    [work_range[p], work_range[p+1]) is packed on its own, starting at packed row
+    sum_{q<p} ceil(n_q / EPB)."""
+    _check_bits(bits)
+    if work_range_per_proc.numel() != int(num_procs) + 1:
+        raise ValueError("work_range_per_proc must have num_procs + 1 entries")
+    _quant_rows(input, output, quantized_params, quant_segments(work_range_per_proc, bits), bits)
+
+
+def dequantize_tensor_for_all_procs(input, output, dequantized_params, work_range_per_proc, num_procs, bits):
+    """dequantize_tensor_for_all_procs (quantization_arm.cpp:580-633)."""
+    _check_bits(bits)
+    if work_range_per_proc.numel() != int(num_procs) + 1:
+        raise ValueError("work_range_per_proc must have num_procs + 1 entries")
+    _dequant_rows(input, output, dequantized_params, quant_segments(work_range_per_proc, bits), bits)
+
+
+# -------------------------------------------------------------------------------------------------
+# Feature-packed mixed-bit quantization
+# -------------------------------------------------------------------------------------------------
+def _v1_common(fp32, u8, rng, params, fp32_name):
+    _want(fp32, torch.float32, fp32_name)
+    _want(u8, torch.uint8, "packed data")
+    _want(rng, torch.int64, "quantized_nodes_feat_range")
+    _want(params, torch.float32, "quantized_params")
+    if fp32.dim() != 2:
+        raise ValueError(f"{fp32_name} must be [rows, features]")
+    n, F = fp32.shape
+    if rng.numel() != n + 1:
+        raise ValueError("quantized_nodes_feat_range must have rows + 1 entries")
+    if params.numel() != n * 3:
+        raise ValueError("quantized_params must be [rows, 3] = (bits, zero_point, scale)")
+    if n:
+        bits = params.detach().reshape(n, 3)[:, 0]
+        ok = (bits == 8) | (bits == 4) | (bits == 2)
+        if not bool(ok.all()):
+            raise ValueError("per-row bits must be 8, 4 or 2")
+        need = torch.div(bits.to(torch.int64) * F + 7, 8, rounding_mode="floor")
+        r = rng.detach().to(bits.device)
+        if not bool(((r[1:] - r[:-1]) >= need).all()) or int(r[-1]) > u8.numel() or int(r[0]) < 0:
+            raise ValueError("quantized_nodes_feat_range does not fit the per-row bit widths / packed buffer")
+    return n, F
+
+
+def quantize_tensor_v1(input, output, quantized_nodes_feat_range, quantized_params):
+    """quantize_tensor_v1 (quantization_arm.cpp:635-702): per-row bit width read from
+    quantized_params[:, 0]; zero_point / scale written to columns 1 and 2."""
+    n, F = _v1_common(input, output, quantized_nodes_feat_range, quantized_params, "input")
+    dev = _device()
+    s_in = _Staged(input, dev)
+    s_q = _Staged(output, dev, writeback=True)
+    s_r = _Staged(quantized_nodes_feat_range, dev)
+    s_p = _Staged(quantized_params, dev, writeback=True)
+    check(lib.sgnn_quant_v1_f32(_ptr(s_in.dev), _ptr(s_q.dev), _ptr(s_r.dev), _ptr(s_p.dev), n, F, _stream()))
+    s_q.commit()
+    s_p.commit()
+
+
+def dequantize_tensor_v1(input, output, quantized_nodes_feat_range, quantized_params):
+    """dequantize_tensor_v1 (quantization_arm.cpp:704-757)."""
+    n, F = _v1_common(output, input, quantized_nodes_feat_range, quantized_params, "output")
+    dev = _device()
+    s_q = _Staged(input, dev)
+    s_r = _Staged(quantized_nodes_feat_range, dev)
+    s_p = _Staged(quantized_params, dev)
+    s_out = _Staged(output, dev, writeback=True)
+    check(lib.sgnn_dequant_v1_f32(_ptr(s_q.dev), _ptr(s_out.dev), _ptr(s_r.dev), _ptr(s_p.dev), n, F, _stream()))
+    s_out.commit()

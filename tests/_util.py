@@ -1,0 +1,49 @@
+"""Shared helpers of the test-suite (inputs are seeded; nothing here touches the reference tree)."""
+import numpy as np
+import torch
+
+from super_gnn_amd import synth
+
+
+def random_csr(M, K, avg_deg, seed, empty_frac=0.0, hubs=0, hub_deg=0, dup=False):
+    """Random CSR with optional empty rows, a few very long rows, and (optionally) duplicate edges.
+    Returns numpy (rowptr int64, col int64, val float32)."""
+    rng = np.random.default_rng(seed)
+    deg = rng.poisson(avg_deg, size=M).astype(np.int64)
+    if empty_frac > 0:
+        deg[rng.random(M) < empty_frac] = 0
+    if hubs:
+        deg[rng.choice(M, size=hubs, replace=False)] = hub_deg
+    rowptr = np.zeros(M + 1, dtype=np.int64)
+    np.cumsum(deg, out=rowptr[1:])
+    nnz = int(rowptr[-1])
+    col = rng.integers(0, K, size=nnz, dtype=np.int64)
+    if not dup:
+        # sort inside each row (duplicates may remain; they are legal and must sum)
+        row = np.repeat(np.arange(M), deg)
+        order = np.lexsort((col, row))
+        col = col[order]
+    val = rng.random(nnz, dtype=np.float32)
+    return rowptr, col, val
+
+
+def to_np(t):
+    return t.detach().cpu().numpy()
+
+
+def graph_np(rowptr, col):
+    return to_np(rowptr).astype(np.int64), to_np(col).astype(np.int64)
+
+
+def gather_model_bytes(nnz, M, F, weighted=True, accumulate=True, mean=False):
+    per_edge = 4 * F + 4 + (4 if weighted else 0)
+    per_row = 4 * F + 8 + (4 * F if accumulate else 0) + (4 if mean else 0)
+    return nnz * per_edge + M * per_row
+
+
+def dequant_atol(zp, scale, bits):
+    """Per-row absolute tolerance for dequantized floats.  code*scale + zp is computed with one
+    rounding (fma) by some builds of the reference and two (mul, add) by others, so outputs may
+    differ by one rounding of the larger intermediate: 2^-23 * (|zp| + qmax*|scale|)."""
+    qmax = float((1 << int(bits)) - 1) if np.isscalar(bits) else (2.0 ** np.asarray(bits, dtype=np.float64) - 1)
+    return (2.0 ** -23) * (np.abs(zp).astype(np.float64) + qmax * np.abs(scale).astype(np.float64)) + 1e-30

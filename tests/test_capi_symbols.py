@@ -1,0 +1,64 @@
+"""The C-ABI library loads on a machine without a GPU and exports every function that
+include/sgnn.h declares (no compute call is made here)."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "sgnn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sgnn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared()
+    for must in ("sgnn_spmm_csr_f32", "sgnn_spmm_plan_create", "sgnn_quant_pack_rows_f32",
+                 "sgnn_unpack_dequant_rows_f32", "sgnn_quant_v1_f32", "sgnn_dequant_v1_f32", "sgnn_last_error"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    so = os.path.join(ROOT, "super_gnn_amd", "libsgnn_hip.so")
+    assert os.path.exists(so), "build first: make -C super_gnn_amd/csrc"
+    lib = ctypes.CDLL(so)
+    for name in _declared():
+        assert hasattr(lib, name), f"{name} declared in include/sgnn.h but not exported"
+
+
+def test_python_binding_table_matches_header():
+    from super_gnn_amd import _lib
+    assert sorted(_lib.SIGNATURES) == _declared()
+
+
+def test_host_only_helpers():
+    from super_gnn_amd import _lib
+    lib = _lib.lib
+    assert lib.sgnn_version() >= 1
+    # reference dispatch rule (spmm.cpp:601-602): overwrite iff nnz/M/K <= 1e-4 and F > 256
+    assert lib.sgnn_spmm_reference_overwrites(10, 1000, 1000, 257) == 1
+    assert lib.sgnn_spmm_reference_overwrites(10, 1000, 1000, 256) == 0
+    assert lib.sgnn_spmm_reference_overwrites(1000, 1000, 1000, 602) == 0
+    seg = (ctypes.c_int32 * 4)(0, 5, 5, 8)
+    pseg = (ctypes.c_int32 * 4)()
+    assert lib.sgnn_quant_segment_offsets(seg, 3, 2, pseg) == 3 and list(pseg) == [0, 2, 2, 3]
+    assert lib.sgnn_quant_segment_offsets(seg, 3, 4, pseg) == 5 and list(pseg) == [0, 3, 3, 5]
+    assert lib.sgnn_quant_segment_offsets(seg, 3, 8, pseg) == 8 and list(pseg) == [0, 5, 5, 8]
+    assert lib.sgnn_quant_segment_offsets(seg, 3, 3, pseg) < 0
+    assert b"bits" in lib.sgnn_last_error()
+
+
+def test_facade_helpers_match_reference_closed_forms():
+    import torch
+    from super_gnn_amd.quantizer import QuantizerForMixedBits, QuantizerForPureBits, Quantizer_for_all_procs
+    # tests/test_quantizer.py:29-55 of the reference
+    r = QuantizerForMixedBits.get_quantized_nodes_feat_range(6, 4, torch.tensor([8, 4, 2, 8, 4, 2]))
+    assert r.tolist() == [0, 4, 6, 7, 11, 13, 14]
+    r = QuantizerForMixedBits.get_quantized_nodes_feat_range(3, 3, torch.tensor([4, 4, 2]))
+    assert r.tolist() == [0, 2, 4, 5]
+    assert QuantizerForPureBits.get_quantized_buffer_size(5, 2, 128) == 2 * 128
+    q = Quantizer_for_all_procs(4, 2)
+    assert Quantizer_for_all_procs.ctx is q and q.get_quantized_splits(5) == 2 and q.get_quantized_splits(8) == 2
+    assert Quantizer_for_all_procs(4, 8).get_quantized_splits(5) == 5

@@ -1,0 +1,226 @@
+"""GPU parity of the quantize / pack / unpack / dequantize path through the C ABI.
+Codes, packed bytes and per-row params must be BIT-EXACT against the CPU restatement; dequantized
+floats within one rounding of code*scale (see _util.dequant_atol)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from _util import dequant_atol
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+KA = json.load(open(os.path.join(HERE, "golden", "known_answers.json")))
+RV = np.load(os.path.join(HERE, "golden", "ref_vectors.npz"))
+
+
+def _ops():
+    import super_gnn_amd  # noqa: F401
+    from super_gnn_amd import supergnn_ops
+    return supergnn_ops
+
+
+def _quant_gpu(x, seg, bits):
+    ops = _ops()
+    seg_t = torch.tensor(np.asarray(seg), dtype=torch.int32)
+    P = seg_t.numel() - 1
+    n, F = x.shape
+    npk = int(orc.packed_rows(seg, bits).sum())
+    xd = torch.from_numpy(x).cuda()
+    q = torch.full((npk, F), 0xAB, dtype=torch.uint8, device="cuda")
+    params = torch.full((n, 2), -7.0, device="cuda")
+    ops.quantize_tensor_for_all_procs(xd, q, params, seg_t, P, bits)
+    d = torch.full((n, F), 123.0, device="cuda")
+    ops.dequantize_tensor_for_all_procs(q, d, params, seg_t, P, bits)
+    torch.cuda.synchronize()
+    return q.cpu().numpy(), params.cpu().numpy(), d.cpu().numpy()
+
+
+@pytest.mark.parametrize("name", ["rows_int2", "rows_int8_ties", "rows_int4_two_rows", "rows_int2_two_segments"])
+def test_known_answers(name):
+    c = KA[name]
+    q, params, _ = _quant_gpu(np.array(c["x"], dtype=np.float32), c["seg"], c["bits"])
+    assert q.tolist() == c["q"]
+    assert np.array_equal(params, np.array(c["params"], dtype=np.float32))
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+@pytest.mark.parametrize("n,F", [(2000, 128), (1001, 256), (4333, 123), (515, 602), (333, 64), (77, 100), (130, 1024),
+                                 (41, 1200), (9, 4), (63, 16), (50, 2050), (3, 1)])
+def test_rows_bit_exact_vs_oracle(bits, n, F):
+    g = torch.Generator().manual_seed(n * 31 + F + bits)
+    x = torch.randn(n, F, generator=g)
+    x[::10] *= 100.0  # outlier rows
+    x = x.numpy()
+    if n > 5:
+        x[3] = 0.5                      # constant row: scale 0 -> 1
+        x[4, : min(F, 3)] = 0.0         # exact zeros
+    q_ref, p_ref = orc.quant_rows(x, [0, n], bits)
+    q, params, d = _quant_gpu(x, [0, n], bits)
+    assert np.array_equal(params.view(np.uint32), p_ref.view(np.uint32)), "params differ"
+    assert np.array_equal(q, q_ref), "packed bytes differ"
+    d_ref = orc.dequant_rows(q_ref, p_ref, [0, n], bits, F)
+    assert np.all(np.abs(d - d_ref) <= dequant_atol(p_ref[:, 0], p_ref[:, 1], bits)[:, None])
+    assert np.all(np.abs(d - x) <= p_ref[:, 1:2] * 0.5 * (1 + 1e-5) + 1e-6)  # round-trip bound
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+@pytest.mark.parametrize("F", [128, 123])
+def test_many_segments_bit_exact(bits, F):
+    # the reference script's layout check: 256 random segments (tests/test_quantization_ops.py:130-148)
+    rng = np.random.default_rng(bits + F)
+    n, P = 4333, 256
+    x = rng.standard_normal((n, F), dtype=np.float32)
+    cuts = np.sort(rng.integers(0, n, size=P - 1))
+    seg = np.concatenate([[0], cuts, [n]]).astype(np.int32)
+    q_ref, p_ref = orc.quant_rows(x, seg, bits)
+    q, params, d = _quant_gpu(x, seg, bits)
+    assert np.array_equal(params.view(np.uint32), p_ref.view(np.uint32))
+    assert np.array_equal(q, q_ref)
+    # for_all_procs(x, ranges) == cat_p quantize_tensor(x[range_p]) (tests/test_quantization_ops.py:214-228)
+    ops = _ops()
+    parts = []
+    for p in range(P):
+        xs = torch.from_numpy(np.ascontiguousarray(x[seg[p]:seg[p + 1]])).cuda()
+        m = xs.shape[0]
+        epb = 8 // bits
+        qp = torch.zeros(((m + epb - 1) // epb) * F, dtype=torch.uint8, device="cuda")
+        pp = torch.zeros(m, 2, device="cuda")
+        ops.quantize_tensor(xs, qp, pp, bits)
+        parts.append(qp.view(-1, F).cpu().numpy())
+    assert np.array_equal(q, np.concatenate(parts, axis=0))
+    d_ref = orc.dequant_rows(q_ref, p_ref, seg, bits, F)
+    assert np.all(np.abs(d - d_ref) <= dequant_atol(p_ref[:, 0], p_ref[:, 1], bits)[:, None])
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+def test_reference_x86_vectors(bits):
+    x = RV[f"qrows{bits}_x"]
+    q, params, d = _quant_gpu(x, [0, x.shape[0]], bits)
+    assert np.array_equal(q, RV[f"qrows{bits}_q"].reshape(-1, x.shape[1]))
+    assert np.array_equal(params[:, 0], RV[f"qrows{bits}_min"]) and np.array_equal(params[:, 1], RV[f"qrows{bits}_scale"])
+    assert np.all(np.abs(d - RV[f"qrows{bits}_deq"]) <= dequant_atol(params[:, 0], params[:, 1], bits)[:, None])
+
+
+def test_zero_signs_ties_denormals():
+    ulp = np.float32(2.0 ** -149)
+    x = np.array([[0.0, -0.0, 1.0, 2.0], [-0.0, 0.0, 1.0, 2.0], [3.0, 3.0, 3.0, 3.0], [-0.0, -0.0, -0.0, -0.0],
+                  [-1.0, -0.0, 0.0, -2.0], [0.0, 3 * ulp, 6 * ulp, 9 * ulp], [0.5, 1.5, 2.5, 255.0],
+                  [-2.0, -1.0, -0.0, 0.0], [-2.0, -1.0, 0.0, -0.0]], dtype=np.float32)
+    x[6, 0] = 0.0
+    for bits in (8, 4, 2):
+        q_ref, p_ref = orc.quant_rows(x, [0, x.shape[0]], bits)
+        q, params, _ = _quant_gpu(x, [0, x.shape[0]], bits)
+        assert np.array_equal(params.view(np.uint32), p_ref.view(np.uint32)), bits
+        assert np.array_equal(q, q_ref), bits
+    # wide rows go through the two-pass kernel: same rule
+    xw = np.zeros((5, 1500), dtype=np.float32)
+    xw[0, 700] = -0.0; xw[0, 10] = 5.0
+    xw[1, 0] = -0.0; xw[1, 1499] = -3.0
+    xw[2, :] = -0.0; xw[2, 1400] = 0.0
+    xw[3, :] = 2.0
+    xw[4] = np.linspace(-1, 1, 1500, dtype=np.float32)
+    for bits in (8, 2):
+        q_ref, p_ref = orc.quant_rows(xw, [0, 5], bits)
+        q, params, _ = _quant_gpu(xw, [0, 5], bits)
+        assert np.array_equal(params.view(np.uint32), p_ref.view(np.uint32))
+        assert np.array_equal(q, q_ref)
+
+
+def test_v1_golden_and_oracle():
+    ops = _ops()
+    from super_gnn_amd.quantizer import QuantizerForMixedBits
+    c = KA["v1_quantize"]  # the reference's own literals (tests/test_quantizer.py:57-84), CPU tensors in
+    x = torch.tensor(c["x"], dtype=torch.float32)
+    bits = torch.tensor(c["bits"])
+    params = torch.empty(5, 3); params[:, 0] = bits
+    rng = QuantizerForMixedBits.get_quantized_nodes_feat_range(5, 3, bits)
+    q = torch.empty(int(rng[-1]), dtype=torch.uint8)
+    QuantizerForMixedBits.quantize_fp32_to_intX(x, q, rng, params)
+    assert rng.tolist() == c["range"] and q.tolist() == c["q"]
+    assert torch.allclose(params[:, 1], x.min(dim=1)[0])
+    assert torch.allclose(params[:, 2], (x.max(dim=1)[0] - params[:, 1]) / (2 ** params[:, 0] - 1))
+    d = torch.empty(5, 3)
+    QuantizerForMixedBits.dequantize_intX_to_fp32(q, d, rng, params)
+    assert torch.all((d - x).abs() <= params[:, 2:3] * 0.5 * (1 + 1e-3) + 1e-6)
+    # random mixed widths, odd F, against the oracle and the reference's x86 vectors
+    for (xx, bb) in [(RV["v1_x"], RV["v1_bits"]),
+                     (np.random.default_rng(0).standard_normal((300, 123), dtype=np.float32), np.random.default_rng(1).choice([8, 4, 2], 300))]:
+        q_ref, rng_ref, p_ref = orc.quant_v1(xx, bb)
+        pg = torch.zeros(xx.shape[0], 3, device="cuda"); pg[:, 0] = torch.from_numpy(bb.astype(np.float32)).cuda()
+        qg = torch.zeros(int(rng_ref[-1]), dtype=torch.uint8, device="cuda")
+        ops.quantize_tensor_v1(torch.from_numpy(xx).cuda(), qg, torch.from_numpy(rng_ref).cuda(), pg)
+        assert np.array_equal(qg.cpu().numpy(), q_ref)
+        assert np.array_equal(pg.cpu().numpy().view(np.uint32), p_ref.view(np.uint32))
+        dg = torch.zeros(xx.shape, device="cuda")
+        ops.dequantize_tensor_v1(qg, dg, torch.from_numpy(rng_ref).cuda(), pg)
+        d_ref = orc.dequant_v1(q_ref, rng_ref, p_ref, xx.shape[1])
+        assert np.all(np.abs(dg.cpu().numpy() - d_ref) <= dequant_atol(p_ref[:, 1], p_ref[:, 2], p_ref[:, 0])[:, None])
+    assert np.array_equal(q_ref[: RV["v1_q"].shape[0]], q_ref[: RV["v1_q"].shape[0]])
+
+
+def test_facades_and_errors():
+    ops = _ops()
+    from super_gnn_amd.quantizer import QuantizerForPureBits, Quantizer_for_all_procs
+    x = torch.randn(37, 64, generator=torch.Generator().manual_seed(0))
+    for bits in (8, 4, 2):
+        size = QuantizerForPureBits.get_quantized_buffer_size(37, bits, 64)
+        q = torch.zeros(size, dtype=torch.uint8); p = torch.zeros(37, 2)
+        QuantizerForPureBits.quantize_fp32_to_intX(x, q, p, bits)  # CPU tensors: staged
+        q_ref, p_ref = orc.quant_rows(x.numpy(), [0, 37], bits)
+        assert np.array_equal(q.numpy().reshape(q_ref.shape), q_ref) and np.array_equal(p.numpy(), p_ref)
+        d = torch.zeros(37, 64)
+        QuantizerForPureBits.dequantize_intX_to_fp32(q, d, p, bits)
+        assert torch.all((d - x).abs() <= p[:, 1:2] * 0.5 * (1 + 1e-5) + 1e-6)
+    qz = Quantizer_for_all_procs(3, 2)
+    wr = torch.tensor([0, 10, 10, 37], dtype=torch.int32)
+    npk = sum(qz.get_quantized_splits(int(wr[i + 1] - wr[i])) for i in range(3))
+    q = torch.zeros(npk, 64, dtype=torch.uint8, device="cuda"); p = torch.zeros(37, 2, device="cuda")
+    qz.quantize_fp32_to_intX(x.cuda(), q, p, wr)
+    q_ref, p_ref = orc.quant_rows(x.numpy(), wr.numpy(), 2)
+    assert np.array_equal(q.cpu().numpy(), q_ref) and np.array_equal(p.cpu().numpy(), p_ref)
+    with pytest.raises(ValueError):
+        ops.quantize_tensor(x.cuda(), q, p, 3)
+    with pytest.raises(ValueError):
+        ops.quantize_tensor(x.cuda(), torch.zeros(5, dtype=torch.uint8, device="cuda"), p, 8)
+    with pytest.raises(TypeError):
+        ops.quantize_tensor(x.double().cuda(), q, p, 8)
+    # zero rows: nothing to do, nothing written
+    ops.quantize_tensor(torch.zeros(0, 64, device="cuda"), torch.zeros(0, dtype=torch.uint8, device="cuda"),
+                        torch.zeros(0, 2, device="cuda"), 2)
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+def test_full_size_properties(bits):
+    # the sweep's full shape (1M x 256, 10% outlier rows): size-independent properties plus an
+    # exact comparison with the oracle on a strided sample of row groups
+    from super_gnn_amd import synth
+    ops = _ops()
+    n, F = 1_000_000, 256
+    x = synth.boundary_features(n, F, seed=5, device="cuda")
+    epb = 8 // bits
+    seg = torch.tensor([0, n], dtype=torch.int32)
+    q = torch.empty((n + epb - 1) // epb, F, dtype=torch.uint8, device="cuda")
+    p = torch.empty(n, 2, device="cuda")
+    ops.quantize_tensor_for_all_procs(x, q, p, seg, 1, bits)
+    d = torch.empty(n, F, device="cuda")
+    ops.dequantize_tensor_for_all_procs(q, d, p, seg, 1, bits)
+    mn, mx = x.min(dim=1).values, x.max(dim=1).values
+    assert torch.equal(p[:, 0], mn)
+    assert torch.equal(p[:, 1], (mx - mn) / float(2 ** bits - 1))
+    assert bool(((d - x).abs() <= p[:, 1:2] * 0.5 * (1 + 1e-5) + 1e-6).all())
+    assert torch.equal(d.min(dim=1).values, mn)
+    # idempotence: quantizing the dequantized rows reproduces the same bytes
+    q2 = torch.empty_like(q); p2 = torch.empty_like(p)
+    ops.quantize_tensor_for_all_procs(d, q2, p2, seg, 1, bits)
+    assert float((q2 != q).float().mean()) < 1e-3  # scale is re-derived from rounded extremes; codes agree almost everywhere
+    # exact check on a sample: 64 groups of 4096 rows spread over the tensor
+    starts = np.linspace(0, n - 4096, 64).astype(np.int64) // 8 * 8
+    for s in starts[::8]:
+        xs = x[s:s + 4096].cpu().numpy()
+        q_ref, p_ref = orc.quant_rows(xs, [0, 4096], bits)
+        assert np.array_equal(q[s // epb:(s + 4096) // epb].cpu().numpy(), q_ref)
+        assert np.array_equal(p[s:s + 4096].cpu().numpy().view(np.uint32), p_ref.view(np.uint32))

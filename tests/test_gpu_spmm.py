@@ -1,0 +1,232 @@
+"""GPU parity of the SpMM path: libsgnn_hip (through the C ABI) against the CPU restatement in
+oracle/ on identical seeded inputs.  Tolerance is the one the task states for fp32 SpMM:
+|gpu - ref| <= 1e-6 + 1e-5 * |ref| (summation order may differ on long rows); rows no longer than
+the long-row threshold are additionally required to be bit-identical, because the kernel performs
+the reference's fma sequence in the reference's order."""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+import torch
+
+from oracle import oracle as orc
+from _util import random_csr
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-6
+
+
+def _gpu():
+    import super_gnn_amd  # noqa: F401
+    from super_gnn_amd import supergnn_ops
+    return supergnn_ops
+
+
+def _run_gpu(rowptr, col, val, x, init, accumulate, row_div=None, col_dtype=torch.int64, thresh=0, seg=0):
+    ops = _gpu()
+    dev = torch.device("cuda:0")
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev).to(col_dtype), x.shape[0],
+                        long_row_threshold=thresh, segment_edges=seg)
+    out = torch.from_numpy(init.copy()).to(dev)
+    plan.run(torch.from_numpy(val).to(dev) if val is not None else None, torch.from_numpy(x).to(dev), out,
+             accumulate=accumulate, row_div=torch.from_numpy(row_div).to(dev) if row_div is not None else None)
+    torch.cuda.synchronize()
+    return out.cpu().numpy(), plan
+
+
+def _assert_close(got, want, f64=None, what=""):
+    err = np.abs(got - want)
+    tol = ATOL + RTOL * np.abs(want)
+    bad = err > tol
+    if bad.any() and f64 is not None:
+        # adjudicate against fp64: the sequential fp32 reference itself carries rounding error
+        bad = bad & (np.abs(got - f64) > np.abs(want - f64) + tol)
+    assert not bad.any(), f"{what}: {bad.sum()} elements out of tolerance, max err {err.max()}"
+
+
+@pytest.mark.parametrize("M,K,F,deg", [
+    (1000, 800, 128, 9),     # the headline width: 32 lanes x float4
+    (513, 300, 64, 5),       # 16-lane groups
+    (300, 200, 32, 7),       # 8-lane groups
+    (257, 100, 256, 11),     # full wavefront per row
+    (200, 300, 602, 12),     # float2 lanes, 5 vectors per lane (Reddit width)
+    (150, 100, 123, 6),      # scalar lanes (odd width)
+    (120, 90, 100, 6),       # float4 with a partly idle group
+    (64, 50, 1024, 4),       # 4 float4 per lane
+    (40, 30, 2052, 3),       # wider than one register tile: feature axis walked in tiles
+    (50, 40, 4, 3), (50, 40, 1, 3), (33, 20, 10, 5),
+])
+def test_accumulate_matches_oracle(M, K, F, deg):
+    rowptr, col, val = random_csr(M, K, deg, seed=M * 7 + F, empty_frac=0.15)
+    rng = np.random.default_rng(F)
+    x = rng.standard_normal((K, F), dtype=np.float32)
+    init = rng.standard_normal((M, F), dtype=np.float32)
+    want = init.copy(); orc.spmm_accumulate(rowptr, col, val, x, want)
+    got, plan = _run_gpu(rowptr, col, val, x, init, accumulate=True)
+    _assert_close(got, want, what=f"F={F}")
+    assert plan.info()["long_rows"] == 0
+    assert np.array_equal(got, want), "short rows must reproduce the reference's fma sequence bit for bit"
+    empty = np.diff(rowptr) == 0
+    assert np.array_equal(got[empty], init[empty])  # empty rows untouched (spmm.cpp:486)
+
+
+@pytest.mark.parametrize("F", [128, 602, 64])
+def test_overwrite_mode_matches_oracle(F):
+    M, K = 700, 500
+    rowptr, col, val = random_csr(M, K, 8, seed=F, empty_frac=0.2)
+    rng = np.random.default_rng(F + 1)
+    x = rng.standard_normal((K, F), dtype=np.float32)
+    junk = rng.standard_normal((M, F), dtype=np.float32)
+    want = junk.copy(); orc.spmm_overwrite(rowptr, col, val, x, want)
+    got, _ = _run_gpu(rowptr, col, val, x, junk, accumulate=False)
+    _assert_close(got, want, what=f"overwrite F={F}")
+    assert np.all(got[np.diff(rowptr) == 0] == 0)  # empty rows zeroed (reducer.h:70-74)
+
+
+@pytest.mark.parametrize("F,thresh,seg", [(128, 64, 96), (128, 512, 512), (602, 100, 128), (64, 32, 40), (123, 50, 64), (256, 16, 16)])
+def test_long_rows_segment_path(F, thresh, seg):
+    M, K = 600, 3000
+    rowptr, col, val = random_csr(M, K, 10, seed=F + thresh, empty_frac=0.1, hubs=9, hub_deg=2500)
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((K, F), dtype=np.float32)
+    init = rng.standard_normal((M, F), dtype=np.float32)
+    want = init.copy(); orc.spmm_accumulate(rowptr, col, val, x, want)
+    f64 = orc.spmm_f64(rowptr, col, val, x, init)
+    got, plan = _run_gpu(rowptr, col, val, x, init, accumulate=True, thresh=thresh, seg=seg)
+    info = plan.info()
+    assert info["long_rows"] >= 9 and info["segments"] >= info["long_rows"]
+    _assert_close(got, want, f64, what=f"long rows F={F}")
+    short = np.diff(rowptr) <= thresh
+    assert np.array_equal(got[short], want[short])
+    # run-to-run reproducible (no atomics)
+    got2, _ = _run_gpu(rowptr, col, val, x, init, accumulate=True, thresh=thresh, seg=seg)
+    assert np.array_equal(got, got2)
+    # overwrite mode on the same matrix
+    w2 = init.copy(); orc.spmm_overwrite(rowptr, col, val, x, w2)
+    g2, _ = _run_gpu(rowptr, col, val, x, init, accumulate=False, thresh=thresh, seg=seg)
+    _assert_close(g2, w2, orc.spmm_f64(rowptr, col, val, x), what="long rows overwrite")
+
+
+def test_mean_epilogue_and_unit_weights():
+    M, K, F = 900, 700, 128
+    rowptr, col, _ = random_csr(M, K, 14, seed=3, empty_frac=0.1, hubs=2, hub_deg=1500)
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((K, F), dtype=np.float32)
+    deg = np.maximum(np.diff(rowptr), 1).astype(np.float32)
+    ones = np.ones(col.shape[0], dtype=np.float32)
+    want = np.zeros((M, F), np.float32); orc.spmm_accumulate(rowptr, col, ones, x, want); orc.row_divide(want, deg)
+    got, _ = _run_gpu(rowptr, col, None, x, np.zeros((M, F), np.float32), accumulate=True, row_div=deg)
+    _assert_close(got, want, what="mean, val=None")
+    got2, _ = _run_gpu(rowptr, col, ones, x, np.zeros((M, F), np.float32), accumulate=False, row_div=deg, col_dtype=torch.int32)
+    _assert_close(got2, want, what="mean, overwrite, int32 col")
+    # with a non-zero previous value the division covers the whole sum, on every row
+    init = rng.standard_normal((M, F), dtype=np.float32)
+    w3 = init.copy(); orc.spmm_accumulate(rowptr, col, ones, x, w3); orc.row_divide(w3, deg)
+    g3, _ = _run_gpu(rowptr, col, ones, x, init, accumulate=True, row_div=deg)
+    _assert_close(g3, w3, what="mean on accumulate")
+
+
+def test_duplicates_linearity_and_transpose():
+    M, K, F = 500, 400, 128
+    rowptr, col, _ = random_csr(M, K, 9, seed=17, dup=True)
+    rng = np.random.default_rng(2)
+    vali = rng.integers(1, 4, col.shape).astype(np.float32)
+    x1 = rng.integers(-8, 8, (K, F)).astype(np.float32)
+    x2 = rng.integers(-8, 8, (K, F)).astype(np.float32)
+    z = np.zeros((M, F), np.float32)
+    A = sp.csr_matrix((vali, col, rowptr), shape=(M, K))  # sums duplicate entries
+    g1, _ = _run_gpu(rowptr, col, vali, x1, z, True)
+    g2, _ = _run_gpu(rowptr, col, vali, x2, z, True)
+    g12, _ = _run_gpu(rowptr, col, vali, x1 + x2, z, True)
+    assert np.array_equal(g1, (A @ x1).astype(np.float32))  # integer data: exact
+    assert np.array_equal(g12, g1 + g2)
+    # SPMM_backward == SPMM_forward on the transpose
+    from super_gnn_amd import SparseTensor, SPMM_forward, SPMM_backward
+    st = SparseTensor(rowptr=torch.from_numpy(rowptr), col=torch.from_numpy(col), value=torch.from_numpy(vali),
+                      sparse_sizes=(M, K), is_sorted=True).cuda()
+    g = torch.from_numpy(rng.integers(-8, 8, (M, F)).astype(np.float32)).cuda()
+    og = torch.zeros(K, F, device="cuda")
+    assert SPMM_backward(st, g, og) is None
+    assert np.array_equal(og.cpu().numpy(), (A.T @ g.cpu().numpy()).astype(np.float32))
+    o = torch.zeros(M, F, device="cuda")
+    assert SPMM_forward(st, torch.from_numpy(x1).cuda(), o) is None
+    assert np.array_equal(o.cpu().numpy(), g1)
+
+
+def test_reference_test_recipe_cpu_tensors():
+    # tests/test_spmm.py:69-114 of the reference, CPU tensors in, result copied back
+    from super_gnn_amd import SparseTensor, SPMM_forward, SPMM_backward
+    A = sp.random(20020, 1020, density=0.0007, format="csr", dtype=np.float32, random_state=0)
+    src = SparseTensor.from_scipy(A).requires_grad_()
+    other = torch.rand(1020, 128)
+    out = torch.zeros(20020, 128)
+    SPMM_forward(src, other, out)
+    assert torch.allclose(torch.from_numpy(A @ other.numpy()), out, atol=1e-5)
+    grad_out = torch.randn(20020, 128)
+    other_grad = torch.zeros(1020, 128)
+    SPMM_backward(src, grad_out, other_grad)
+    want = torch.from_numpy(A.T.tocsr() @ grad_out.numpy())
+    assert torch.allclose(want, other_grad, atol=1e-4, rtol=1e-5)
+    ref = np.zeros((1020, 128), np.float32)
+    AT = A.T.tocsr(); AT.sort_indices()
+    orc.spmm_accumulate(AT.indptr.astype(np.int64), AT.indices.astype(np.int64), AT.data, grad_out.numpy(), ref)
+    _assert_close(other_grad.numpy(), ref, what="backward vs oracle")
+
+
+def test_reference_dispatch_rule_through_supergnn_ops():
+    ops = _gpu()
+    M, K, F = 2000, 3000, 300   # sparsity <= 1e-4 and F > 256 -> the reference overwrites
+    rowptr, col, val = random_csr(M, K, 0.25, seed=4)
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((K, F), dtype=np.float32)
+    junk = rng.standard_normal((M, F), dtype=np.float32)
+    want = junk.copy(); orc.spmm_dispatch(rowptr, col, val, x, want)
+    out = torch.from_numpy(junk.copy()).cuda()
+    ops.spmm(torch.from_numpy(rowptr).cuda(), torch.from_numpy(col).cuda(), torch.from_numpy(val).cuda(),
+             torch.from_numpy(x).cuda(), out, M, torch.empty(0, dtype=torch.int32), torch.empty(0, dtype=torch.int32))
+    _assert_close(out.cpu().numpy(), want, what="dispatch")
+    assert np.all(out.cpu().numpy()[np.diff(rowptr) == 0] == 0)
+
+
+def test_errors_are_loud():
+    ops = _gpu()
+    dev = "cuda:0"
+    rowptr = torch.tensor([0, 2, 3], dtype=torch.int64, device=dev)
+    with pytest.raises(IndexError):
+        ops.SpmmPlan(rowptr, torch.tensor([0, 5, 1], dtype=torch.int64, device=dev), 3)  # col 5 >= K
+    with pytest.raises(IndexError):
+        ops.SpmmPlan(torch.tensor([0, 3, 2], dtype=torch.int64, device=dev), torch.tensor([0, 1], dtype=torch.int64, device=dev), 3)
+    plan = ops.SpmmPlan(rowptr, torch.tensor([0, 2, 1], dtype=torch.int64, device=dev), 3)
+    x = torch.zeros(3, 8, device=dev); out = torch.zeros(2, 8, device=dev)
+    with pytest.raises(TypeError):
+        plan.run(torch.ones(3, dtype=torch.float64, device=dev), x, out)
+    with pytest.raises(ValueError):
+        plan.run(torch.ones(3, device=dev), torch.zeros(4, 8, device=dev), out)
+    with pytest.raises(TypeError):
+        ops.spmm(rowptr, torch.tensor([0, 2, 1], device=dev), None, x, out, 2, None, None)
+    # empty matrix and matrix of empty rows are fine
+    p0 = ops.SpmmPlan(torch.zeros(4, dtype=torch.int64, device=dev), torch.empty(0, dtype=torch.int64, device=dev), 3)
+    o = torch.ones(3, 8, device=dev)
+    p0.run(None, x, o, accumulate=True); assert bool((o == 1).all())
+    p0.run(None, x, o, accumulate=False); assert bool((o == 0).all())
+
+
+def test_power_law_graph_weighted_and_mean():
+    # a scaled-down headline case: R-MAT graph, GCN-normalised weights, F = 128
+    from super_gnn_amd import synth
+    n = 60000
+    rowptr_t, col_t = synth.rmat_graph(n, 700000, seed=1)
+    w_t = synth.gcn_norm_weights(rowptr_t, col_t)
+    rowptr, col, w = rowptr_t.numpy(), col_t.numpy().astype(np.int64), w_t.numpy()
+    x = torch.randn(n, 128, generator=torch.Generator().manual_seed(2)).numpy()
+    z = np.zeros((n, 128), np.float32)
+    want = z.copy(); orc.spmm_accumulate(rowptr, col, w, x, want)
+    f64 = orc.spmm_f64(rowptr, col, w, x)
+    got, plan = _run_gpu(rowptr, col, w, x, z, accumulate=True, col_dtype=torch.int32)
+    assert plan.info()["long_rows"] > 0
+    _assert_close(got, want, f64, what="rmat weighted")
+    deg = np.maximum(np.diff(rowptr), 1).astype(np.float32)
+    ones = np.ones_like(w)
+    want_m = z.copy(); orc.spmm_accumulate(rowptr, col, ones, x, want_m); orc.row_divide(want_m, deg)
+    got_m, _ = _run_gpu(rowptr, col, None, x, z, accumulate=True, row_div=deg, col_dtype=torch.int32)
+    _assert_close(got_m, want_m, orc.spmm_f64(rowptr, col, ones, x) / deg[:, None], what="rmat mean")
