@@ -1,0 +1,294 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one pass of the hot path over one batch of synthetic input that is already resident in
+HBM: by default the headline configuration, a weighted-sum SpMM (out += A @ X, GCN-normalised edge
+weights) over an R-MAT power-law graph with 2.45 M nodes / ~62 M stored edges at F = 128 fp32.
+The same run also reports, as extras, the mean-aggregation variant, the int8/int4/int2
+quantize+pack and unpack+dequantize kernels on 1 M x 256 boundary rows, a plain streaming copy (the
+attainable-bandwidth yardstick), and a CPU baseline timed on this machine's host cores.
+
+Prints ONE JSON line on stdout (everything else goes to stderr).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this file (see profiles/), scaled by what the same counters read for sgnn_stream_copy_f32 of a
+# known size.  Keyed by workload name; None = not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def spmm_gather_bytes(nnz, rows, F, weighted, accumulate, mean):
+    """Algorithmic bytes of one SpMM under the gather model (no cache credit), int32 columns:
+    per edge 4F (dense row) + 4 (col) + 4 (val, if weighted); per row 4F (write) + 8 (rowptr)
+    + 4F when accumulating onto a previous out + 4 for the mean divisor."""
+    per_edge = 4 * F + 4 + (4 if weighted else 0)
+    per_row = 4 * F + 8 + (4 * F if accumulate else 0) + (4 if mean else 0)
+    return nnz * per_edge + rows * per_row
+
+
+def quant_bytes(rows, F, bits):
+    """Fused quantize+pack (and, read the other way, unpack+dequantize): per row 4F + F*bits/8 + 8."""
+    return rows * (4 * F + F * bits // 8 + 8)
+
+
+def time_steps(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def build_headline_graph(nodes, und_edges, F, device):
+    import torch
+    from super_gnn_amd import synth
+    t0 = time.perf_counter()
+    rowptr, col = synth.rmat_graph(nodes, und_edges, a=0.57, b=0.19, c=0.19, seed=1, device=device)
+    w = synth.gcn_norm_weights(rowptr, col)
+    g = torch.Generator(device=device)
+    g.manual_seed(2)
+    x = torch.randn(nodes, F, generator=g, device=device, dtype=torch.float32)
+    torch.cuda.synchronize()
+    log(f"[bench] graph: {nodes} nodes, {col.numel()} stored edges, max degree "
+        f"{int((rowptr[1:] - rowptr[:-1]).max())}, built in {time.perf_counter() - t0:.1f}s")
+    return rowptr, col, w, x
+
+
+def cpu_baseline_spmm(rowptr, col, w, x, target_edges=16_000_000, reps=3):
+    """Time the CPU path on a bounded sample: the leading rows holding ~target_edges edges, gathered
+    from the full X (so the gather footprint is the real one).  Uses the reference's own x86
+    extension when oracle/_ref is loadable on this host, else the C restatement."""
+    import numpy as np
+    import torch
+    from oracle import oracle as orc
+    rp = rowptr.cpu()
+    m = int(torch.searchsorted(rp, torch.tensor(target_edges)).item())
+    m = max(1, min(m, rp.numel() - 1))
+    nnz = int(rp[m])
+    rp_s = rp[: m + 1].contiguous()
+    col_s = col[:nnz].to(torch.int64).cpu().contiguous()
+    w_s = w[:nnz].cpu().contiguous()
+    xh = x.cpu()
+    F = xh.shape[1]
+    out = torch.zeros(m, F)
+    ref = orc.ref_ops()
+    if ref is not None:
+        kind, T = "reference", torch.get_num_threads()
+        tgt = torch.linspace(0, nnz, T + 1).to(torch.int64)
+        rs = torch.searchsorted(rp_s, tgt).to(torch.int32)  # nnz-balanced contiguous row split
+        rs[0], rs[-1] = 0, m
+        cs = torch.tensor([0, F], dtype=torch.int32)
+        run = lambda: ref.spmm(rp_s, col_s, w_s, xh, out, m, rs, cs)  # noqa: E731
+    else:
+        kind, T = "port", orc.num_threads()
+        a = (rp_s.numpy(), col_s.numpy(), w_s.numpy(), xh.numpy(), out.numpy())
+        run = lambda: orc.spmm_accumulate(*a)  # noqa: E731
+    run()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        run()
+        ts.append(time.perf_counter() - t0)
+    t = float(np.median(ts))
+    return {"value": nnz / t / 1e9, "unit": "GEdges/s", "cores": int(T), "kind": kind,
+            "sample": f"first {m} rows ({nnz} edges) of the same graph, full X, F={F}, median of {reps}",
+            "ms": t * 1e3}
+
+
+def cpu_baseline_quant(x, bits, rows=200_000, reps=3):
+    import numpy as np
+    from oracle import oracle as orc
+    xs = x[:rows].cpu().numpy()
+    orc.quant_rows(xs, [0, rows], bits)
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        orc.quant_rows(xs, [0, rows], bits)
+        ts.append(time.perf_counter() - t0)
+    t = float(np.median(ts))
+    return {"value": quant_bytes(rows, xs.shape[1], bits) / t / 1e9, "unit": "GB/s", "cores": orc.num_threads(),
+            "kind": "port", "sample": f"first {rows} rows, int{bits}, median of {reps}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy"],
+                    help="rmat: headline SpMM (default); quant: int2 quantize+pack as the step; copy: streaming copy")
+    ap.add_argument("--nodes", type=int, default=2_450_000)
+    ap.add_argument("--und-edges", type=int, default=31_000_000)
+    ap.add_argument("--feat", type=int, default=128)
+    ap.add_argument("--quant-rows", type=int, default=1_000_000)
+    ap.add_argument("--quant-feat", type=int, default=256)
+    ap.add_argument("--bits", type=int, default=2)
+    ap.add_argument("--no-extras", action="store_true", help="skip the extra kernels (used under rocprofv3)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this build runs one partition on ONE GPU; there is no multi-GPU path to time "
+            f"(--gpus {args.gpus} refused).")
+        sys.exit(2)
+
+    import torch
+    import super_gnn_amd  # noqa: F401  (raises if libsgnn_hip.so is missing)
+    from super_gnn_amd import _lib, synth, supergnn_ops as ops
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    stream = ops._stream
+
+    extra = {}
+    # ---- streaming copy yardstick --------------------------------------------------------------
+    n_copy = 256 * 1024 * 1024  # 1 GiB in + 1 GiB out
+    src = torch.empty(n_copy, device=dev).normal_()
+    dst = torch.empty_like(src)
+    copy_fn = lambda: _lib.check(_lib.lib.sgnn_stream_copy_f32(src.data_ptr(), dst.data_ptr(), n_copy, stream()))  # noqa: E731
+    if args.workload == "copy" or not args.no_extras:
+        ms = time_steps(copy_fn, 10, 3)
+        extra["stream_copy_GBps"] = round(2 * 4 * n_copy / ms / 1e6, 1)
+        log(f"[bench] stream copy: {extra['stream_copy_GBps']} GB/s (read+write)")
+
+    result = None
+    if args.workload == "copy":
+        _lib.profile_start()
+        ms = time_steps(copy_fn, args.steps, args.warmup)
+        prof = _lib.profile_stop()
+        n, tot = prof["stream_copy_kernel"]
+        ach = 2 * 4 * n_copy / (tot / n) / 1e6
+        result = {"metric": "stream copy GB/s", "value": round(2 * 4 * n_copy / ms / 1e6, 2), "unit": "GB/s",
+                  "config": {"workload": "stream_copy_1GiB"}, "ms_per_step": ms, "dtype": "f32",
+                  "roofline": {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                               "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "stream_copy_kernel"},
+                  "cpu_baseline": None}
+    del src, dst
+
+    # ---- quantize / dequantize sweep -----------------------------------------------------------
+    if args.workload == "quant" or not args.no_extras:
+        n, F = args.quant_rows, args.quant_feat
+        xq = synth.boundary_features(n, F, seed=5, device=dev)
+        seg = torch.tensor([0, n], dtype=torch.int32)
+        d = torch.empty(n, F, device=dev)
+        for bits in (8, 4, 2):
+            if args.workload == "quant" and args.no_extras and bits != args.bits:
+                continue
+            epb = 8 // bits
+            q = torch.empty((n + epb - 1) // epb, F, dtype=torch.uint8, device=dev)
+            p = torch.empty(n, 2, device=dev)
+            qf = lambda: ops.quantize_tensor_for_all_procs(xq, q, p, seg, 1, bits)  # noqa: E731
+            df = lambda: ops.dequantize_tensor_for_all_procs(q, d, p, seg, 1, bits)  # noqa: E731
+            is_main = args.workload == "quant" and bits == args.bits
+            st, wu = (args.steps, args.warmup) if is_main else (10, 3)
+            _lib.profile_start()
+            ms_q = time_steps(qf, st, wu)
+            prof = _lib.profile_stop()
+            ms_d = time_steps(df, 10, 3)
+            b = quant_bytes(n, F, bits)
+            extra[f"quant_pack_int{bits}_GBps"] = round(b / ms_q / 1e6, 1)
+            extra[f"unpack_dequant_int{bits}_GBps"] = round(b / ms_d / 1e6, 1)
+            log(f"[bench] int{bits}: quantize+pack {b / ms_q / 1e6:.0f} GB/s ({ms_q:.3f} ms), "
+                f"unpack+dequant {b / ms_d / 1e6:.0f} GB/s ({ms_d:.3f} ms)")
+            if is_main:
+                nl, tot = prof["quant_pack_rows_kernel"]
+                ach = b / (tot / nl) / 1e6
+                wl = f"quant_pack_int{bits}_{n}x{F}"
+                result = {"metric": f"quantize-pack GB/s at int{bits}", "value": round(b / ms_q / 1e6, 2),
+                          "unit": "GB/s", "config": {"workload": wl, "rows": n, "F": F, "bits": bits},
+                          "ms_per_step": ms_q, "dtype": "f32->u8",
+                          "roofline": {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS,
+                                       "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4),
+                                       "traffic": MEASURED_TRAFFIC_BYTES.get(wl), "kernel": "quant_pack_rows_kernel",
+                                       "kernel_avg_ms": round(tot / nl, 5), "algorithmic_bytes": b},
+                          "cpu_baseline": None if args.no_cpu else cpu_baseline_quant(xq, bits)}
+        if not args.no_cpu and args.workload != "quant":
+            extra["cpu_quant_pack_int2"] = cpu_baseline_quant(xq, 2)
+        del xq, d
+
+    # ---- headline SpMM -------------------------------------------------------------------------
+    if args.workload == "rmat":
+        F = args.feat
+        rowptr, col, w, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
+        M, nnz = rowptr.numel() - 1, col.numel()
+        t0 = time.perf_counter()
+        plan = ops.SpmmPlan(rowptr, col, M)
+        torch.cuda.synchronize()
+        info = plan.info()
+        extra["plan_build_ms"] = round((time.perf_counter() - t0) * 1e3, 1)
+        extra["plan"] = {k: info[k] for k in ("long_rows", "segments", "long_edges", "long_row_threshold", "segment_edges")}
+        log(f"[bench] plan: {extra['plan']} built in {extra['plan_build_ms']} ms")
+        out = torch.zeros(M, F, device=dev)
+        step = lambda: plan.run(w, x, out, accumulate=True)  # noqa: E731
+        _lib.profile_start()
+        ms = time_steps(step, args.steps, args.warmup)
+        prof = _lib.profile_stop()
+        per_kernel = {k: round(v[1] / v[0], 5) for k, v in prof.items()}
+        log(f"[bench] weighted sum: {ms:.3f} ms/step, {nnz / ms / 1e6:.2f} GEdges/s, kernels (avg ms) {per_kernel}")
+        # dominant kernel: the short-row kernel; its share of the algorithmic bytes
+        short_edges = nnz - info["long_edges"]
+        short_rows = M - info["long_rows"]
+        b_short = spmm_gather_bytes(short_edges, short_rows, F, weighted=True, accumulate=True, mean=False)
+        b_total = spmm_gather_bytes(nnz, M, F, weighted=True, accumulate=True, mean=False)
+        dom = max(prof, key=lambda k: prof[k][1])
+        dom_ms = prof[dom][1] / prof[dom][0]
+        if dom == "spmm_short_kernel":
+            dom_bytes = b_short
+        elif dom == "spmm_segment_kernel":
+            dom_bytes = info["long_edges"] * (4 * F + 8) + info["segments"] * 4 * F
+        else:
+            dom_bytes = b_total
+        ach = dom_bytes / dom_ms / 1e6
+        wl = f"rmat_{M}n_{nnz}e_F{F}_gcn_weighted_sum"
+        # mean aggregation (unit weights + fused /deg) as an extra
+        if not args.no_extras:
+            deg = (rowptr[1:] - rowptr[:-1]).clamp(min=1).to(torch.float32)
+            out2 = torch.zeros(M, F, device=dev)
+            ms_mean = time_steps(lambda: plan.run(None, x, out2, accumulate=True, row_div=deg), 10, 3)
+            extra["spmm_mean_GEdges_per_s"] = round(nnz / ms_mean / 1e6, 3)
+            extra["spmm_mean_gather_GBps"] = round(spmm_gather_bytes(nnz, M, F, False, True, True) / ms_mean / 1e6, 1)
+            del out2
+        extra["spmm_total_gather_GBps"] = round(b_total / ms / 1e6, 1)
+        extra["spmm_total_frac_of_hbm_peak"] = round(b_total / ms / 1e6 / HBM_PEAK_GBPS, 4)
+        extra["spmm_GFLOPs"] = round(2.0 * nnz * F / ms / 1e6, 1)
+        extra["kernel_avg_ms"] = per_kernel
+        result = {"metric": "SpMM GEdges/s + % HBM roofline (F=128 fp32); quantize-pack GB/s at int2",
+                  "value": round(nnz / ms / 1e6, 4), "unit": "GEdges/s",
+                  "config": {"workload": wl, "nodes": M, "edges": nnz, "F": F, "aggregation": "weighted_sum",
+                             "accumulate": True, "index_dtype": "int32"},
+                  "ms_per_step": ms, "dtype": "f32",
+                  "roofline": {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                               "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl),
+                               "kernel": dom, "kernel_avg_ms": round(dom_ms, 5), "algorithmic_bytes": int(dom_bytes)},
+                  "cpu_baseline": None if args.no_cpu else cpu_baseline_spmm(rowptr, col, w, x)}
+
+    line = {"metric": result["metric"], "value": result["value"], "unit": result["unit"], "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(result["ms_per_step"], 5),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": result["dtype"],
+            "data": "synthetic", "config": result["config"], "roofline": result["roofline"],
+            "cpu_baseline": result["cpu_baseline"], "extra": extra}
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

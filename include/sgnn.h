@@ -128,6 +128,26 @@ int sgnn_quant_v1_f32(const float *x, uint8_t *q, const int64_t *range, float *p
 int sgnn_dequant_v1_f32(const uint8_t *q, float *x, const int64_t *range, const float *params,
                         int64_t n, int64_t F, sgnn_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Measurement helpers (no reference counterpart; the reference times with std::chrono under
+ * #define PROFILE, super_gnn/ops/csrc/spmm.cpp:12,352-354,518-523)
+ * ------------------------------------------------------------------------------------------- */
+
+/* on != 0: drop earlier records and start recording one HIP event pair around every kernel
+ * launch, on the stream the kernel is launched on.  on == 0: stop recording (records kept). */
+int sgnn_profile_enable(int on);
+
+/* Waits for the recorded launches of kernel_id and returns their count and summed duration. */
+int sgnn_profile_read(int kernel_id, int64_t *launches, double *total_ms);
+
+/* Kernel ids are 0 .. sgnn_profile_kernel_count()-1; the name is the __global__ function's. */
+const char *sgnn_profile_kernel_name(int kernel_id);
+int sgnn_profile_kernel_count(void);
+
+/* dst[0..n) = src[0..n) with 128-bit non-temporal accesses: the attainable-bandwidth yardstick
+ * and the calibration kernel for hardware traffic counters.  n % 4 == 0, 16-byte aligned. */
+int sgnn_stream_copy_f32(const float *src, float *dst, int64_t n, sgnn_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

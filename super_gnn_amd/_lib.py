@@ -27,6 +27,11 @@ SIGNATURES = {
     "sgnn_unpack_dequant_rows_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
     "sgnn_quant_v1_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "sgnn_dequant_v1_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    "sgnn_profile_enable": (_int, [_int]),
+    "sgnn_profile_read": (_int, [_int, ctypes.POINTER(_i64), ctypes.POINTER(ctypes.c_double)]),
+    "sgnn_profile_kernel_name": (ctypes.c_char_p, [_int]),
+    "sgnn_profile_kernel_count": (_int, []),
+    "sgnn_stream_copy_f32": (_int, [_vp, _vp, _i64, _vp]),
 }
 
 
@@ -60,3 +65,20 @@ def check(status):
             raise IndexError(f"libsgnn_hip: {msg}")
         raise SgnnError(f"libsgnn_hip (status {status}): {msg}")
     return status
+
+
+def profile_start():
+    """Start recording a HIP event pair around every kernel launch of the library."""
+    check(lib.sgnn_profile_enable(1))
+
+
+def profile_stop():
+    """Stop recording and return {kernel name: (launches, total_ms)} for kernels that ran."""
+    check(lib.sgnn_profile_enable(0))
+    out = {}
+    for k in range(lib.sgnn_profile_kernel_count()):
+        n, ms = _i64(0), ctypes.c_double(0.0)
+        check(lib.sgnn_profile_read(k, ctypes.byref(n), ctypes.byref(ms)))
+        if n.value:
+            out[lib.sgnn_profile_kernel_name(k).decode()] = (n.value, ms.value)
+    return out

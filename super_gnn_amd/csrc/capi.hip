@@ -1,4 +1,8 @@
 // Error reporting and version of the C ABI.
+#include <algorithm>
+#include <mutex>
+#include <vector>
+
 #include "common.hpp"
 
 namespace sgnn {
@@ -18,7 +22,94 @@ int fail(int code, const char *fmt, ...) {
     return code;
 }
 
+// ---- HIP-event profiler ------------------------------------------------------------------------
+struct ProfRecord {
+    int id;
+    hipEvent_t start, stop;
+};
+static std::mutex g_prof_mu;
+static bool g_prof_on = false;
+static std::vector<ProfRecord> g_prof;
+
+ProfScope::ProfScope(int id, hipStream_t st) : id_(id), st_(st) {
+    if (!g_prof_on) return;
+    if (hipEventCreate(&start_) != hipSuccess) { start_ = nullptr; return; }
+    (void)hipEventRecord(start_, st_);
+}
+
+ProfScope::~ProfScope() {
+    if (!start_) return;
+    hipEvent_t stop = nullptr;
+    if (hipEventCreate(&stop) != hipSuccess) { (void)hipEventDestroy(start_); return; }
+    (void)hipEventRecord(stop, st_);
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof.push_back({id_, start_, stop});
+}
+
+static const char *kKernelNames[K_COUNT] = {
+    "spmm_short_kernel",  "spmm_segment_kernel", "spmm_long_final_kernel", "quant_pack_rows_kernel",
+    "unpack_dequant_rows_kernel", "quant_v1_kernel", "dequant_v1_kernel", "stream_copy_kernel",
+    "fused_dq_spmm_short_kernel", "fused_dq_spmm_segment_kernel"};
+
+// ---- plain streaming copy: the attainable-bandwidth yardstick and the counter calibration -----
+__global__ __launch_bounds__(256) void stream_copy_kernel(const float4 *__restrict__ src, float4 *__restrict__ dst,
+                                                          int64_t n4) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (; i < n4; i += stride) {
+        const f4 v = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(src) + i);
+        __builtin_nontemporal_store(v, reinterpret_cast<f4 *>(dst) + i);
+    }
+}
+
 }  // namespace sgnn
+
+using namespace sgnn;
+
+extern "C" int sgnn_profile_enable(int on) {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    if (on) {
+        for (auto &r : g_prof) { (void)hipEventDestroy(r.start); (void)hipEventDestroy(r.stop); }
+        g_prof.clear();
+    }
+    g_prof_on = on != 0;
+    return SGNN_OK;
+}
+
+extern "C" int sgnn_profile_read(int kernel_id, int64_t *launches, double *total_ms) {
+    SGNN_REQUIRE(kernel_id >= 0 && kernel_id < K_COUNT && launches && total_ms, "bad profile query");
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    *launches = 0;
+    *total_ms = 0.0;
+    for (auto &r : g_prof) {
+        if (r.id != kernel_id) continue;
+        SGNN_HIP_CHECK(hipEventSynchronize(r.stop));
+        float ms = 0.0f;
+        SGNN_HIP_CHECK(hipEventElapsedTime(&ms, r.start, r.stop));
+        *launches += 1;
+        *total_ms += ms;
+    }
+    return SGNN_OK;
+}
+
+extern "C" const char *sgnn_profile_kernel_name(int kernel_id) {
+    return (kernel_id >= 0 && kernel_id < K_COUNT) ? kKernelNames[kernel_id] : "";
+}
+
+extern "C" int sgnn_profile_kernel_count(void) { return K_COUNT; }
+
+extern "C" int sgnn_stream_copy_f32(const float *src, float *dst, int64_t n, sgnn_stream_t stream) {
+    SGNN_REQUIRE(n >= 0 && n % 4 == 0, "n must be a non-negative multiple of 4");
+    if (n == 0) return SGNN_OK;
+    SGNN_REQUIRE(src && dst && aligned(src, 16) && aligned(dst, 16), "src/dst must be non-null and 16-byte aligned");
+    const int64_t n4 = n / 4;
+    const int nb = (int)std::min<int64_t>((n4 + 255) / 256, 256 * 64);
+    ProfScope prof(K_STREAM_COPY, (hipStream_t)stream);
+    hipLaunchKernelGGL(stream_copy_kernel, dim3(nb), dim3(256), 0, (hipStream_t)stream, (const float4 *)src, (float4 *)dst, n4);
+    SGNN_HIP_CHECK(hipGetLastError());
+    return SGNN_OK;
+}
 
 extern "C" const char *sgnn_last_error(void) { return sgnn::last_error().c_str(); }
 

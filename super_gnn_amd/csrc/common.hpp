@@ -30,6 +30,31 @@ int fail(int code, const char *fmt, ...);
         if (!(cond)) return ::sgnn::fail(SGNN_ERR_ARG, __VA_ARGS__);                          \
     } while (0)
 
+// Kernels the built-in HIP-event profiler can attribute time to (see sgnn_profile_* in sgnn.h).
+enum KernelId {
+    K_SPMM_SHORT = 0,
+    K_SPMM_SEGMENT,
+    K_SPMM_LONG_FINAL,
+    K_QUANT_PACK_ROWS,
+    K_UNPACK_DEQUANT_ROWS,
+    K_QUANT_V1,
+    K_DEQUANT_V1,
+    K_STREAM_COPY,
+    K_FUSED_SHORT,
+    K_FUSED_SEGMENT,
+    K_COUNT
+};
+
+// Records a HIP event pair around the launches made while it is alive, on the launch stream,
+// when profiling is enabled; free otherwise.
+struct ProfScope {
+    ProfScope(int id, hipStream_t st);
+    ~ProfScope();
+    int id_;
+    hipStream_t st_;
+    hipEvent_t start_ = nullptr;
+};
+
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 // Workgroups are dealt round-robin to the XCDs (workgroup i runs on XCD i % 8).  This maps the

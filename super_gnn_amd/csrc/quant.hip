@@ -431,6 +431,7 @@ static void launch_rows(const RowsArgs &a, hipStream_t st) {
     constexpr int GPB = kQBlock / G;
     const int n_units = (a.n_packed + NPR - 1) / NPR;
     const int nb = (n_units + GPB - 1) / GPB;
+    ProfScope prof(a.quantize ? K_QUANT_PACK_ROWS : K_UNPACK_DEQUANT_ROWS, st);
     if (a.quantize)
         hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
                            a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
@@ -442,6 +443,7 @@ static void launch_rows(const RowsArgs &a, hipStream_t st) {
 template <int BITS>
 static void launch_rows_wide(const RowsArgs &a, hipStream_t st) {
     const int nb = (a.n_packed + kQBlock / 64 - 1) / (kQBlock / 64);
+    ProfScope prof(a.quantize ? K_QUANT_PACK_ROWS : K_UNPACK_DEQUANT_ROWS, st);
     if (a.quantize)
         hipLaunchKernelGGL((quant_pack_rows_wide_kernel<BITS>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
                            a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F);

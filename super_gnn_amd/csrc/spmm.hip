@@ -286,13 +286,18 @@ static void launch_all(const ShortArgs &a, const SegArgs &s, const FinalArgs &f,
     constexpr int GPB = kBlock / G;
     if (a.M > 0) {
         const uint32_t nb = (uint32_t)((a.M + GPB - 1) / GPB);
+        ProfScope prof(K_SPMM_SHORT, st);
         hipLaunchKernelGGL((spmm_short_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, a.rowptr, a.col, a.val, a.x,
                            a.out, a.M, a.F, a.ldx, a.ldo, a.accumulate, a.row_div, a.long_thresh, nb);
     }
     if (s.n_seg > 0) {
-        hipLaunchKernelGGL((spmm_segment_kernel<VEC, G, NV>), dim3(s.n_seg), dim3(kBlock), 0, st, s.col, s.val, s.x,
-                           s.partial, s.seg_begin, s.seg_len, s.F, s.ldx);
+        {
+            ProfScope prof(K_SPMM_SEGMENT, st);
+            hipLaunchKernelGGL((spmm_segment_kernel<VEC, G, NV>), dim3(s.n_seg), dim3(kBlock), 0, st, s.col, s.val,
+                               s.x, s.partial, s.seg_begin, s.seg_len, s.F, s.ldx);
+        }
         const uint32_t nb = (uint32_t)((f.n_long + GPB - 1) / GPB);
+        ProfScope prof(K_SPMM_LONG_FINAL, st);
         hipLaunchKernelGGL((spmm_long_final_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, f.long_rows,
                            f.long_segptr, f.partial, f.out, f.n_long, f.F, f.ldo, f.accumulate, f.row_div);
     }

@@ -151,21 +151,17 @@ class SpmmPlan:
                 pass
 
 
-_PLAN_CACHE = OrderedDict()
-_PLAN_CACHE_MAX = 16
-
-
 def _cached_plan(rowptr, col, K):
-    key = (rowptr.data_ptr(), rowptr._version, rowptr.numel(), col.data_ptr(), col._version, col.numel(), int(K),
-           str(rowptr.device))
-    plan = _PLAN_CACHE.get(key)
-    if plan is None:
-        plan = SpmmPlan(rowptr, col, K)
-        _PLAN_CACHE[key] = plan
-        while len(_PLAN_CACHE) > _PLAN_CACHE_MAX:
-            _PLAN_CACHE.popitem(last=False)
-    else:
-        _PLAN_CACHE.move_to_end(key)
+    """Plan cached ON the rowptr tensor object (the reference caches its row split on the matrix
+    object the same way).  The entry pins the col tensor it was built from and both version
+    counters, so a recycled allocation or an in-place edit can never alias a stale plan."""
+    entries = rowptr.__dict__.setdefault("_sgnn_plans", [])
+    for e in entries:
+        if e[0] is col and e[1] == (rowptr._version, col._version, int(K)):
+            return e[2]
+    plan = SpmmPlan(rowptr, col, K)
+    entries[:] = [e for e in entries if e[0] is not col][-3:]
+    entries.append((col, (rowptr._version, col._version, int(K)), plan))
     return plan
 
 
@@ -217,22 +213,18 @@ class _Segments:
         self.pseg_host = pseg_host
 
 
-_SEG_CACHE = OrderedDict()
-
-
 def quant_segments(work_range, bits):
-    """Device copies of the segment table and its packed-row offsets, cached per table."""
+    """Device copies of the segment table and its packed-row offsets, cached on the tensor object
+    (keyed by its version counter, so in-place edits rebuild them)."""
+    _want(work_range, torch.int32, "work_range_per_proc")
     dev = _device()
-    key = (work_range.data_ptr(), work_range._version, work_range.numel(), int(bits), str(work_range.device), str(dev))
-    s = _SEG_CACHE.get(key)
+    cache = work_range.__dict__.setdefault("_sgnn_segments", {})
+    key = (int(bits), work_range._version, str(dev))
+    s = cache.get(key)
     if s is None:
-        _want(work_range, torch.int32, "work_range_per_proc")
+        cache.clear()
         s = _Segments(work_range.detach().cpu(), int(bits), dev)
-        _SEG_CACHE[key] = s
-        while len(_SEG_CACHE) > 64:
-            _SEG_CACHE.popitem(last=False)
-    else:
-        _SEG_CACHE.move_to_end(key)
+        cache[key] = s
     return s
 
 
@@ -286,12 +278,17 @@ def _dequant_rows(inp_u8, out, params, segs, bits):
     s_out.commit()
 
 
+_SINGLE_SEG = OrderedDict()
+
+
 def _single_segment(n, bits):
-    key = ("single", int(n), int(bits), str(_device()))
-    s = _SEG_CACHE.get(key)
+    key = (int(n), int(bits), str(_device()))
+    s = _SINGLE_SEG.get(key)
     if s is None:
         s = _Segments(torch.tensor([0, int(n)], dtype=torch.int32), int(bits), _device())
-        _SEG_CACHE[key] = s
+        _SINGLE_SEG[key] = s
+        while len(_SINGLE_SEG) > 64:
+            _SINGLE_SEG.popitem(last=False)
     return s
 
 

@@ -34,13 +34,28 @@ def _run_gpu(rowptr, col, val, x, init, accumulate, row_div=None, col_dtype=torc
     return out.cpu().numpy(), plan
 
 
-def _assert_close(got, want, f64=None, what=""):
+def _abs_sum64(rowptr, col, val, x, init=None):
+    """sum_e |val_e * x[col_e, f]| (+ |init|) in fp64: the scale of the rounding-error bound."""
+    v = np.abs(val) if val is not None else None
+    return orc.spmm_f64(rowptr, col, v, np.abs(x), np.abs(init) if init is not None else None)
+
+
+def _assert_close(got, want, f64=None, abs_sum=None, deg=None, what=""):
+    """Elementwise |gpu - ref32| <= 1e-6 + 1e-5*|ref32|.  Elements of LONG rows that miss it are
+    adjudicated against the fp64 sum: two fp32 summation orders of n terms may legitimately differ
+    by up to the forward error bound (n+1)*2^-24 * sum|terms| each (Higham, Accuracy and Stability
+    of Numerical Algorithms, eq. 4.4), which for cancelling sums exceeds 1e-5 relative.  Such an
+    element passes iff the GPU value meets that bound, and overall the GPU must not be less accurate
+    than the sequential fp32 reference."""
     err = np.abs(got - want)
     tol = ATOL + RTOL * np.abs(want)
     bad = err > tol
     if bad.any() and f64 is not None:
-        # adjudicate against fp64: the sequential fp32 reference itself carries rounding error
-        bad = bad & (np.abs(got - f64) > np.abs(want - f64) + tol)
+        bound = (deg[:, None].astype(np.float64) + 1.0) * 2.0 ** -24 * abs_sum
+        bad = bad & (np.abs(got - f64) > bound + ATOL)
+        rms_gpu = np.sqrt(np.mean((got - f64) ** 2))
+        rms_ref = np.sqrt(np.mean((want - f64) ** 2))
+        assert rms_gpu <= 1.5 * rms_ref + 1e-7, f"{what}: gpu rms error {rms_gpu} vs reference fp32 {rms_ref}"
     assert not bad.any(), f"{what}: {bad.sum()} elements out of tolerance, max err {err.max()}"
 
 
@@ -92,10 +107,11 @@ def test_long_rows_segment_path(F, thresh, seg):
     init = rng.standard_normal((M, F), dtype=np.float32)
     want = init.copy(); orc.spmm_accumulate(rowptr, col, val, x, want)
     f64 = orc.spmm_f64(rowptr, col, val, x, init)
+    S, deg = _abs_sum64(rowptr, col, val, x, init), np.diff(rowptr)
     got, plan = _run_gpu(rowptr, col, val, x, init, accumulate=True, thresh=thresh, seg=seg)
     info = plan.info()
     assert info["long_rows"] >= 9 and info["segments"] >= info["long_rows"]
-    _assert_close(got, want, f64, what=f"long rows F={F}")
+    _assert_close(got, want, f64, S, deg, what=f"long rows F={F}")
     short = np.diff(rowptr) <= thresh
     assert np.array_equal(got[short], want[short])
     # run-to-run reproducible (no atomics)
@@ -104,7 +120,7 @@ def test_long_rows_segment_path(F, thresh, seg):
     # overwrite mode on the same matrix
     w2 = init.copy(); orc.spmm_overwrite(rowptr, col, val, x, w2)
     g2, _ = _run_gpu(rowptr, col, val, x, init, accumulate=False, thresh=thresh, seg=seg)
-    _assert_close(g2, w2, orc.spmm_f64(rowptr, col, val, x), what="long rows overwrite")
+    _assert_close(g2, w2, orc.spmm_f64(rowptr, col, val, x), _abs_sum64(rowptr, col, val, x), deg, what="long rows overwrite")
 
 
 def test_mean_epilogue_and_unit_weights():
@@ -115,15 +131,18 @@ def test_mean_epilogue_and_unit_weights():
     deg = np.maximum(np.diff(rowptr), 1).astype(np.float32)
     ones = np.ones(col.shape[0], dtype=np.float32)
     want = np.zeros((M, F), np.float32); orc.spmm_accumulate(rowptr, col, ones, x, want); orc.row_divide(want, deg)
+    f64 = orc.spmm_f64(rowptr, col, ones, x) / deg[:, None]
+    S, dg = _abs_sum64(rowptr, col, ones, x) / deg[:, None], np.diff(rowptr)
     got, _ = _run_gpu(rowptr, col, None, x, np.zeros((M, F), np.float32), accumulate=True, row_div=deg)
-    _assert_close(got, want, what="mean, val=None")
+    _assert_close(got, want, f64, S, dg, what="mean, val=None")
     got2, _ = _run_gpu(rowptr, col, ones, x, np.zeros((M, F), np.float32), accumulate=False, row_div=deg, col_dtype=torch.int32)
-    _assert_close(got2, want, what="mean, overwrite, int32 col")
+    _assert_close(got2, want, f64, S, dg, what="mean, overwrite, int32 col")
     # with a non-zero previous value the division covers the whole sum, on every row
     init = rng.standard_normal((M, F), dtype=np.float32)
     w3 = init.copy(); orc.spmm_accumulate(rowptr, col, ones, x, w3); orc.row_divide(w3, deg)
     g3, _ = _run_gpu(rowptr, col, ones, x, init, accumulate=True, row_div=deg)
-    _assert_close(g3, w3, what="mean on accumulate")
+    _assert_close(g3, w3, orc.spmm_f64(rowptr, col, ones, x, init) / deg[:, None],
+                  _abs_sum64(rowptr, col, ones, x, init) / deg[:, None], dg, what="mean on accumulate")
 
 
 def test_duplicates_linearity_and_transpose():
@@ -222,11 +241,15 @@ def test_power_law_graph_weighted_and_mean():
     z = np.zeros((n, 128), np.float32)
     want = z.copy(); orc.spmm_accumulate(rowptr, col, w, x, want)
     f64 = orc.spmm_f64(rowptr, col, w, x)
+    dg = np.diff(rowptr)
     got, plan = _run_gpu(rowptr, col, w, x, z, accumulate=True, col_dtype=torch.int32)
     assert plan.info()["long_rows"] > 0
-    _assert_close(got, want, f64, what="rmat weighted")
+    _assert_close(got, want, f64, _abs_sum64(rowptr, col, w, x), dg, what="rmat weighted")
+    short = dg <= plan.info()["long_row_threshold"]
+    assert np.array_equal(got[short], want[short])
     deg = np.maximum(np.diff(rowptr), 1).astype(np.float32)
     ones = np.ones_like(w)
     want_m = z.copy(); orc.spmm_accumulate(rowptr, col, ones, x, want_m); orc.row_divide(want_m, deg)
     got_m, _ = _run_gpu(rowptr, col, None, x, z, accumulate=True, row_div=deg, col_dtype=torch.int32)
-    _assert_close(got_m, want_m, orc.spmm_f64(rowptr, col, ones, x) / deg[:, None], what="rmat mean")
+    _assert_close(got_m, want_m, orc.spmm_f64(rowptr, col, ones, x) / deg[:, None],
+                  _abs_sum64(rowptr, col, ones, x) / deg[:, None], dg, what="rmat mean")
