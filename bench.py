@@ -72,6 +72,13 @@ def build_headline_graph(nodes, und_edges, F, device):
     torch.cuda.synchronize()
     log(f"[bench] graph: {nodes} nodes, {col.numel()} stored edges, max degree "
         f"{int((rowptr[1:] - rowptr[:-1]).max())}, built in {time.perf_counter() - t0:.1f}s")
+    deg = rowptr[1:] - rowptr[:-1]
+    edges = [0, 1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1 << 30]
+    hist = []
+    for lo, hi in zip(edges[:-1], edges[1:]):
+        m = (deg >= lo) & (deg < hi)
+        hist.append(f"[{lo},{hi if hi < (1 << 30) else 'inf'}): {int(m.sum())} rows / {int(deg[m].sum())} edges")
+    log("[bench] degree histogram: " + "; ".join(hist))
     return rowptr, col, w, x
 
 
@@ -144,6 +151,8 @@ def main():
     ap.add_argument("--quant-rows", type=int, default=1_000_000)
     ap.add_argument("--quant-feat", type=int, default=256)
     ap.add_argument("--bits", type=int, default=2)
+    ap.add_argument("--long-threshold", type=int, default=0, help="SpMM plan: rows longer than this are split (0 = default)")
+    ap.add_argument("--segment-edges", type=int, default=0, help="SpMM plan: edges per long-row segment (0 = default)")
     ap.add_argument("--no-extras", action="store_true", help="skip the extra kernels (used under rocprofv3)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -232,7 +241,7 @@ def main():
         rowptr, col, w, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
         M, nnz = rowptr.numel() - 1, col.numel()
         t0 = time.perf_counter()
-        plan = ops.SpmmPlan(rowptr, col, M)
+        plan = ops.SpmmPlan(rowptr, col, M, long_row_threshold=args.long_threshold, segment_edges=args.segment_edges)
         torch.cuda.synchronize()
         info = plan.info()
         extra["plan_build_ms"] = round((time.perf_counter() - t0) * 1e3, 1)

@@ -42,6 +42,7 @@ enum KernelId {
     K_STREAM_COPY,
     K_FUSED_SHORT,
     K_FUSED_SEGMENT,
+    K_SPMM_EMPTY_ROWS,
     K_COUNT
 };
 
