@@ -143,6 +143,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--uniform-rows", type=int, default=0, help="diagnostic: replace the R-MAT graph by uniform random "
+                    "rows of --uniform-degree neighbours over --nodes columns")
+    ap.add_argument("--uniform-degree", type=int, default=25)
     ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy"],
                     help="rmat: headline SpMM (default); quant: int2 quantize+pack as the step; copy: streaming copy")
     ap.add_argument("--nodes", type=int, default=2_450_000)
@@ -152,7 +155,7 @@ def main():
     ap.add_argument("--quant-feat", type=int, default=256)
     ap.add_argument("--bits", type=int, default=2)
     ap.add_argument("--long-threshold", type=int, default=0, help="SpMM plan: rows longer than this are split (0 = default)")
-    ap.add_argument("--segment-edges", type=int, default=0, help="SpMM plan: edges per long-row segment (0 = default)")
+    ap.add_argument("--piece-edges", type=int, default=0, help="SpMM plan: minimum edges per long-row piece (0 = default)")
     ap.add_argument("--no-extras", action="store_true", help="skip the extra kernels (used under rocprofv3)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -238,14 +241,23 @@ def main():
     # ---- headline SpMM -------------------------------------------------------------------------
     if args.workload == "rmat":
         F = args.feat
-        rowptr, col, w, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
+        if args.uniform_rows:
+            g = torch.Generator(device=dev); g.manual_seed(11)
+            M, dg = args.uniform_rows, args.uniform_degree
+            col = torch.sort(torch.randint(0, args.nodes, (M, dg), generator=g, device=dev), dim=1).values
+            col = col.reshape(-1).to(torch.int32).contiguous()
+            rowptr = torch.arange(M + 1, device=dev, dtype=torch.int64) * dg
+            w = torch.rand(col.numel(), generator=g, device=dev)
+            x = torch.randn(args.nodes, F, generator=g, device=dev)
+        else:
+            rowptr, col, w, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
         M, nnz = rowptr.numel() - 1, col.numel()
         t0 = time.perf_counter()
-        plan = ops.SpmmPlan(rowptr, col, M, long_row_threshold=args.long_threshold, segment_edges=args.segment_edges)
+        plan = ops.SpmmPlan(rowptr, col, x.shape[0], long_row_threshold=args.long_threshold, piece_edges=args.piece_edges)
         torch.cuda.synchronize()
         info = plan.info()
         extra["plan_build_ms"] = round((time.perf_counter() - t0) * 1e3, 1)
-        extra["plan"] = {k: info[k] for k in ("long_rows", "segments", "long_edges", "long_row_threshold", "segment_edges")}
+        extra["plan"] = {k: info[k] for k in ("long_rows", "pieces", "long_edges", "long_row_threshold", "piece_edges")}
         log(f"[bench] plan: {extra['plan']} built in {extra['plan_build_ms']} ms")
         out = torch.zeros(M, F, device=dev)
         step = lambda: plan.run(w, x, out, accumulate=True)  # noqa: E731
@@ -263,12 +275,12 @@ def main():
         dom_ms = prof[dom][1] / prof[dom][0]
         if dom == "spmm_short_kernel":
             dom_bytes = b_short
-        elif dom == "spmm_segment_kernel":
-            dom_bytes = info["long_edges"] * (4 * F + 8) + info["segments"] * 4 * F
+        elif dom == "spmm_piece_kernel":
+            dom_bytes = info["long_edges"] * (4 * F + 8) + info["pieces"] * 4 * F
         else:
             dom_bytes = b_total
         ach = dom_bytes / dom_ms / 1e6
-        wl = f"rmat_{M}n_{nnz}e_F{F}_gcn_weighted_sum"
+        wl = f"rmat_{M}n_{nnz}e_F{F}_gcn_weighted_sum" if not args.uniform_rows else f"uniform_{M}x{args.nodes}_deg{args.uniform_degree}_F{F}"
         # mean aggregation (unit weights + fused /deg) as an extra
         if not args.no_extras:
             deg = (rowptr[1:] - rowptr[:-1]).clamp(min=1).to(torch.float32)

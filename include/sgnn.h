@@ -43,26 +43,33 @@ int sgnn_version(void);
  * SpMM
  * ------------------------------------------------------------------------------------------- */
 
-/* Per-matrix schedule: 32-bit column indices, the row classes (short rows: one lane group per
- * row; long rows: split into edge segments, one workgroup per segment) and the partial-sum
- * buffer of the long rows.  Plays the role of the row_splits the reference computes once per
- * matrix and caches on it (super_gnn/ops/spmm_kernel.py:49-58, distribute_work_for_row :8-29).
+/* Per-matrix schedule: 32-bit column indices, the row classes and their work lists.
+ *   short rows : chunks of consecutive rows (~128 edges), one lane group per chunk;
+ *   long rows  : edges regrouped by column class (a hash of col, 8 classes) and cut into pieces, one lane group per
+ *                piece, workgroup i serving class i % 8 so that each XCD's L2 caches its own class
+ *                of dense rows; partial sums land in a buffer owned by the plan;
+ *   empty rows : a list, used only by the modes that must write them.
+ * Plays the role of the row_splits the reference computes once per matrix and caches on it
+ * (super_gnn/ops/spmm_kernel.py:49-58, distribute_work_for_row :8-29).
  * The plan owns device copies of rowptr and of the (narrowed) column indices. */
 typedef struct sgnn_spmm_plan sgnn_spmm_plan;
 
 /* rowptr: int64[M+1] (device). col: int64[nnz] if col_is_i64 else int32[nnz] (device).
- * K = number of sparse columns = rows of the dense operand.  Every col must lie in [0, K) and
- * rowptr must be non-decreasing with rowptr[0] == 0: both are checked (SGNN_ERR_RANGE).
- * long_row_threshold / segment_edges: <= 0 selects the defaults.
- * Synchronises the stream (the row classes are built on the host). */
+ * K = number of sparse columns = rows of the dense operand.  M, K and nnz must be below 2^31 (the
+ * reference's kernel computes its offsets in 32-bit int as well, super_gnn/ops/csrc/spmm.cpp:30,94).
+ * Every col must lie in [0, K) and rowptr must be non-decreasing with rowptr[0] == 0: both are
+ * checked (SGNN_ERR_RANGE).
+ * long_row_threshold: rows with more edges take the long-row path (<= 0: default 128).
+ * piece_edges: minimum edges per long-row piece (<= 0: default 32).
+ * Synchronises the stream (the work lists are built on the host). */
 int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int col_is_i64, int64_t M,
-                          int64_t K, int64_t nnz, int long_row_threshold, int segment_edges,
+                          int64_t K, int64_t nnz, int long_row_threshold, int piece_edges,
                           sgnn_stream_t stream, sgnn_spmm_plan **plan_out);
 
 int sgnn_spmm_plan_destroy(sgnn_spmm_plan *plan);
 
-/* info[0]=M, [1]=K, [2]=nnz, [3]=#long rows, [4]=#segments, [5]=edges in long rows,
- * [6]=long_row_threshold, [7]=segment_edges. */
+/* info[0]=M, [1]=K, [2]=nnz, [3]=#long rows, [4]=#pieces, [5]=edges in long rows,
+ * [6]=long_row_threshold, [7]=piece_edges. */
 int sgnn_spmm_plan_info(const sgnn_spmm_plan *plan, int64_t info[8]);
 
 /* out[M,F] (+)= A[M,K] * x[K,F], fp32, row-major, leading dimensions ldx / ldo (in floats).
@@ -75,8 +82,8 @@ int sgnn_spmm_plan_info(const sgnn_spmm_plan *plan, int64_t info[8]);
  * val == NULL means all ones.  row_div != NULL fuses the mean epilogue
  * out[m,:] = (...) / row_div[m] for EVERY row m (super_gnn/layers/sageconv.py:78).
  * Short rows are summed in CSR edge order with one fused multiply-add per edge starting from
- * the old out value, as the reference does; long rows are summed per segment and the segment
- * partials are added in segment order (deterministic, no atomics). */
+ * the old out value, as the reference does (bit-identical results); long rows are summed per piece
+ * and the piece partials are added in piece order (deterministic, no atomics). */
 int sgnn_spmm_csr_f32(sgnn_spmm_plan *plan, const float *val, const float *x, float *out,
                       int64_t F, int64_t ldx, int64_t ldo, int accumulate, const float *row_div,
                       sgnn_stream_t stream);

@@ -47,7 +47,7 @@ ProfScope::~ProfScope() {
 }
 
 static const char *kKernelNames[K_COUNT] = {
-    "spmm_short_kernel",  "spmm_segment_kernel", "spmm_long_final_kernel", "quant_pack_rows_kernel",
+    "spmm_short_kernel",  "spmm_piece_kernel", "spmm_long_final_kernel", "quant_pack_rows_kernel",
     "unpack_dequant_rows_kernel", "quant_v1_kernel", "dequant_v1_kernel", "stream_copy_kernel",
     "fused_dq_spmm_short_kernel", "fused_dq_spmm_segment_kernel", "spmm_empty_rows_kernel"};
 

@@ -33,7 +33,7 @@ int fail(int code, const char *fmt, ...);
 // Kernels the built-in HIP-event profiler can attribute time to (see sgnn_profile_* in sgnn.h).
 enum KernelId {
     K_SPMM_SHORT = 0,
-    K_SPMM_SEGMENT,
+    K_SPMM_PIECE,
     K_SPMM_LONG_FINAL,
     K_QUANT_PACK_ROWS,
     K_UNPACK_DEQUANT_ROWS,

@@ -14,10 +14,11 @@
 //     the next one, whose old value was prefetched).  Edges are summed in CSR order with one fma
 //     per edge, starting from the old out value: the same operation sequence as the reference's
 //     kernel_1xN (spmm.cpp:87-162), so these rows are bit-identical to the reference.
-//   * long rows (power-law hubs): the edge list is cut into segments; one workgroup per segment,
-//     its lane groups take contiguous sub-ranges, partial sums are combined through LDS in a
-//     fixed order and written to a partial buffer; a last small kernel adds a row's partials in
-//     segment order.  No float atomics: results are reproducible run to run.
+//   * long rows (power-law hubs): at plan time the row's edges are regrouped by column class
+//     (a hash of the column index, 8 classes) and each class run is cut into pieces; one lane group sums one piece into a partial
+//     buffer, and a last small kernel adds a row's partials in piece order (deterministic, no
+//     float atomics).  Workgroup i only takes pieces of class i % 8, i.e. each XCD gathers only
+//     its own class of dense rows, so the eight L2 caches hold disjoint sets of popular rows.
 #include <algorithm>
 #include <cstdlib>
 #include <functional>
@@ -28,8 +29,8 @@
 namespace sgnn {
 
 constexpr int kBlock = 256;
-constexpr int kDefaultLongThreshold = 128;
-constexpr int kDefaultSegmentEdges = 512;
+constexpr int kDefaultLongThreshold = 128;  // rows with more edges go to the class-partitioned piece path
+constexpr int kDefaultPieceEdges = 32;      // minimum edges per piece of a long row
 
 __host__ __device__ constexpr int unroll_of(int nv) { return nv == 1 ? 8 : nv == 2 ? 4 : nv == 3 ? 3 : 2; }
 
@@ -52,66 +53,53 @@ __device__ __forceinline__ int64_t uniform64(int64_t v) {
     return (int64_t)(((uint64_t)hi << 32) | lo);
 }
 
-// Accumulate `deg` edges starting at colp/valp into acc for one feature tile.
-template <int VEC, int G, int NV, bool FLAVOURS>
-__device__ __forceinline__ void gather_edges(float (&acc)[NV][VEC], const int32_t *__restrict__ colp,
-                                             const float *__restrict__ valp, int deg,
-                                             const float *__restrict__ x, int64_t ldx, const int (&off)[NV],
-                                             const bool (&act)[NV], int lig) {
+// Accumulate the `deg` edges listed at colp into acc for one feature tile.  The weight of edge i is
+// val[eperm[i]] (val may be null = all ones).
+template <int VEC, int G, int NV>
+__device__ __forceinline__ void gather_piece(float (&acc)[NV][VEC], const int32_t *__restrict__ colp,
+                                             const int32_t *__restrict__ eperm, const float *__restrict__ val,
+                                             int deg, const float *__restrict__ x, int64_t ldx,
+                                             const int (&off)[NV], const bool (&act)[NV], int lig) {
     constexpr int U = unroll_of(NV);
+    // (col,val) pairs are fetched G at a time, one chunk ahead of the gathers that consume them.
+    int nc = 0;
+    float nw = 1.0f;
+    if (lig < deg) {
+        nc = __builtin_nontemporal_load(colp + lig);
+        if (val) nw = val[__builtin_nontemporal_load(eperm + lig)];
+    }
     for (int base = 0; base < deg; base += G) {
-        const int idx = base + lig;
-        int myc = 0;
-        float myw = 0.0f;
-        if (idx < deg) {
-            myc = __builtin_nontemporal_load(colp + idx);
-            myw = valp ? __builtin_nontemporal_load(valp + idx) : 1.0f;
+        const int myc = nc;
+        const float myw = nw;
+        const int nidx = base + G + lig;
+        if (nidx < deg) {
+            nc = __builtin_nontemporal_load(colp + nidx);
+            if (val) nw = val[__builtin_nontemporal_load(eperm + nidx)];
         }
         const int cnt = deg - base < G ? deg - base : G;
-        int j = 0;
-        for (; j + U <= cnt; j += U) {
+        for (int j = 0; j < cnt; j += U) {
             float xv[U][NV][VEC];
+            // U gathers back to back; past the end the last edge's row is fetched again (a cache
+            // hit) so that no branch separates the loads.
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int cf = group_bcast_i<G>(myc, j + u);
-                const float *xr = x + (int64_t)(cf & 0x7fffffff) * ldx;
-                if (FLAVOURS && cf < 0) {
+                const int src = j + u < cnt ? j + u : cnt - 1;
+                const int c = group_bcast_i<G>(myc, src);
+                const float *xr = x + (int64_t)c * ldx;
+#pragma unroll
+                for (int v = 0; v < NV; ++v)
+                    if (act[v]) vec_load<VEC>(xv[u][v], xr + off[v]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (j + u < cnt) {
+                    const float w = group_bcast_f<G>(myw, j + u);
 #pragma unroll
                     for (int v = 0; v < NV; ++v)
-                        if (act[v]) vec_load_nt<VEC>(xv[u][v], xr + off[v]);
-                } else {
 #pragma unroll
-                    for (int v = 0; v < NV; ++v)
-                        if (act[v]) vec_load<VEC>(xv[u][v], xr + off[v]);
+                        for (int k = 0; k < VEC; ++k) acc[v][k] = fmaf(w, xv[u][v][k], acc[v][k]);
                 }
             }
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const float w = group_bcast_f<G>(myw, j + u);
-#pragma unroll
-                for (int v = 0; v < NV; ++v)
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) acc[v][k] = fmaf(w, xv[u][v][k], acc[v][k]);
-            }
-        }
-        for (; j < cnt; ++j) {
-            const int cf = group_bcast_i<G>(myc, j);
-            const float w = group_bcast_f<G>(myw, j);
-            const float *xr = x + (int64_t)(cf & 0x7fffffff) * ldx;
-            float xv[NV][VEC];
-            if (FLAVOURS && cf < 0) {
-#pragma unroll
-                for (int v = 0; v < NV; ++v)
-                    if (act[v]) vec_load_nt<VEC>(xv[v], xr + off[v]);
-            } else {
-#pragma unroll
-                for (int v = 0; v < NV; ++v)
-                    if (act[v]) vec_load<VEC>(xv[v], xr + off[v]);
-            }
-#pragma unroll
-            for (int v = 0; v < NV; ++v)
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) acc[v][k] = fmaf(w, xv[v][k], acc[v][k]);
         }
     }
 }
@@ -193,13 +181,19 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
             }
         }
 
+        int nc = 0;
+        float nw = 1.0f;
+        if (lig < E) {
+            nc = __builtin_nontemporal_load(colp + lig);
+            if (valp) nw = __builtin_nontemporal_load(valp + lig);
+        }
         for (int base = 0; base < E; base += G) {
-            const int idx = base + lig;
-            int myc = 0;
-            float myw = 1.0f;
-            if (idx < E) {
-                myc = __builtin_nontemporal_load(colp + idx) & 0x7fffffff;
-                if (valp) myw = __builtin_nontemporal_load(valp + idx);
+            const int myc = nc;
+            const float myw = nw;
+            const int nidx = base + G + lig;  // next chunk, fetched one chunk ahead of its gathers
+            if (nidx < E) {
+                nc = __builtin_nontemporal_load(colp + nidx);
+                if (valp) nw = __builtin_nontemporal_load(valp + nidx);
             }
             const int cnt = E - base < G ? E - base : G;
             for (int j = 0; j < cnt; j += U) {
@@ -296,31 +290,32 @@ __global__ __launch_bounds__(kBlock) void spmm_empty_rows_kernel(const int32_t *
 }
 
 // ------------------------------------------------------------------------------------------------
-// Long rows, step 1: one workgroup per edge segment -> partial[s, :].
+// Long rows, step 1: pieces.  At plan time a long row's edges are regrouped by column class
+// (a hash of the column index, 8 classes) and each class run is cut into pieces; a piece is summed by one lane group into
+// partial[piece, :].  All pieces a workgroup handles belong to ONE class, and workgroup i takes
+// class i % 8: workgroups are dealt round-robin to the 8 XCDs, so every XCD gathers only the dense
+// rows of its own class and the eight 4 MB L2s hold eight DISJOINT sets of popular rows instead of
+// eight copies of the same set.
 // ------------------------------------------------------------------------------------------------
 template <int VEC, int G, int NV>
-__global__ __launch_bounds__(kBlock) void spmm_segment_kernel(
-    const int32_t *__restrict__ col, const float *__restrict__ val, const float *__restrict__ x,
-    float *__restrict__ partial, const int64_t *__restrict__ seg_begin, const int32_t *__restrict__ seg_len,
+__global__ __launch_bounds__(kBlock) void spmm_piece_kernel(
+    const int32_t *__restrict__ col_long, const int32_t *__restrict__ eperm, const float *__restrict__ val,
+    const float *__restrict__ x, float *__restrict__ partial, const int32_t *__restrict__ item_begin,
+    const int32_t *__restrict__ item_len, const int32_t *__restrict__ cls_list, const int32_t *__restrict__ cls_off,
     int F, int64_t ldx) {
     constexpr int GPB = kBlock / G;
     constexpr int TILE = G * VEC * NV;
-    __shared__ float red[GPB][TILE];
-    const int s = blockIdx.x;
     const int gid = threadIdx.x / G, lig = threadIdx.x % G;
-    const int64_t b = uniform64(seg_begin[s]);
-    const int len = __builtin_amdgcn_readfirstlane(seg_len[s]);
-    const int per = (len + GPB - 1) / GPB;
-    int my_b = gid * per;
-    int my_e = my_b + per < len ? my_b + per : len;
+    const int cls = blockIdx.x % kNumXCD;
+    const int idx = cls_off[cls] + (int)(blockIdx.x / kNumXCD) * GPB + gid;
+    if (idx >= cls_off[cls + 1]) return;
+    int item = cls_list[idx];
+    int b = item_begin[item], len = item_len[item];
     if constexpr (G == 64) {
-        my_b = __builtin_amdgcn_readfirstlane(my_b);
-        my_e = __builtin_amdgcn_readfirstlane(my_e);
+        item = __builtin_amdgcn_readfirstlane(item);
+        b = __builtin_amdgcn_readfirstlane(b);
+        len = __builtin_amdgcn_readfirstlane(len);
     }
-    const int my_deg = my_e > my_b ? my_e - my_b : 0;
-    const int32_t *colp = col + b + my_b;
-    const float *valp = val ? val + b + my_b : nullptr;
-
     for (int f0 = 0; f0 < F; f0 += TILE) {
         int off[NV];
         bool act[NV];
@@ -332,38 +327,29 @@ __global__ __launch_bounds__(kBlock) void spmm_segment_kernel(
 #pragma unroll
             for (int k = 0; k < VEC; ++k) acc[v][k] = 0.0f;
         }
-        gather_edges<VEC, G, NV, true>(acc, colp, valp, my_deg, x, ldx, off, act, lig);
+        gather_piece<VEC, G, NV>(acc, col_long + b, eperm + b, val, len, x, ldx, off, act, lig);
 #pragma unroll
         for (int v = 0; v < NV; ++v)
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) red[gid][(v * G + lig) * VEC + k] = acc[v][k];
-        __syncthreads();
-        const int width = F - f0 < TILE ? F - f0 : TILE;
-        for (int i = threadIdx.x; i < width; i += kBlock) {
-            float sum = red[0][i];
-#pragma unroll
-            for (int g = 1; g < GPB; ++g) sum += red[g][i];
-            partial[(int64_t)s * F + f0 + i] = sum;
-        }
-        __syncthreads();
+            if (act[v]) vec_store<VEC>(partial + (int64_t)item * F + off[v], acc[v]);
     }
 }
 
 // ------------------------------------------------------------------------------------------------
-// Long rows, step 2: add a row's segment partials in segment order, epilogue, store.
+// Long rows, step 2: add a row's piece partials in piece order, epilogue, store.
 // ------------------------------------------------------------------------------------------------
 template <int VEC, int G, int NV>
 __global__ __launch_bounds__(kBlock) void spmm_long_final_kernel(
-    const int32_t *__restrict__ long_rows, const int32_t *__restrict__ long_segptr,
+    const int32_t *__restrict__ long_rows, const int32_t *__restrict__ long_pbeg,
     const float *__restrict__ partial, float *__restrict__ out, int n_long, int F, int64_t ldo,
     int accumulate, const float *__restrict__ row_div) {
     constexpr int GPB = kBlock / G;
     constexpr int TILE = G * VEC * NV;
+    constexpr int UP = 8;
     const int gid = threadIdx.x / G, lig = threadIdx.x % G;
     const int li = blockIdx.x * GPB + gid;
     if (li >= n_long) return;
     const int64_t row = long_rows[li];
-    const int s0 = long_segptr[li], s1 = long_segptr[li + 1];
+    const int s0 = long_pbeg[li], s1 = long_pbeg[li + 1];
     float *orow = out + row * ldo;
     const float div = row_div ? row_div[row] : 1.0f;
     for (int f0 = 0; f0 < F; f0 += TILE) {
@@ -375,11 +361,20 @@ __global__ __launch_bounds__(kBlock) void spmm_long_final_kernel(
 #pragma unroll
             for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
             if (accumulate) vec_load_nt<VEC>(acc, orow + off);
-            for (int s = s0; s < s1; ++s) {
-                float p[VEC];
-                vec_load<VEC>(p, partial + (int64_t)s * F + off);
+            for (int s = s0; s < s1; s += UP) {
+                float p[UP][VEC];
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) acc[k] += p[k];
+                for (int u = 0; u < UP; ++u) {
+                    const int si = s + u < s1 ? s + u : s1 - 1;
+                    vec_load<VEC>(p[u], partial + (int64_t)si * F + off);
+                }
+#pragma unroll
+                for (int u = 0; u < UP; ++u) {
+                    if (s + u < s1) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) acc[k] += p[u][k];
+                    }
+                }
             }
             if (row_div) {
 #pragma unroll
@@ -391,37 +386,84 @@ __global__ __launch_bounds__(kBlock) void spmm_long_final_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
+// Plan-time: regroup every long row's edges by column class, keeping the CSR order inside a class
+// (a stable 8-way split done by one workgroup per row).
+// ------------------------------------------------------------------------------------------------
+// Column class: a multiplicative hash, NOT col % 8.  Dense row c starts at byte c * 4F, so a class
+// taken from the low bits of c would pin address bits that the L2 and HBM channel interleaving
+// use, and an XCD would then hammer a fraction of its cache channels.
+__device__ __forceinline__ int col_class(int32_t c) {
+    return (int)(((uint32_t)c * 0x9E3779B1u) >> 29);
+}
+
+__global__ __launch_bounds__(kBlock) void partition_long_rows_kernel(
+    const int64_t *__restrict__ rowptr, const int32_t *__restrict__ col, const int32_t *__restrict__ long_rows,
+    const int32_t *__restrict__ long_off, int32_t *__restrict__ col_long, int32_t *__restrict__ eperm,
+    int32_t *__restrict__ cls_count) {
+    __shared__ int cnt[kNumXCD], base[kNumXCD], wave_cnt[kBlock / 64][kNumXCD];
+    const int slot = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t row = long_rows[slot];
+    const int64_t b = rowptr[row];
+    const int n = (int)(rowptr[row + 1] - b);
+    const int dst0 = long_off[slot];
+    if (tid < kNumXCD) cnt[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < n; i += kBlock) atomicAdd(&cnt[col_class(col[b + i])], 1);
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int k = 0; k < kNumXCD; ++k) {
+            base[k] = run;
+            run += cnt[k];
+            cls_count[slot * kNumXCD + k] = cnt[k];
+        }
+    }
+    __syncthreads();
+    for (int c0 = 0; c0 < n; c0 += kBlock) {
+        const int i = c0 + tid;
+        const bool valid = i < n;
+        const int c = valid ? col[b + i] : 0;
+        const int k = col_class(c);
+        int my_rank = 0;
+#pragma unroll
+        for (int kk = 0; kk < kNumXCD; ++kk) {
+            const unsigned long long m = __ballot(valid && k == kk);
+            if (k == kk) my_rank = __popcll(m & ((1ull << lane) - 1ull));
+            if (lane == 0) wave_cnt[wave][kk] = __popcll(m);
+        }
+        __syncthreads();
+        if (valid) {
+            int pre = 0;
+            for (int w = 0; w < wave; ++w) pre += wave_cnt[w][k];
+            const int dst = dst0 + base[k] + pre + my_rank;
+            col_long[dst] = c;
+            eperm[dst] = (int32_t)(b + i);
+        }
+        __syncthreads();
+        if (tid < kNumXCD) {
+            int add = 0;
+            for (int w = 0; w < kBlock / 64; ++w) add += wave_cnt[w][tid];
+            base[tid] += add;
+        }
+        __syncthreads();
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Column index narrowing + range check.
 // ------------------------------------------------------------------------------------------------
 template <typename SrcT>
 __global__ __launch_bounds__(kBlock) void narrow_cols_kernel(const SrcT *__restrict__ src, int32_t *__restrict__ dst,
-                                                             int64_t n, int64_t K, int *__restrict__ bad,
-                                                             int *__restrict__ popularity) {
+                                                             int64_t n, int64_t K, int *__restrict__ bad) {
     int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     bool any_bad = false;
     for (; i < n; i += stride) {
         const int64_t c = (int64_t)src[i];
-        if (c < 0 || c >= K) {
-            any_bad = true;
-        } else if (popularity) {
-            atomicAdd(popularity + c, 1);
-        }
+        if (c < 0 || c >= K) any_bad = true;
         dst[i] = (int32_t)c;
     }
     if (any_bad) atomicOr(bad, 1);
-}
-
-// Marks the gathers of unpopular dense rows as streaming (sign bit of the stored column index):
-// they are fetched with non-temporal loads so that they do not evict the popular rows from L2.
-__global__ __launch_bounds__(kBlock) void mark_cold_cols_kernel(int32_t *__restrict__ col, int64_t n,
-                                                                const int *__restrict__ popularity, int hot_min) {
-    int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * kBlock;
-    for (; i < n; i += stride) {
-        const int32_t c = col[i];
-        if (popularity[c] < hot_min) col[i] = c | (int32_t)0x80000000;
-    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -432,17 +474,18 @@ struct ShortArgs {
     const int2 *chunks; int n_chunks; const int32_t *empty_rows; int n_empty;
     int F; int64_t ldx, ldo; int accumulate; const float *row_div;
 };
-struct SegArgs {
-    const int32_t *col; const float *val; const float *x; float *partial; const int64_t *seg_begin;
-    const int32_t *seg_len; int n_seg; int F; int64_t ldx;
+struct PieceArgs {
+    const int32_t *col_long; const int32_t *eperm; const float *val; const float *x; float *partial;
+    const int32_t *item_begin; const int32_t *item_len; const int32_t *cls_list; const int32_t *cls_off;
+    int max_cls_items; int F; int64_t ldx;
 };
 struct FinalArgs {
-    const int32_t *long_rows; const int32_t *long_segptr; const float *partial; float *out; int n_long;
+    const int32_t *long_rows; const int32_t *long_pbeg; const float *partial; float *out; int n_long;
     int F; int64_t ldo; int accumulate; const float *row_div;
 };
 
 template <int VEC, int G, int NV>
-static void launch_all(const ShortArgs &a, const SegArgs &s, const FinalArgs &f, hipStream_t st) {
+static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &f, hipStream_t st) {
     constexpr int GPB = kBlock / G;
     if (a.n_chunks > 0) {
         const uint32_t nb = (uint32_t)((a.n_chunks + GPB - 1) / GPB);
@@ -456,16 +499,18 @@ static void launch_all(const ShortArgs &a, const SegArgs &s, const FinalArgs &f,
         hipLaunchKernelGGL((spmm_empty_rows_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, a.empty_rows, a.n_empty,
                            a.out, a.F, a.ldo, a.accumulate, a.row_div);
     }
-    if (s.n_seg > 0) {
+    if (f.n_long > 0) {
         {
-            ProfScope prof(K_SPMM_SEGMENT, st);
-            hipLaunchKernelGGL((spmm_segment_kernel<VEC, G, NV>), dim3(s.n_seg), dim3(kBlock), 0, st, s.col, s.val,
-                               s.x, s.partial, s.seg_begin, s.seg_len, s.F, s.ldx);
+            // workgroup i serves class i % 8: grid = 8 * (workgroups of the fullest class)
+            const uint32_t nb = (uint32_t)kNumXCD * (uint32_t)((s.max_cls_items + GPB - 1) / GPB);
+            ProfScope prof(K_SPMM_PIECE, st);
+            hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, s.col_long, s.eperm,
+                               s.val, s.x, s.partial, s.item_begin, s.item_len, s.cls_list, s.cls_off, s.F, s.ldx);
         }
         const uint32_t nb = (uint32_t)((f.n_long + GPB - 1) / GPB);
         ProfScope prof(K_SPMM_LONG_FINAL, st);
         hipLaunchKernelGGL((spmm_long_final_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, f.long_rows,
-                           f.long_segptr, f.partial, f.out, f.n_long, f.F, f.ldo, f.accumulate, f.row_div);
+                           f.long_pbeg, f.partial, f.out, f.n_long, f.F, f.ldo, f.accumulate, f.row_div);
     }
 }
 
@@ -473,7 +518,7 @@ static void launch_all(const ShortArgs &a, const SegArgs &s, const FinalArgs &f,
 static int group_width(int nvec) { return nvec <= 8 ? 8 : nvec <= 16 ? 16 : nvec <= 32 ? 32 : 64; }
 
 template <int VEC>
-static int dispatch_shape(int nvec, const ShortArgs &a, const SegArgs &s, const FinalArgs &f, hipStream_t st) {
+static int dispatch_shape(int nvec, const ShortArgs &a, const PieceArgs &s, const FinalArgs &f, hipStream_t st) {
     if (nvec <= 8) launch_all<VEC, 8, 1>(a, s, f, st);
     else if (nvec <= 16) launch_all<VEC, 16, 1>(a, s, f, st);
     else if (nvec <= 32) launch_all<VEC, 32, 1>(a, s, f, st);
@@ -491,27 +536,32 @@ static int dispatch_shape(int nvec, const ShortArgs &a, const SegArgs &s, const 
 
 using namespace sgnn;
 
-// Number of dense rows treated as "popular" (kept on the normal, cache-retaining load path).
-// Everything else is gathered with streaming loads.  0 disables the classification.
-static int hot_rows_budget() {
-    const char *e = getenv("SGNN_SPMM_HOT_ROWS");
-    return e ? atoi(e) : 8192;
+static int env_int(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : dflt;
 }
 
 struct sgnn_spmm_plan {
     int device = 0;
     int64_t M = 0, K = 0, nnz = 0;
-    int long_thresh = 0, seg_edges = 0, hot_min = 0;
+    int long_thresh = 0, piece_edges = 0;
     int64_t *rowptr = nullptr;  // device, owned
     int32_t *col = nullptr;     // device, owned
-    int64_t n_long = 0, n_seg = 0, long_edges = 0;
-    int32_t *long_rows = nullptr;    // [n_long]
-    int32_t *long_segptr = nullptr;  // [n_long + 1]
-    int64_t *seg_begin = nullptr;    // [n_seg]
-    int32_t *seg_len = nullptr;      // [n_seg]
-    float *partial = nullptr;        // [n_seg * F], grown on demand
+    // long rows
+    int64_t n_long = 0, n_items = 0, long_edges = 0;
+    int max_cls_items = 0;
+    int32_t *long_rows = nullptr;   // [n_long] row ids
+    int32_t *long_pbeg = nullptr;   // [n_long + 1] first piece of each long row
+    int32_t *col_long = nullptr;    // [long_edges] columns regrouped by class inside each long row
+    int32_t *eperm = nullptr;       // [long_edges] original edge index of each regrouped edge
+    int32_t *item_begin = nullptr;  // [n_items] offset into col_long / eperm
+    int32_t *item_len = nullptr;    // [n_items]
+    int32_t *cls_list = nullptr;    // [n_items] piece ids grouped by class
+    int32_t *cls_off = nullptr;     // [9]
+    float *partial = nullptr;       // [n_items * F], grown on demand
     size_t partial_floats = 0;
-    int32_t *empty_rows = nullptr;   // [n_empty]
+    // rows without edges
+    int32_t *empty_rows = nullptr;
     int64_t n_empty = 0;
     // Short-row chunks, one list per chunk row limit (7, 15, 31), built on first use.
     std::vector<int64_t> h_rowptr;
@@ -519,12 +569,11 @@ struct sgnn_spmm_plan {
     int64_t n_chunks[3] = {-1, -1, -1};
 };
 
-constexpr int kChunkEdges = 128;  // target edges per short-row chunk
-
 // Cuts the short, non-empty rows into chunks of consecutive rows: at most `limit` rows and about
-// kChunkEdges edges each, never containing a long row, starting and ending on a non-empty row.
+// `target` edges each, never containing a long row, starting and ending on a non-empty row.
 static int build_chunks(sgnn_spmm_plan *p, int which, hipStream_t st) {
     const int limit = which == 0 ? 7 : which == 1 ? 15 : 31;
+    const int target = env_int("SGNN_SPMM_CHUNK_EDGES", 128);
     const std::vector<int64_t> &rp = p->h_rowptr;
     std::vector<int2> out;
     const int64_t M = p->M;
@@ -534,7 +583,7 @@ static int build_chunks(sgnn_spmm_plan *p, int which, hipStream_t st) {
         if (d0 == 0 || d0 > p->long_thresh) { ++m; continue; }
         const int64_t start = m;
         int64_t last = m, edges = 0;
-        while (m < M && m - start < limit && edges < kChunkEdges) {
+        while (m < M && m - start < limit && edges < target) {
             const int64_t d = rp[m + 1] - rp[m];
             if (d > p->long_thresh) break;
             if (d > 0) last = m;
@@ -557,9 +606,13 @@ extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     (void)hipFree(p->rowptr);
     (void)hipFree(p->col);
     (void)hipFree(p->long_rows);
-    (void)hipFree(p->long_segptr);
-    (void)hipFree(p->seg_begin);
-    (void)hipFree(p->seg_len);
+    (void)hipFree(p->long_pbeg);
+    (void)hipFree(p->col_long);
+    (void)hipFree(p->eperm);
+    (void)hipFree(p->item_begin);
+    (void)hipFree(p->item_len);
+    (void)hipFree(p->cls_list);
+    (void)hipFree(p->cls_off);
     (void)hipFree(p->partial);
     (void)hipFree(p->empty_rows);
     for (int i = 0; i < 3; ++i) (void)hipFree(p->chunks[i]);
@@ -567,12 +620,18 @@ extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     return SGNN_OK;
 }
 
+template <typename T>
+static int upload(T **dst, const std::vector<T> &src, hipStream_t st) {
+    if (src.empty()) return SGNN_OK;
+    SGNN_HIP_CHECK(hipMalloc(dst, sizeof(T) * src.size()));
+    SGNN_HIP_CHECK(hipMemcpyAsync(*dst, src.data(), sizeof(T) * src.size(), hipMemcpyHostToDevice, st));
+    return SGNN_OK;
+}
+
 static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void *col, int col_is_i64,
-                            int long_row_threshold, int segment_edges, hipStream_t st) {
+                            hipStream_t st) {
     const int64_t M = p->M, K = p->K, nnz = p->nnz;
     SGNN_HIP_CHECK(hipGetDevice(&p->device));
-    p->long_thresh = long_row_threshold > 0 ? long_row_threshold : kDefaultLongThreshold;
-    p->seg_edges = segment_edges > 0 ? segment_edges : kDefaultSegmentEdges;
 
     std::vector<int64_t> &h_rowptr = p->h_rowptr;
     h_rowptr.resize((size_t)M + 1);
@@ -584,92 +643,119 @@ static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void
     if (h_rowptr[M] != nnz)
         return fail(SGNN_ERR_RANGE, "rowptr[M] = %lld but nnz = %lld", (long long)h_rowptr[M], (long long)nnz);
 
-    std::vector<int32_t> long_rows, long_segptr, seg_len, empty_rows;
-    std::vector<int64_t> seg_begin;
-    long_segptr.push_back(0);
+    // ---- row classes ------------------------------------------------------------------------
+    std::vector<int32_t> long_rows, long_off, empty_rows;
     for (int64_t m = 0; m < M; ++m) {
-        const int64_t b = h_rowptr[m], deg = h_rowptr[m + 1] - b;
+        const int64_t deg = h_rowptr[m + 1] - h_rowptr[m];
         if (deg == 0) empty_rows.push_back((int32_t)m);
         if (deg <= p->long_thresh) continue;
         long_rows.push_back((int32_t)m);
-        for (int64_t o = 0; o < deg; o += p->seg_edges) {
-            seg_begin.push_back(b + o);
-            seg_len.push_back((int32_t)std::min<int64_t>(p->seg_edges, deg - o));
-        }
-        if (seg_begin.size() > (size_t)INT32_MAX) return fail(SGNN_ERR_ARG, "too many long-row segments");
-        long_segptr.push_back((int32_t)seg_begin.size());
+        long_off.push_back((int32_t)p->long_edges);
         p->long_edges += deg;
     }
     p->n_long = (int64_t)long_rows.size();
-    p->n_seg = (int64_t)seg_begin.size();
     p->n_empty = (int64_t)empty_rows.size();
-    if (p->n_empty > 0) {
-        SGNN_HIP_CHECK(hipMalloc(&p->empty_rows, sizeof(int32_t) * empty_rows.size()));
-        SGNN_HIP_CHECK(hipMemcpyAsync(p->empty_rows, empty_rows.data(), sizeof(int32_t) * empty_rows.size(), hipMemcpyHostToDevice, st));
-        SGNN_HIP_CHECK(hipStreamSynchronize(st));
-    }
 
+    // ---- device copies: rowptr, narrowed + range-checked columns -------------------------------
     SGNN_HIP_CHECK(hipMalloc(&p->rowptr, sizeof(int64_t) * (size_t)(M + 1)));
     SGNN_HIP_CHECK(hipMemcpyAsync(p->rowptr, rowptr, sizeof(int64_t) * (size_t)(M + 1), hipMemcpyDeviceToDevice, st));
     SGNN_HIP_CHECK(hipMalloc(&p->col, sizeof(int32_t) * (size_t)std::max<int64_t>(nnz, 1)));
+    int rc = upload(&p->empty_rows, empty_rows, st);
+    if (rc != SGNN_OK) return rc;
     if (nnz > 0) {
-        int *bad = nullptr;  // [0] = range flag, [1 .. K] = per-column popularity (in-degree)
-        const int hot_rows = hot_rows_budget();
-        const bool want_pop = hot_rows > 0 && K > hot_rows;
-        SGNN_HIP_CHECK(hipMalloc(&bad, sizeof(int) * (size_t)(1 + (want_pop ? K : 0))));
-        SGNN_HIP_CHECK(hipMemsetAsync(bad, 0, sizeof(int) * (size_t)(1 + (want_pop ? K : 0)), st));
-        int *pop = want_pop ? bad + 1 : nullptr;
+        int *bad = nullptr;
+        SGNN_HIP_CHECK(hipMalloc(&bad, sizeof(int)));
+        SGNN_HIP_CHECK(hipMemsetAsync(bad, 0, sizeof(int), st));
         const int nb = (int)std::min<int64_t>((nnz + kBlock - 1) / kBlock, 65536);
         if (col_is_i64)
-            hipLaunchKernelGGL((narrow_cols_kernel<int64_t>), dim3(nb), dim3(kBlock), 0, st, (const int64_t *)col, p->col, nnz, K, bad, pop);
+            hipLaunchKernelGGL((narrow_cols_kernel<int64_t>), dim3(nb), dim3(kBlock), 0, st, (const int64_t *)col, p->col, nnz, K, bad);
         else
-            hipLaunchKernelGGL((narrow_cols_kernel<int32_t>), dim3(nb), dim3(kBlock), 0, st, (const int32_t *)col, p->col, nnz, K, bad, pop);
-        std::vector<int> h_pop(1 + (want_pop ? (size_t)K : 0));
+            hipLaunchKernelGGL((narrow_cols_kernel<int32_t>), dim3(nb), dim3(kBlock), 0, st, (const int32_t *)col, p->col, nnz, K, bad);
+        int h_bad = 0;
         hipError_t e1 = hipGetLastError();
-        hipError_t e2 = hipMemcpyAsync(h_pop.data(), bad, sizeof(int) * h_pop.size(), hipMemcpyDeviceToHost, st);
+        hipError_t e2 = hipMemcpyAsync(&h_bad, bad, sizeof(int), hipMemcpyDeviceToHost, st);
         hipError_t e3 = hipStreamSynchronize(st);
-        if (e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess && h_pop[0] == 0 && want_pop) {
-            // popularity of the hot_rows-th most popular column = the admission threshold
-            std::vector<int> sorted(h_pop.begin() + 1, h_pop.end());
-            std::nth_element(sorted.begin(), sorted.begin() + hot_rows, sorted.end(), std::greater<int>());
-            const int hot_min = std::max(sorted[hot_rows] + 1, 2);
-            hipLaunchKernelGGL(mark_cold_cols_kernel, dim3(nb), dim3(kBlock), 0, st, p->col, nnz, pop, hot_min);
-            e1 = hipGetLastError();
-            e3 = hipStreamSynchronize(st);
-            p->hot_min = hot_min;
-        }
         (void)hipFree(bad);
         SGNN_HIP_CHECK(e1);
         SGNN_HIP_CHECK(e2);
         SGNN_HIP_CHECK(e3);
-        if (h_pop[0]) return fail(SGNN_ERR_RANGE, "a column index lies outside [0, %lld)", (long long)K);
+        if (h_bad) return fail(SGNN_ERR_RANGE, "a column index lies outside [0, %lld)", (long long)K);
     }
+
+    // ---- long rows: regroup by column class, cut into pieces ----------------------------------
     if (p->n_long > 0) {
-        SGNN_HIP_CHECK(hipMalloc(&p->long_rows, sizeof(int32_t) * long_rows.size()));
-        SGNN_HIP_CHECK(hipMalloc(&p->long_segptr, sizeof(int32_t) * long_segptr.size()));
-        SGNN_HIP_CHECK(hipMalloc(&p->seg_begin, sizeof(int64_t) * seg_begin.size()));
-        SGNN_HIP_CHECK(hipMalloc(&p->seg_len, sizeof(int32_t) * seg_len.size()));
-        SGNN_HIP_CHECK(hipMemcpyAsync(p->long_rows, long_rows.data(), sizeof(int32_t) * long_rows.size(), hipMemcpyHostToDevice, st));
-        SGNN_HIP_CHECK(hipMemcpyAsync(p->long_segptr, long_segptr.data(), sizeof(int32_t) * long_segptr.size(), hipMemcpyHostToDevice, st));
-        SGNN_HIP_CHECK(hipMemcpyAsync(p->seg_begin, seg_begin.data(), sizeof(int64_t) * seg_begin.size(), hipMemcpyHostToDevice, st));
-        SGNN_HIP_CHECK(hipMemcpyAsync(p->seg_len, seg_len.data(), sizeof(int32_t) * seg_len.size(), hipMemcpyHostToDevice, st));
-        SGNN_HIP_CHECK(hipStreamSynchronize(st));  // the host vectors die at return
+        if ((rc = upload(&p->long_rows, long_rows, st)) != SGNN_OK) return rc;
+        int32_t *d_long_off = nullptr, *d_cls_count = nullptr;
+        if ((rc = upload(&d_long_off, long_off, st)) != SGNN_OK) return rc;
+        SGNN_HIP_CHECK(hipMalloc(&d_cls_count, sizeof(int32_t) * (size_t)p->n_long * kNumXCD));
+        SGNN_HIP_CHECK(hipMalloc(&p->col_long, sizeof(int32_t) * (size_t)p->long_edges));
+        SGNN_HIP_CHECK(hipMalloc(&p->eperm, sizeof(int32_t) * (size_t)p->long_edges));
+        hipLaunchKernelGGL(partition_long_rows_kernel, dim3((uint32_t)p->n_long), dim3(kBlock), 0, st, p->rowptr, p->col,
+                           p->long_rows, d_long_off, p->col_long, p->eperm, d_cls_count);
+        std::vector<int32_t> cls_count((size_t)p->n_long * kNumXCD);
+        hipError_t e1 = hipGetLastError();
+        hipError_t e2 = hipMemcpyAsync(cls_count.data(), d_cls_count, sizeof(int32_t) * cls_count.size(), hipMemcpyDeviceToHost, st);
+        hipError_t e3 = hipStreamSynchronize(st);
+        (void)hipFree(d_long_off);
+        (void)hipFree(d_cls_count);
+        SGNN_HIP_CHECK(e1);
+        SGNN_HIP_CHECK(e2);
+        SGNN_HIP_CHECK(e3);
+
+        std::vector<int32_t> item_begin, item_len, long_pbeg, cls_off(kNumXCD + 1, 0);
+        std::vector<std::vector<int32_t>> cls_items(kNumXCD);
+        long_pbeg.push_back(0);
+        for (int64_t slot = 0; slot < p->n_long; ++slot) {
+            int32_t base = long_off[slot];
+            for (int c = 0; c < kNumXCD; ++c) {
+                const int32_t n = cls_count[slot * kNumXCD + c];
+                if (n == 0) continue;
+                // at most 32 pieces per (row, class) so that the final sum stays short
+                const int32_t len = std::max<int32_t>(p->piece_edges, (n + 31) / 32);
+                for (int32_t o = 0; o < n; o += len) {
+                    cls_items[c].push_back((int32_t)item_begin.size());
+                    item_begin.push_back(base + o);
+                    item_len.push_back(std::min<int32_t>(len, n - o));
+                }
+                base += n;
+            }
+            if (item_begin.size() > (size_t)INT32_MAX / 2) return fail(SGNN_ERR_ARG, "too many long-row pieces");
+            long_pbeg.push_back((int32_t)item_begin.size());
+        }
+        p->n_items = (int64_t)item_begin.size();
+        std::vector<int32_t> cls_list;
+        cls_list.reserve(item_begin.size());
+        for (int c = 0; c < kNumXCD; ++c) {
+            cls_off[c] = (int32_t)cls_list.size();
+            cls_list.insert(cls_list.end(), cls_items[c].begin(), cls_items[c].end());
+            p->max_cls_items = std::max<int>(p->max_cls_items, (int)cls_items[c].size());
+        }
+        cls_off[kNumXCD] = (int32_t)cls_list.size();
+        if ((rc = upload(&p->long_pbeg, long_pbeg, st)) != SGNN_OK) return rc;
+        if ((rc = upload(&p->item_begin, item_begin, st)) != SGNN_OK) return rc;
+        if ((rc = upload(&p->item_len, item_len, st)) != SGNN_OK) return rc;
+        if ((rc = upload(&p->cls_list, cls_list, st)) != SGNN_OK) return rc;
+        if ((rc = upload(&p->cls_off, cls_off, st)) != SGNN_OK) return rc;
     }
+    SGNN_HIP_CHECK(hipStreamSynchronize(st));  // the host vectors die at return
     return SGNN_OK;
 }
 
 extern "C" int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int col_is_i64, int64_t M, int64_t K,
-                                     int64_t nnz, int long_row_threshold, int segment_edges, sgnn_stream_t stream,
-                                     sgnn_spmm_plan **plan_out) {
+                                     int64_t nnz, int long_row_threshold, int piece_edges,
+                                     sgnn_stream_t stream, sgnn_spmm_plan **plan_out) {
     SGNN_REQUIRE(plan_out != nullptr, "plan_out is null");
     *plan_out = nullptr;
     SGNN_REQUIRE(rowptr != nullptr, "rowptr is null");
     SGNN_REQUIRE(M >= 0 && K >= 0 && nnz >= 0, "negative size (M=%lld K=%lld nnz=%lld)", (long long)M, (long long)K, (long long)nnz);
-    SGNN_REQUIRE(M < INT32_MAX && K < INT32_MAX, "M and K must fit 31 bits (M=%lld K=%lld)", (long long)M, (long long)K);
+    SGNN_REQUIRE(M < INT32_MAX && K < INT32_MAX && nnz < INT32_MAX,
+                 "M, K and nnz must fit 31 bits (M=%lld K=%lld nnz=%lld)", (long long)M, (long long)K, (long long)nnz);
     SGNN_REQUIRE(nnz == 0 || col != nullptr, "col is null with nnz=%lld", (long long)nnz);
     sgnn_spmm_plan *p = new sgnn_spmm_plan();
     p->M = M; p->K = K; p->nnz = nnz;
-    const int rc = plan_create_impl(p, rowptr, col, col_is_i64, long_row_threshold, segment_edges, (hipStream_t)stream);
+    p->long_thresh = long_row_threshold > 0 ? long_row_threshold : env_int("SGNN_SPMM_LONG_THRESHOLD", kDefaultLongThreshold);
+    p->piece_edges = piece_edges > 0 ? piece_edges : env_int("SGNN_SPMM_PIECE_EDGES", kDefaultPieceEdges);
+    const int rc = plan_create_impl(p, rowptr, col, col_is_i64, (hipStream_t)stream);
     if (rc != SGNN_OK) {
         sgnn_spmm_plan_destroy(p);
         return rc;
@@ -680,8 +766,8 @@ extern "C" int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int
 
 extern "C" int sgnn_spmm_plan_info(const sgnn_spmm_plan *p, int64_t info[8]) {
     SGNN_REQUIRE(p != nullptr && info != nullptr, "null argument");
-    info[0] = p->M; info[1] = p->K; info[2] = p->nnz; info[3] = p->n_long; info[4] = p->n_seg;
-    info[5] = p->long_edges; info[6] = p->long_thresh; info[7] = p->seg_edges;
+    info[0] = p->M; info[1] = p->K; info[2] = p->nnz; info[3] = p->n_long; info[4] = p->n_items;
+    info[5] = p->long_edges; info[6] = p->long_thresh; info[7] = p->piece_edges;
     return SGNN_OK;
 }
 
@@ -705,8 +791,8 @@ extern "C" int sgnn_spmm_csr_f32(sgnn_spmm_plan *p, const float *val, const floa
     SGNN_HIP_CHECK(hipGetDevice(&dev));
     SGNN_REQUIRE(dev == p->device, "plan was created on device %d, current device is %d", p->device, dev);
 
-    if (p->n_seg > 0) {
-        const size_t need = (size_t)p->n_seg * (size_t)F;
+    if (p->n_items > 0) {
+        const size_t need = (size_t)p->n_items * (size_t)F;
         if (need > p->partial_floats) {
             // The old buffer may still be read by work queued on another stream: drain first.
             SGNN_HIP_CHECK(hipDeviceSynchronize());
@@ -729,8 +815,9 @@ extern "C" int sgnn_spmm_csr_f32(sgnn_spmm_plan *p, const float *val, const floa
     }
     ShortArgs a{p->rowptr, p->col, val, x, out, p->chunks[which], (int)p->n_chunks[which], p->empty_rows,
                 (int)p->n_empty, (int)F, ldx, ldo, accumulate, row_div};
-    SegArgs s{p->col, val, x, p->partial, p->seg_begin, p->seg_len, (int)p->n_seg, (int)F, ldx};
-    FinalArgs f{p->long_rows, p->long_segptr, p->partial, out, (int)p->n_long, (int)F, ldo, accumulate, row_div};
+    PieceArgs s{p->col_long, p->eperm, val, x, p->partial, p->item_begin, p->item_len, p->cls_list, p->cls_off,
+                p->max_cls_items, (int)F, ldx};
+    FinalArgs f{p->long_rows, p->long_pbeg, p->partial, out, (int)p->n_long, (int)F, ldo, accumulate, row_div};
     if (vec == 4) dispatch_shape<4>(nvec, a, s, f, st);
     else if (vec == 2) dispatch_shape<2>(nvec, a, s, f, st);
     else dispatch_shape<1>(nvec, a, s, f, st);

@@ -90,7 +90,7 @@ class SpmmPlan:
     and 32-bit column indices plus the long-row segments; build once, reuse every call -- the role
     row_splits play in the reference (super_gnn/ops/spmm_kernel.py:49-58)."""
 
-    def __init__(self, rowptr, col, num_cols, long_row_threshold=0, segment_edges=0):
+    def __init__(self, rowptr, col, num_cols, long_row_threshold=0, piece_edges=0):
         _want(rowptr, torch.int64, "rowptr")
         if col.dtype not in (torch.int64, torch.int32):
             raise TypeError(f"col must be int64 or int32, got {col.dtype}")
@@ -104,14 +104,14 @@ class SpmmPlan:
             raise ValueError("rowptr must have at least one entry")
         h = ctypes.c_void_p()
         check(lib.sgnn_spmm_plan_create(_ptr(rp), _ptr(cl), int(cl.dtype == torch.int64), self.M, self.K, self.nnz,
-                                        int(long_row_threshold), int(segment_edges), _stream(), ctypes.byref(h)))
+                                        int(long_row_threshold), int(piece_edges), _stream(), ctypes.byref(h)))
         self._h = h
         self.device = dev
 
     def info(self):
         buf = (ctypes.c_int64 * 8)()
         check(lib.sgnn_spmm_plan_info(self._h, buf))
-        keys = ("M", "K", "nnz", "long_rows", "segments", "long_edges", "long_row_threshold", "segment_edges")
+        keys = ("M", "K", "nnz", "long_rows", "pieces", "long_edges", "long_row_threshold", "piece_edges")
         return dict(zip(keys, list(buf)))
 
     def run(self, value, mat, out, accumulate=True, row_div=None):

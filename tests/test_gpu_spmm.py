@@ -26,7 +26,7 @@ def _run_gpu(rowptr, col, val, x, init, accumulate, row_div=None, col_dtype=torc
     ops = _gpu()
     dev = torch.device("cuda:0")
     plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev).to(col_dtype), x.shape[0],
-                        long_row_threshold=thresh, segment_edges=seg)
+                        long_row_threshold=thresh, piece_edges=seg)
     out = torch.from_numpy(init.copy()).to(dev)
     plan.run(torch.from_numpy(val).to(dev) if val is not None else None, torch.from_numpy(x).to(dev), out,
              accumulate=accumulate, row_div=torch.from_numpy(row_div).to(dev) if row_div is not None else None)
@@ -110,7 +110,7 @@ def test_long_rows_segment_path(F, thresh, seg):
     S, deg = _abs_sum64(rowptr, col, val, x, init), np.diff(rowptr)
     got, plan = _run_gpu(rowptr, col, val, x, init, accumulate=True, thresh=thresh, seg=seg)
     info = plan.info()
-    assert info["long_rows"] >= 9 and info["segments"] >= info["long_rows"]
+    assert info["long_rows"] >= 9 and info["pieces"] >= info["long_rows"]
     _assert_close(got, want, f64, S, deg, what=f"long rows F={F}")
     short = np.diff(rowptr) <= thresh
     assert np.array_equal(got[short], want[short])
