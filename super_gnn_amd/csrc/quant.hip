@@ -11,6 +11,7 @@
 #include <algorithm>
 #include <cfloat>
 #include <climits>
+#include <cstdlib>
 
 #include "common.hpp"
 
@@ -98,7 +99,7 @@ __device__ __forceinline__ uint32_t quant_code(float x, float zp, float sc) {
 // Fused quantize + pack, row-group layout.  One group of G lanes handles kRowsPerGroup fp32 rows
 // (= 1 packed row at int2, 2 at int4, 4 at int8); G*VEC*NV >= F so a row lives in registers.
 // ------------------------------------------------------------------------------------------------
-template <int BITS, int VEC, int G, int NV>
+template <int BITS, int VEC, int G, int NV, bool kForceExactDivision>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
     const float *__restrict__ x, uint8_t *__restrict__ q, float *__restrict__ params,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
@@ -195,6 +196,65 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
         if (lig == 0) *reinterpret_cast<float2 *>(params + row[r] * 2) = make_float2(mn, s);
     }
 
+    // Codes.  The reference's code is RNE(RN((x - zp) / scale)).  A correctly rounded fp32 division
+    // costs ~15 instructions per element, which would make this streaming kernel ALU-bound, so the
+    // quotient is first formed as (x - zp) * RN(1/scale): that product is within 2^-23 relative of
+    // the true quotient, the IEEE quotient within 2^-24, and both are below 256, so the two differ
+    // by less than 2^-14.  If the product is further than 2^-14 from every half-integer, rounding
+    // it gives the same integer as rounding the IEEE quotient.  Any lane that sees an element
+    // inside that guard band (about 1 in 8000), or a row whose scale is outside the range where
+    // the reciprocal is a normal number, recomputes its elements with the IEEE division, so the
+    // stored bytes are always those of the exact formula.
+    float rinv[R];
+    bool lane_exact = kForceExactDivision;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        rinv[r] = 1.0f / sc[r];
+        if (valid[r] && !(sc[r] >= 0x1p-100f && sc[r] <= 0x1p100f)) lane_exact = true;
+    }
+    uint32_t words[NPR][NV];
+#pragma unroll
+    for (int pi = 0; pi < NPR; ++pi) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            uint32_t word = 0;
+            if (act[v]) {
+#pragma unroll
+                for (int k = 0; k < EPB; ++k) {
+                    const int r = pi * EPB + k;
+                    if (!valid[r]) continue;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        const float qf = (xv[r][v][e] - zp[r]) * rinv[r];
+                        const float ri = rintf(qf);
+                        if (!(fabsf(qf - ri) < 0.5f - 0x1p-14f)) lane_exact = true;
+                        word |= (uint32_t)ri << (8 * e + (EPB - 1 - k) * BITS);
+                    }
+                }
+            }
+            words[pi][v] = word;
+        }
+    }
+    if (lane_exact) {
+#pragma unroll
+        for (int pi = 0; pi < NPR; ++pi) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                uint32_t word = 0;
+                if (act[v]) {
+#pragma unroll
+                    for (int k = 0; k < EPB; ++k) {
+                        const int r = pi * EPB + k;
+                        if (!valid[r]) continue;
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e)
+                            word |= quant_code(xv[r][v][e], zp[r], sc[r]) << (8 * e + (EPB - 1 - k) * BITS);
+                    }
+                }
+                words[pi][v] = word;
+            }
+        }
+    }
 #pragma unroll
     for (int pi = 0; pi < NPR; ++pi) {
         const int gp = unit * NPR + pi;
@@ -203,18 +263,164 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             if (!act[v]) continue;
-            uint32_t word = 0;
-#pragma unroll
-            for (int k = 0; k < EPB; ++k) {
-                const int r = pi * EPB + k;
-                if (!valid[r]) continue;
-#pragma unroll
-                for (int e = 0; e < VEC; ++e)
-                    word |= quant_code(xv[r][v][e], zp[r], sc[r]) << (8 * e + (EPB - 1 - k) * BITS);
-            }
+            const uint32_t word = words[pi][v];
             if constexpr (VEC == 4) __builtin_nontemporal_store(word, reinterpret_cast<uint32_t *>(qr + off[v]));
             else if constexpr (VEC == 2) __builtin_nontemporal_store((uint16_t)word, reinterpret_cast<uint16_t *>(qr + off[v]));
             else qr[off[v]] = (uint8_t)word;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Fused quantize + pack, row-group layout, one fp32 row per 16 lanes (float4 lanes, F <= 1024).
+//
+// A 16-lane DPP row owns one fp32 row (NV float4 per lane), so the per-row min/max reductions are
+// four DPP butterfly steps with no cross-row traffic, and the per-row scalars (zero_point, scale,
+// reciprocal) are computed once per lane instead of once per row per lane.  A wavefront handles
+// 4*RL consecutive rows (RL rows per lane, chosen so that every lane keeps >= 4 loads in flight);
+// the four DPP rows hold four consecutive fp32 rows, i.e. exactly the rows that share a packed byte
+// at int2 (two DPP rows at int4), so packing is a shift in each lane followed by an OR across DPP
+// rows.
+// ------------------------------------------------------------------------------------------------
+template <int BITS, int NV, int RL, bool kForceExactDivision>
+__global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
+    const float *__restrict__ x, uint8_t *__restrict__ q, float *__restrict__ params,
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
+    constexpr int EPB = 8 / BITS;
+    constexpr int VEC = 4;
+    const int lane = threadIdx.x & 63, d = lane >> 4, l16 = lane & 15;
+    const int unit = blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
+    if (unit >= n_units) return;  // wave-uniform
+
+    int64_t row[RL];
+    bool valid[RL];
+    int gp[RL];
+#pragma unroll
+    for (int rl = 0; rl < RL; ++rl) {
+        const int pr = (unit * RL + rl) * 4 + d;  // row index in the padded (EPB rows per packed row) space
+        const int g = pr / EPB, k = pr % EPB;
+        gp[rl] = g;
+        valid[rl] = false;
+        row[rl] = 0;
+        if (g < n_packed) {
+            const int p = P == 1 ? 0 : find_segment(pseg, P, g);
+            row[rl] = (int64_t)seg[p] + (int64_t)(g - pseg[p]) * EPB + k;
+            valid[rl] = row[rl] < seg[p + 1];
+        }
+    }
+    int off[NV];
+    bool act[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        off[v] = (v * 16 + l16) * VEC;
+        act[v] = off[v] < F;
+    }
+    float xv[RL][NV][VEC];
+#pragma unroll
+    for (int rl = 0; rl < RL; ++rl) {
+        if (!valid[rl]) continue;
+        const float *xr = x + row[rl] * F;
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+            if (act[v]) vec_load_nt<VEC>(xv[rl][v], xr + off[v]);
+    }
+
+    float zp[RL], sc[RL], rinv[RL];
+    bool lane_exact = kForceExactDivision;
+#pragma unroll
+    for (int rl = 0; rl < RL; ++rl) {
+        zp[rl] = 0.0f;
+        sc[rl] = 1.0f;
+        rinv[rl] = 1.0f;
+        if (!valid[rl]) continue;  // uniform within a DPP row: the row-level DPP steps below see full rows
+        float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            if (!act[v]) continue;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                mn = fminf(mn, xv[rl][v][k]);
+                mx = fmaxf(mx, xv[rl][v][k]);
+            }
+        }
+        mn = group_allreduce_f<16, OpMinF>(mn);
+        mx = group_allreduce_f<16, OpMaxF>(mx);
+        if (mn == 0.0f || mx == 0.0f) {
+            // first-occurrence rule for compare-equal zeros (quantization_arm.cpp:98-101)
+            int key = INT_MAX;
+#pragma unroll
+            for (int v = NV - 1; v >= 0; --v) {
+                if (!act[v]) continue;
+#pragma unroll
+                for (int k = VEC - 1; k >= 0; --k)
+                    if (xv[rl][v][k] == 0.0f) key = ((off[v] + k) << 1) | (int)(__float_as_uint(xv[rl][v][k]) >> 31);
+            }
+            key = group_allmin_i<16>(key);
+            const float z = (key & 1) ? -0.0f : 0.0f;
+            if (mn == 0.0f) mn = z;
+            if (mx == 0.0f) mx = z;
+        }
+        // a NaN is sticky only as element 0, which lane 0 of the DPP row holds
+        const unsigned long long nanmask = __ballot(l16 == 0 && xv[rl][0][0] != xv[rl][0][0]);
+        if ((nanmask >> (lane & 48)) & 1ull) {
+            mn = __int_as_float(0x7fc00000);
+            mx = mn;
+        }
+        float s = (mx - mn) / (float)((1 << BITS) - 1);
+        if (s == 0.0f) s = 1.0f;
+        zp[rl] = mn;
+        sc[rl] = s;
+        rinv[rl] = 1.0f / s;
+        if (!(s >= 0x1p-100f && s <= 0x1p100f)) lane_exact = true;
+        if (l16 == 0) *reinterpret_cast<float2 *>(params + row[rl] * 2) = make_float2(mn, s);
+    }
+
+    // Codes: (x - zp) * RN(1/scale), accepted when provably equal to the IEEE quotient after
+    // rounding; otherwise this lane redoes its elements with the IEEE division.
+    const int shift = (EPB - 1 - (d % EPB)) * BITS;
+    uint32_t words[RL][NV];
+#pragma unroll
+    for (int rl = 0; rl < RL; ++rl) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            uint32_t word = 0;
+            if (valid[rl] && act[v]) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float qf = (xv[rl][v][e] - zp[rl]) * rinv[rl];
+                    const float ri = rintf(qf);
+                    if (!(fabsf(qf - ri) < 0.5f - 0x1p-14f)) lane_exact = true;
+                    word |= (uint32_t)ri << (8 * e);
+                }
+            }
+            words[rl][v] = word;
+        }
+    }
+    if (lane_exact) {
+#pragma unroll
+        for (int rl = 0; rl < RL; ++rl) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                uint32_t word = 0;
+                if (valid[rl] && act[v]) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) word |= quant_code(xv[rl][v][e], zp[rl], sc[rl]) << (8 * e);
+                }
+                words[rl][v] = word;
+            }
+        }
+    }
+    // Pack: shift to the row's bit position, OR across the DPP rows that share a packed row, store.
+#pragma unroll
+    for (int rl = 0; rl < RL; ++rl) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            uint32_t w = words[rl][v] << shift;
+            if constexpr (EPB >= 2) w |= (uint32_t)__shfl_xor((int)w, 16, 64);
+            if constexpr (EPB == 4) w |= (uint32_t)__shfl_xor((int)w, 32, 64);
+            const bool mine = EPB == 1 ? true : EPB == 2 ? ((d & 1) == (v & 1)) : (d == (v & 3));
+            if (mine && act[v] && gp[rl] < n_packed)
+                __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(q + (int64_t)gp[rl] * F + off[v]));
         }
     }
 }
@@ -423,6 +629,8 @@ struct RowsArgs {
     const float *x_in; uint8_t *q_out; float *params_out;            // quantize
     const uint8_t *q_in; float *x_out; const float *params_in;        // dequantize
     const int32_t *seg; const int32_t *pseg; int P; int n_packed; int F; bool quantize;
+    bool layout16;        // diagnostic switch: one fp32 row per 16 lanes (default) vs per lane group
+    bool exact_division;  // diagnostic: IEEE division for every element (the results are identical either way)
 };
 
 template <int BITS, int VEC, int G, int NV>
@@ -432,12 +640,31 @@ static void launch_rows(const RowsArgs &a, hipStream_t st) {
     const int n_units = (a.n_packed + NPR - 1) / NPR;
     const int nb = (n_units + GPB - 1) / GPB;
     ProfScope prof(a.quantize ? K_QUANT_PACK_ROWS : K_UNPACK_DEQUANT_ROWS, st);
-    if (a.quantize)
-        hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
-                           a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+    if (a.quantize && a.exact_division)
+        hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
+                           a.q_out, a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+    else if (a.quantize)
+        hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV, false>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
+                           a.q_out, a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
     else
         hipLaunchKernelGGL((unpack_dequant_rows_kernel<BITS, VEC, G, NV>), dim3(nb), dim3(kQBlock), 0, st, a.q_in,
                            a.x_out, a.params_in, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+}
+
+template <int BITS, int NV>
+static void launch_quant16(const RowsArgs &a, hipStream_t st) {
+    constexpr int RL = NV >= 4 ? 1 : 4 / NV;
+    constexpr int EPB = 8 / BITS;
+    const int64_t padded = (int64_t)a.n_packed * EPB;
+    const int n_units = (int)((padded + 4 * RL - 1) / (4 * RL));
+    const int nb = (n_units + kQBlock / 64 - 1) / (kQBlock / 64);
+    ProfScope prof(K_QUANT_PACK_ROWS, st);
+    if (a.exact_division)
+        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
+                           a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+    else
+        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
+                           a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
 }
 
 template <int BITS>
@@ -454,6 +681,15 @@ static void launch_rows_wide(const RowsArgs &a, hipStream_t st) {
 
 template <int BITS, int VEC>
 static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
+    if constexpr (VEC == 4) {
+        if (a.quantize && a.layout16) {
+            if (nvec <= 16) return launch_quant16<BITS, 1>(a, st);
+            if (nvec <= 32) return launch_quant16<BITS, 2>(a, st);
+            if (nvec <= 64) return launch_quant16<BITS, 4>(a, st);
+            if (nvec <= 128) return launch_quant16<BITS, 8>(a, st);
+            if (nvec <= 256) return launch_quant16<BITS, 16>(a, st);
+        }
+    }
     if (nvec <= 16) return launch_rows<BITS, VEC, 16, 1>(a, st);
     if (nvec <= 32) return launch_rows<BITS, VEC, 32, 1>(a, st);
     if (nvec <= 64) return launch_rows<BITS, VEC, 64, 1>(a, st);
@@ -525,6 +761,8 @@ extern "C" int sgnn_quant_pack_rows_f32(const float *x, uint8_t *q, float *param
     RowsArgs a{};
     a.x_in = x; a.q_out = q; a.params_out = params; a.seg = seg; a.pseg = pseg; a.P = P;
     a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = true;
+    { const char *e = getenv("SGNN_QUANT_EXACT_DIV"); a.exact_division = e && e[0] == '1'; }
+    { const char *e = getenv("SGNN_QUANT_LAYOUT16"); a.layout16 = !(e && e[0] == '0'); }
     return run_rows(a, bits, n_rows, x, q, (hipStream_t)stream);
 }
 

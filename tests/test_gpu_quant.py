@@ -227,3 +227,45 @@ def test_full_size_properties(bits):
         q_ref, p_ref = orc.quant_rows(xs, [0, 4096], bits)
         assert np.array_equal(q[s // epb:(s + 4096) // epb].cpu().numpy(), q_ref)
         assert np.array_equal(p[s:s + 4096].cpu().numpy().view(np.uint32), p_ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+def test_fast_quotient_equals_ieee_division(bits):
+    """The kernel forms (x-zp)*RN(1/scale) and falls back to the IEEE division near half-integers;
+    its bytes must equal those of the all-IEEE variant (SGNN_QUANT_EXACT_DIV=1) on the full-size
+    input and on rows built to sit on rounding ties."""
+    import os
+    from super_gnn_amd import synth
+    ops = _ops()
+    qmax = (1 << bits) - 1
+    g = torch.Generator(device="cuda"); g.manual_seed(bits)
+    n, F = 1_000_000, 256
+    x = synth.boundary_features(n, F, seed=5, device="cuda")
+    # adversarial block: min 0, max qmax*s, values at (k + 0.5 +- tiny) * s for assorted scales s
+    na = 4096
+    s = torch.rand(na, 1, generator=g, device="cuda") * 3 + 0.01
+    k = torch.randint(0, qmax, (na, F), generator=g, device="cuda").float()
+    eps = (torch.randint(-3, 4, (na, F), generator=g, device="cuda").float()) * 2.0 ** -22
+    adv = (k + 0.5) * (1 + eps) * s
+    adv[:, 0] = 0.0
+    adv[:, 1] = qmax * s[:, 0]
+    x[:na] = adv
+    # rows with extreme scales: reciprocal not a normal number -> whole-row fallback
+    x[na] = torch.linspace(0, 1e-38, F, device="cuda")
+    x[na + 1] = torch.linspace(-3e38, 3e38, F, device="cuda")
+    epb = 8 // bits
+    seg = torch.tensor([0, n], dtype=torch.int32)
+    outs = []
+    for exact in ("0", "1"):
+        os.environ["SGNN_QUANT_EXACT_DIV"] = exact
+        q = torch.empty((n + epb - 1) // epb, F, dtype=torch.uint8, device="cuda")
+        p = torch.empty(n, 2, device="cuda")
+        ops.quantize_tensor_for_all_procs(x, q, p, seg, 1, bits)
+        torch.cuda.synchronize()
+        outs.append((q, p))
+    os.environ.pop("SGNN_QUANT_EXACT_DIV")
+    assert torch.equal(outs[0][0], outs[1][0])
+    assert torch.equal(outs[0][1].view(torch.int32), outs[1][1].view(torch.int32))
+    xs = x[: na + 8].cpu().numpy()
+    q_ref, p_ref = orc.quant_rows(xs, [0, na + 8], bits)
+    assert np.array_equal(outs[0][0][: (na + 8) // epb].cpu().numpy(), q_ref)
