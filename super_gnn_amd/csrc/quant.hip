@@ -484,6 +484,66 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
+// Unpack + dequantize, one fp32 row per 16 lanes (float4 lanes, F <= 1024): the mirror image of
+// quant_pack_rows16_kernel.  Every lane reads the packed words of its own row's packed row (the DPP
+// rows that share a packed row read the same words), extracts its row's code and writes its row.
+// ------------------------------------------------------------------------------------------------
+template <int BITS, int NV, int RL>
+__global__ __launch_bounds__(kQBlock) void unpack_dequant_rows16_kernel(
+    const uint8_t *__restrict__ q, float *__restrict__ x, const float *__restrict__ params,
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
+    constexpr int EPB = 8 / BITS;
+    constexpr int VEC = 4;
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    const int lane = threadIdx.x & 63, d = lane >> 4, l16 = lane & 15;
+    const int unit = blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
+    if (unit >= n_units) return;
+    const int shift = (EPB - 1 - (d % EPB)) * BITS;
+
+    int64_t row[RL];
+    bool valid[RL];
+    uint32_t words[RL][NV];
+    float2 ps[RL];
+#pragma unroll
+    for (int rl = 0; rl < RL; ++rl) {
+        const int pr = (unit * RL + rl) * 4 + d;
+        const int g = pr / EPB, k = pr % EPB;
+        valid[rl] = false;
+        row[rl] = 0;
+        ps[rl] = make_float2(0.0f, 0.0f);
+        if (g < n_packed) {
+            const int p = P == 1 ? 0 : find_segment(pseg, P, g);
+            row[rl] = (int64_t)seg[p] + (int64_t)(g - pseg[p]) * EPB + k;
+            valid[rl] = row[rl] < seg[p + 1];
+        }
+        if (valid[rl]) {
+            ps[rl] = *reinterpret_cast<const float2 *>(params + row[rl] * 2);
+            const uint8_t *qr = q + (int64_t)g * F;
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                const int off = (v * 16 + l16) * VEC;
+                if (off < F) words[rl][v] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(qr + off));
+            }
+        }
+    }
+#pragma unroll
+    for (int rl = 0; rl < RL; ++rl) {
+        if (!valid[rl]) continue;
+        float *xr = x + row[rl] * F;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int off = (v * 16 + l16) * VEC;
+            if (off >= F) continue;
+            float o[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                o[e] = fmaf((float)((words[rl][v] >> (8 * e + shift)) & MASK), ps[rl].y, ps[rl].x);
+            vec_store_nt<VEC>(xr + off, o);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Any-F fallbacks (F wider than a register tile): one wavefront per packed row, two passes.
 // ------------------------------------------------------------------------------------------------
 template <int BITS>
@@ -667,6 +727,18 @@ static void launch_quant16(const RowsArgs &a, hipStream_t st) {
                            a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
 }
 
+template <int BITS, int NV>
+static void launch_dequant16(const RowsArgs &a, hipStream_t st) {
+    constexpr int RL = NV >= 4 ? 1 : 4 / NV;
+    constexpr int EPB = 8 / BITS;
+    const int64_t padded = (int64_t)a.n_packed * EPB;
+    const int n_units = (int)((padded + 4 * RL - 1) / (4 * RL));
+    const int nb = (n_units + kQBlock / 64 - 1) / (kQBlock / 64);
+    ProfScope prof(K_UNPACK_DEQUANT_ROWS, st);
+    hipLaunchKernelGGL((unpack_dequant_rows16_kernel<BITS, NV, RL>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, a.x_out,
+                       a.params_in, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+}
+
 template <int BITS>
 static void launch_rows_wide(const RowsArgs &a, hipStream_t st) {
     const int nb = (a.n_packed + kQBlock / 64 - 1) / (kQBlock / 64);
@@ -688,6 +760,15 @@ static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
             if (nvec <= 64) return launch_quant16<BITS, 4>(a, st);
             if (nvec <= 128) return launch_quant16<BITS, 8>(a, st);
             if (nvec <= 256) return launch_quant16<BITS, 16>(a, st);
+        }
+        // Measured on MI355X: at int2 one packed word feeds four fp32 rows and the group-per-packed-row
+        // kernel (one load, four whole-row stores) wins; at int4 / int8 the row-per-16-lanes kernel does.
+        if (!a.quantize && a.layout16 && BITS != 2) {
+            if (nvec <= 16) return launch_dequant16<BITS, 1>(a, st);
+            if (nvec <= 32) return launch_dequant16<BITS, 2>(a, st);
+            if (nvec <= 64) return launch_dequant16<BITS, 4>(a, st);
+            if (nvec <= 128) return launch_dequant16<BITS, 8>(a, st);
+            if (nvec <= 256) return launch_dequant16<BITS, 16>(a, st);
         }
     }
     if (nvec <= 16) return launch_rows<BITS, VEC, 16, 1>(a, st);
@@ -773,6 +854,7 @@ extern "C" int sgnn_unpack_dequant_rows_f32(const uint8_t *q, float *x, const fl
     RowsArgs a{};
     a.q_in = q; a.x_out = x; a.params_in = params; a.seg = seg; a.pseg = pseg; a.P = P;
     a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = false;
+    { const char *e = getenv("SGNN_QUANT_LAYOUT16"); a.layout16 = !(e && e[0] == '0'); }
     return run_rows(a, bits, n_rows, x, q, (hipStream_t)stream);
 }
 
