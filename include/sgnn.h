@@ -122,6 +122,29 @@ int sgnn_unpack_dequant_rows_f32(const uint8_t *q, float *x, const float *params
                                  int64_t n_packed_rows, int64_t F, int bits, sgnn_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Fused unpack + dequantize + SpMM (pre/post-aggregation mode)
+ * ------------------------------------------------------------------------------------------- */
+
+/* row_slot[r] = pseg[p] * EPB + (r - seg[p]) for the segment p that holds row r: the position of
+ * row r in the padded row space of the packed buffer (packed row = slot / EPB, position inside the
+ * byte = slot % EPB).  seg, pseg, row_slot are device arrays.  When every segment but the last
+ * holds a multiple of EPB rows the table is the identity and callers may pass NULL instead. */
+int sgnn_quant_row_slots(const int32_t *seg, const int32_t *pseg, int P, int bits, int64_t n_rows,
+                         int32_t *row_slot, sgnn_stream_t stream);
+
+/* out[M,F] (+)= A[M,K] * dequant(q)[K,F]: the dense operand is handed over as it arrives from the
+ * boundary exchange -- packed codes q u8[n_packed,F] in the row-group layout plus params f32[K,2] --
+ * and is decoded inside the gather, value = fma(code, scale, zero_point), then one fma per edge.
+ * Replaces the pair "dequantize into recv_buf, then SPMM_forward(remote graph, recv_buf, out)" of
+ * super_gnn/aggregator.py:72-93 (forward) and :159-171 (backward); no fp32 recv_buf is written or
+ * re-read.  The result is bit-identical to running sgnn_unpack_dequant_rows_f32 followed by
+ * sgnn_spmm_csr_f32 with the same plan.  F % 4 == 0 required; other arguments as in
+ * sgnn_spmm_csr_f32.  row_slot: see sgnn_quant_row_slots (NULL = identity). */
+int sgnn_spmm_csr_dq_f32(sgnn_spmm_plan *plan, const float *val, const uint8_t *q, const float *params,
+                         const int32_t *row_slot, int bits, float *out, int64_t F, int64_t ldo,
+                         int accumulate, const float *row_div, sgnn_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Feature-packed mixed-bit quantization ("v1")
  * ------------------------------------------------------------------------------------------- */
 

@@ -41,7 +41,7 @@ enum KernelId {
     K_DEQUANT_V1,
     K_STREAM_COPY,
     K_FUSED_SHORT,
-    K_FUSED_SEGMENT,
+    K_FUSED_PIECE,
     K_SPMM_EMPTY_ROWS,
     K_COUNT
 };

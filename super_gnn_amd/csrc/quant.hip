@@ -682,6 +682,22 @@ __global__ __launch_bounds__(kQBlock) void dequant_v1_kernel(const uint8_t *__re
     }
 }
 
+// Position of every row in the padded row space (EPB rows per packed row, every segment starting
+// on a packed-row boundary): slot[r] = pseg[p] * EPB + (r - seg[p]) for the segment p holding r.
+// Packed row = slot / EPB, position inside the byte = slot % EPB.
+__global__ __launch_bounds__(kQBlock) void row_slots_kernel(const int32_t *__restrict__ seg,
+                                                            const int32_t *__restrict__ pseg, int P, int epb,
+                                                            int64_t n_rows, int32_t *__restrict__ slot) {
+    const int64_t r = (int64_t)blockIdx.x * kQBlock + threadIdx.x;
+    if (r >= n_rows) return;
+    int lo = 0, hi = P - 1;  // the p with seg[p] <= r < seg[p+1]
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (seg[mid + 1] > r) hi = mid; else lo = mid + 1;
+    }
+    slot[r] = pseg[lo] * epb + (int32_t)(r - seg[lo]);
+}
+
 // ------------------------------------------------------------------------------------------------
 // Launch tables.
 // ------------------------------------------------------------------------------------------------
@@ -833,6 +849,19 @@ extern "C" int64_t sgnn_quant_segment_offsets(const int32_t *seg_host, int P, in
         pseg_host[p + 1] = (int32_t)acc;
     }
     return acc;
+}
+
+extern "C" int sgnn_quant_row_slots(const int32_t *seg, const int32_t *pseg, int P, int bits, int64_t n_rows,
+                                    int32_t *row_slot, sgnn_stream_t stream) {
+    SGNN_REQUIRE(bits == 8 || bits == 4 || bits == 2, "bits=%d, expected 8, 4 or 2", bits);
+    SGNN_REQUIRE(P >= 1 && n_rows >= 0 && n_rows < INT32_MAX / 4, "bad segment table size");
+    if (n_rows == 0) return SGNN_OK;
+    SGNN_REQUIRE(seg && pseg && row_slot, "null pointer argument");
+    const int64_t nb = (n_rows + kQBlock - 1) / kQBlock;
+    hipLaunchKernelGGL(row_slots_kernel, dim3((uint32_t)nb), dim3(kQBlock), 0, (hipStream_t)stream, seg, pseg, P, 8 / bits,
+                       n_rows, row_slot);
+    SGNN_HIP_CHECK(hipGetLastError());
+    return SGNN_OK;
 }
 
 extern "C" int sgnn_quant_pack_rows_f32(const float *x, uint8_t *q, float *params, const int32_t *seg,

@@ -53,13 +53,82 @@ __device__ __forceinline__ int64_t uniform64(int64_t v) {
     return (int64_t)(((uint64_t)hi << 32) | lo);
 }
 
+// The dense operand of the product: fp32 rows (BITS == 0), or rows that arrive quantized and
+// bit-packed in the row-group layout (BITS in {8, 4, 2}; see quant.hip) and are decoded on the fly.
+struct DenseSrc {
+    const float *x;        // fp32: [K, ldx]
+    int64_t ldx;
+    const uint8_t *q;      // quantized: packed rows of qF bytes
+    const float *params;   // quantized: (zero_point, scale) per dense row
+    const int32_t *slot;   // quantized: dense row -> index in the padded row space (null = identity)
+    int qF;
+};
+
+// What one gather of one dense row leaves in a lane's registers: the fp32 values themselves, or
+// the packed words plus the row's decode parameters (decoded only when consumed, so that the U
+// loads of a batch are all in flight before the first conversion).
+template <int VEC, int NV, int BITS>
+struct Fetched {
+    float f[BITS == 0 ? NV : 1][BITS == 0 ? VEC : 1];
+    uint32_t w[BITS == 0 ? 1 : NV];
+    float zp, sc;
+    int shift;
+};
+
+template <int VEC, int NV, int BITS>
+__device__ __forceinline__ void fetch_row(Fetched<VEC, NV, BITS> &r, const DenseSrc &d, int c, const int (&off)[NV],
+                                          const bool (&act)[NV]) {
+    if constexpr (BITS == 0) {
+        const float *xr = d.x + (int64_t)c * d.ldx;
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+            if (act[v]) vec_load<VEC>(r.f[v], xr + off[v]);
+    } else {
+        constexpr int EPB = 8 / BITS;
+        const int sl = d.slot ? d.slot[c] : c;
+        const float2 ps = *reinterpret_cast<const float2 *>(d.params + (int64_t)c * 2);
+        r.zp = ps.x;
+        r.sc = ps.y;
+        r.shift = (EPB - 1 - (sl % EPB)) * BITS;
+        const uint8_t *qr = d.q + (int64_t)(sl / EPB) * d.qF;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            if (!act[v]) continue;
+            if constexpr (VEC == 4) r.w[v] = *reinterpret_cast<const uint32_t *>(qr + off[v]);
+            else if constexpr (VEC == 2) r.w[v] = *reinterpret_cast<const uint16_t *>(qr + off[v]);
+            else r.w[v] = qr[off[v]];
+        }
+    }
+}
+
+// acc += w * row, one fma per element.  A quantized row is first decoded exactly as the stand-alone
+// unpack+dequantize kernel does, fma(code, scale, zero_point), so the fused product equals
+// "dequantize, then multiply" bit for bit.
+template <int VEC, int NV, int BITS>
+__device__ __forceinline__ void fma_row(float (&acc)[NV][VEC], float w, const Fetched<VEC, NV, BITS> &r) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            float xv;
+            if constexpr (BITS == 0) {
+                xv = r.f[v][k];
+            } else {
+                const uint32_t code = (r.w[v] >> (8 * k + r.shift)) & ((1u << BITS) - 1u);
+                xv = fmaf((float)code, r.sc, r.zp);
+            }
+            acc[v][k] = fmaf(w, xv, acc[v][k]);
+        }
+    }
+}
+
 // Accumulate the `deg` edges listed at colp into acc for one feature tile.  The weight of edge i is
 // val[eperm[i]] (val may be null = all ones).
-template <int VEC, int G, int NV>
+template <int VEC, int G, int NV, int BITS>
 __device__ __forceinline__ void gather_piece(float (&acc)[NV][VEC], const int32_t *__restrict__ colp,
                                              const int32_t *__restrict__ eperm, const float *__restrict__ val,
-                                             int deg, const float *__restrict__ x, int64_t ldx,
-                                             const int (&off)[NV], const bool (&act)[NV], int lig) {
+                                             int deg, const DenseSrc &dense, const int (&off)[NV],
+                                             const bool (&act)[NV], int lig) {
     constexpr int U = unroll_of(NV);
     // (col,val) pairs are fetched G at a time, one chunk ahead of the gathers that consume them.
     int nc = 0;
@@ -78,27 +147,17 @@ __device__ __forceinline__ void gather_piece(float (&acc)[NV][VEC], const int32_
         }
         const int cnt = deg - base < G ? deg - base : G;
         for (int j = 0; j < cnt; j += U) {
-            float xv[U][NV][VEC];
+            Fetched<VEC, NV, BITS> xv[U];
             // U gathers back to back; past the end the last edge's row is fetched again (a cache
             // hit) so that no branch separates the loads.
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int src = j + u < cnt ? j + u : cnt - 1;
-                const int c = group_bcast_i<G>(myc, src);
-                const float *xr = x + (int64_t)c * ldx;
-#pragma unroll
-                for (int v = 0; v < NV; ++v)
-                    if (act[v]) vec_load<VEC>(xv[u][v], xr + off[v]);
+                fetch_row<VEC, NV, BITS>(xv[u], dense, group_bcast_i<G>(myc, src), off, act);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (j + u < cnt) {
-                    const float w = group_bcast_f<G>(myw, j + u);
-#pragma unroll
-                    for (int v = 0; v < NV; ++v)
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k) acc[v][k] = fmaf(w, xv[u][v][k], acc[v][k]);
-                }
+                if (j + u < cnt) fma_row<VEC, NV, BITS>(acc, group_bcast_f<G>(myw, j + u), xv[u]);
             }
         }
     }
@@ -121,11 +180,11 @@ __device__ __forceinline__ uint32_t group_ballot(bool pred) {
 // Rows per chunk: each of the first nr+1 lanes of the group holds one rowptr entry.
 __host__ __device__ constexpr int chunk_row_limit(int G) { return (G < 32 ? G : 32) - 1; }
 
-template <int VEC, int G, int NV>
+template <int VEC, int G, int NV, int BITS>
 __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
     const int64_t *__restrict__ rowptr, const int32_t *__restrict__ col, const float *__restrict__ val,
-    const float *__restrict__ x, float *__restrict__ out, const int2 *__restrict__ chunks, int n_chunks, int F,
-    int64_t ldx, int64_t ldo, int accumulate, const float *__restrict__ row_div, uint32_t nblocks) {
+    const DenseSrc dense, float *__restrict__ out, const int2 *__restrict__ chunks, int n_chunks, int F,
+    int64_t ldo, int accumulate, const float *__restrict__ row_div, uint32_t nblocks) {
     constexpr int GPB = kBlock / G;
     constexpr int TILE = G * VEC * NV;
     constexpr int U = unroll_of(NV);
@@ -197,17 +256,13 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
             }
             const int cnt = E - base < G ? E - base : G;
             for (int j = 0; j < cnt; j += U) {
-                float xv[U][NV][VEC];
+                Fetched<VEC, NV, BITS> xv[U];
                 // U gathers back to back.  Past the end of the chunk the last edge's row is
                 // fetched again (a cache hit) so that no branch separates the loads.
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const int src = j + u < cnt ? j + u : cnt - 1;
-                    const int c = group_bcast_i<G>(myc, src);
-                    const float *xr = x + (int64_t)c * ldx;
-#pragma unroll
-                    for (int v = 0; v < NV; ++v)
-                        if (act[v]) vec_load<VEC>(xv[u][v], xr + off[v]);
+                    fetch_row<VEC, NV, BITS>(xv[u], dense, group_bcast_i<G>(myc, src), off, act);
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -236,11 +291,7 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
                                     if (act[v]) vec_load_nt<VEC>(nxt_old[v], out + (int64_t)(rb + nxt) * ldo + off[v]);
                             }
                         }
-                        const float w = group_bcast_f<G>(myw, j + u);
-#pragma unroll
-                        for (int v = 0; v < NV; ++v)
-#pragma unroll
-                            for (int k = 0; k < VEC; ++k) acc[v][k] = fmaf(w, xv[u][v][k], acc[v][k]);
+                        fma_row<VEC, NV, BITS>(acc, group_bcast_f<G>(myw, j + u), xv[u]);
                     }
                 }
             }
@@ -297,12 +348,12 @@ __global__ __launch_bounds__(kBlock) void spmm_empty_rows_kernel(const int32_t *
 // rows of its own class and the eight 4 MB L2s hold eight DISJOINT sets of popular rows instead of
 // eight copies of the same set.
 // ------------------------------------------------------------------------------------------------
-template <int VEC, int G, int NV>
+template <int VEC, int G, int NV, int BITS>
 __global__ __launch_bounds__(kBlock) void spmm_piece_kernel(
     const int32_t *__restrict__ col_long, const int32_t *__restrict__ eperm, const float *__restrict__ val,
-    const float *__restrict__ x, float *__restrict__ partial, const int32_t *__restrict__ item_begin,
+    const DenseSrc dense, float *__restrict__ partial, const int32_t *__restrict__ item_begin,
     const int32_t *__restrict__ item_len, const int32_t *__restrict__ cls_list, const int32_t *__restrict__ cls_off,
-    int F, int64_t ldx) {
+    int F) {
     constexpr int GPB = kBlock / G;
     constexpr int TILE = G * VEC * NV;
     const int gid = threadIdx.x / G, lig = threadIdx.x % G;
@@ -327,7 +378,7 @@ __global__ __launch_bounds__(kBlock) void spmm_piece_kernel(
 #pragma unroll
             for (int k = 0; k < VEC; ++k) acc[v][k] = 0.0f;
         }
-        gather_piece<VEC, G, NV>(acc, col_long + b, eperm + b, val, len, x, ldx, off, act, lig);
+        gather_piece<VEC, G, NV, BITS>(acc, col_long + b, eperm + b, val, len, dense, off, act, lig);
 #pragma unroll
         for (int v = 0; v < NV; ++v)
             if (act[v]) vec_store<VEC>(partial + (int64_t)item * F + off[v], acc[v]);
@@ -470,28 +521,28 @@ __global__ __launch_bounds__(kBlock) void narrow_cols_kernel(const SrcT *__restr
 // Launch tables.
 // ------------------------------------------------------------------------------------------------
 struct ShortArgs {
-    const int64_t *rowptr; const int32_t *col; const float *val; const float *x; float *out;
+    const int64_t *rowptr; const int32_t *col; const float *val; DenseSrc dense; float *out;
     const int2 *chunks; int n_chunks; const int32_t *empty_rows; int n_empty;
-    int F; int64_t ldx, ldo; int accumulate; const float *row_div;
+    int F; int64_t ldo; int accumulate; const float *row_div;
 };
 struct PieceArgs {
-    const int32_t *col_long; const int32_t *eperm; const float *val; const float *x; float *partial;
+    const int32_t *col_long; const int32_t *eperm; const float *val; float *partial;
     const int32_t *item_begin; const int32_t *item_len; const int32_t *cls_list; const int32_t *cls_off;
-    int max_cls_items; int F; int64_t ldx;
+    int max_cls_items; int F;
 };
 struct FinalArgs {
     const int32_t *long_rows; const int32_t *long_pbeg; const float *partial; float *out; int n_long;
     int F; int64_t ldo; int accumulate; const float *row_div;
 };
 
-template <int VEC, int G, int NV>
+template <int VEC, int G, int NV, int BITS>
 static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &f, hipStream_t st) {
     constexpr int GPB = kBlock / G;
     if (a.n_chunks > 0) {
         const uint32_t nb = (uint32_t)((a.n_chunks + GPB - 1) / GPB);
-        ProfScope prof(K_SPMM_SHORT, st);
-        hipLaunchKernelGGL((spmm_short_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, a.rowptr, a.col, a.val, a.x,
-                           a.out, a.chunks, a.n_chunks, a.F, a.ldx, a.ldo, a.accumulate, a.row_div, nb);
+        ProfScope prof(BITS == 0 ? K_SPMM_SHORT : K_FUSED_SHORT, st);
+        hipLaunchKernelGGL((spmm_short_kernel<VEC, G, NV, BITS>), dim3(nb), dim3(kBlock), 0, st, a.rowptr, a.col, a.val,
+                           a.dense, a.out, a.chunks, a.n_chunks, a.F, a.ldo, a.accumulate, a.row_div, nb);
     }
     if (a.n_empty > 0 && (!a.accumulate || a.row_div)) {
         const uint32_t nb = (uint32_t)((a.n_empty + GPB - 1) / GPB);
@@ -503,9 +554,9 @@ static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &
         {
             // workgroup i serves class i % 8: grid = 8 * (workgroups of the fullest class)
             const uint32_t nb = (uint32_t)kNumXCD * (uint32_t)((s.max_cls_items + GPB - 1) / GPB);
-            ProfScope prof(K_SPMM_PIECE, st);
-            hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, s.col_long, s.eperm,
-                               s.val, s.x, s.partial, s.item_begin, s.item_len, s.cls_list, s.cls_off, s.F, s.ldx);
+            ProfScope prof(BITS == 0 ? K_SPMM_PIECE : K_FUSED_PIECE, st);
+            hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS>), dim3(nb), dim3(kBlock), 0, st, s.col_long, s.eperm,
+                               s.val, a.dense, s.partial, s.item_begin, s.item_len, s.cls_list, s.cls_off, s.F);
         }
         const uint32_t nb = (uint32_t)((f.n_long + GPB - 1) / GPB);
         ProfScope prof(K_SPMM_LONG_FINAL, st);
@@ -519,16 +570,29 @@ static int group_width(int nvec) { return nvec <= 8 ? 8 : nvec <= 16 ? 16 : nvec
 
 template <int VEC>
 static int dispatch_shape(int nvec, const ShortArgs &a, const PieceArgs &s, const FinalArgs &f, hipStream_t st) {
-    if (nvec <= 8) launch_all<VEC, 8, 1>(a, s, f, st);
-    else if (nvec <= 16) launch_all<VEC, 16, 1>(a, s, f, st);
-    else if (nvec <= 32) launch_all<VEC, 32, 1>(a, s, f, st);
-    else if (nvec <= 64) launch_all<VEC, 64, 1>(a, s, f, st);
-    else if (nvec <= 128) launch_all<VEC, 64, 2>(a, s, f, st);
-    else if (nvec <= 192) launch_all<VEC, 64, 3>(a, s, f, st);
-    else if (nvec <= 256) launch_all<VEC, 64, 4>(a, s, f, st);
-    else if (nvec <= 320) launch_all<VEC, 64, 5>(a, s, f, st);
-    else if (nvec <= 384) launch_all<VEC, 64, 6>(a, s, f, st);
-    else launch_all<VEC, 64, 8>(a, s, f, st);  // feature axis walked in tiles of 512 vectors
+    if (nvec <= 8) launch_all<VEC, 8, 1, 0>(a, s, f, st);
+    else if (nvec <= 16) launch_all<VEC, 16, 1, 0>(a, s, f, st);
+    else if (nvec <= 32) launch_all<VEC, 32, 1, 0>(a, s, f, st);
+    else if (nvec <= 64) launch_all<VEC, 64, 1, 0>(a, s, f, st);
+    else if (nvec <= 128) launch_all<VEC, 64, 2, 0>(a, s, f, st);
+    else if (nvec <= 192) launch_all<VEC, 64, 3, 0>(a, s, f, st);
+    else if (nvec <= 256) launch_all<VEC, 64, 4, 0>(a, s, f, st);
+    else if (nvec <= 320) launch_all<VEC, 64, 5, 0>(a, s, f, st);
+    else if (nvec <= 384) launch_all<VEC, 64, 6, 0>(a, s, f, st);
+    else launch_all<VEC, 64, 8, 0>(a, s, f, st);  // feature axis walked in tiles of 512 vectors
+    return SGNN_OK;
+}
+
+// Quantized dense operand: float4-wide lanes only (F % 4 == 0), one packed word per lane and vector.
+template <int BITS>
+static int dispatch_shape_dq(int nvec, const ShortArgs &a, const PieceArgs &s, const FinalArgs &f, hipStream_t st) {
+    if (nvec <= 8) launch_all<4, 8, 1, BITS>(a, s, f, st);
+    else if (nvec <= 16) launch_all<4, 16, 1, BITS>(a, s, f, st);
+    else if (nvec <= 32) launch_all<4, 32, 1, BITS>(a, s, f, st);
+    else if (nvec <= 64) launch_all<4, 64, 1, BITS>(a, s, f, st);
+    else if (nvec <= 128) launch_all<4, 64, 2, BITS>(a, s, f, st);
+    else if (nvec <= 256) launch_all<4, 64, 4, BITS>(a, s, f, st);
+    else launch_all<4, 64, 8, BITS>(a, s, f, st);
     return SGNN_OK;
 }
 
@@ -777,16 +841,13 @@ extern "C" int sgnn_spmm_reference_overwrites(int64_t nnz, int64_t M, int64_t K,
     return (sparsity <= 0.0001f && F > 256) ? 1 : 0;
 }
 
-extern "C" int sgnn_spmm_csr_f32(sgnn_spmm_plan *p, const float *val, const float *x, float *out, int64_t F,
-                                 int64_t ldx, int64_t ldo, int accumulate, const float *row_div,
-                                 sgnn_stream_t stream) {
+static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, int bits, float *out, int64_t F,
+                    int64_t ldo, int accumulate, const float *row_div, hipStream_t st) {
     SGNN_REQUIRE(p != nullptr, "plan is null");
     SGNN_REQUIRE(F > 0 && F < (1 << 24), "feature width F=%lld out of range", (long long)F);
-    SGNN_REQUIRE(ldx >= F && ldo >= F, "leading dimension smaller than F (ldx=%lld ldo=%lld F=%lld)", (long long)ldx, (long long)ldo, (long long)F);
+    SGNN_REQUIRE(ldo >= F, "leading dimension smaller than F (ldo=%lld F=%lld)", (long long)ldo, (long long)F);
     if (p->M == 0) return SGNN_OK;
     SGNN_REQUIRE(out != nullptr, "out is null");
-    SGNN_REQUIRE(x != nullptr || p->nnz == 0, "x is null");
-    hipStream_t st = (hipStream_t)stream;
     int dev = 0;
     SGNN_HIP_CHECK(hipGetDevice(&dev));
     SGNN_REQUIRE(dev == p->device, "plan was created on device %d, current device is %d", p->device, dev);
@@ -804,8 +865,14 @@ extern "C" int sgnn_spmm_csr_f32(sgnn_spmm_plan *p, const float *val, const floa
         }
     }
     int vec = 1;
-    if (F % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 && aligned(x, 16) && aligned(out, 16)) vec = 4;
-    else if (F % 2 == 0 && ldx % 2 == 0 && ldo % 2 == 0 && aligned(x, 8) && aligned(out, 8)) vec = 2;
+    if (bits != 0) {
+        vec = 4;  // checked by the caller: F % 4 == 0 and 4-byte aligned packed rows
+        SGNN_REQUIRE(ldo % 4 == 0 && aligned(out, 16), "out must be 16-byte aligned with ldo %% 4 == 0 for the fused path");
+    } else if (F % 4 == 0 && dense.ldx % 4 == 0 && ldo % 4 == 0 && aligned(dense.x, 16) && aligned(out, 16)) {
+        vec = 4;
+    } else if (F % 2 == 0 && dense.ldx % 2 == 0 && ldo % 2 == 0 && aligned(dense.x, 8) && aligned(out, 8)) {
+        vec = 2;
+    }
     const int nvec = (int)(F / vec);
     const int gw = group_width(nvec);
     const int which = gw == 8 ? 0 : gw == 16 ? 1 : 2;
@@ -813,14 +880,39 @@ extern "C" int sgnn_spmm_csr_f32(sgnn_spmm_plan *p, const float *val, const floa
         const int rc = build_chunks(p, which, st);
         if (rc != SGNN_OK) return rc;
     }
-    ShortArgs a{p->rowptr, p->col, val, x, out, p->chunks[which], (int)p->n_chunks[which], p->empty_rows,
-                (int)p->n_empty, (int)F, ldx, ldo, accumulate, row_div};
-    PieceArgs s{p->col_long, p->eperm, val, x, p->partial, p->item_begin, p->item_len, p->cls_list, p->cls_off,
-                p->max_cls_items, (int)F, ldx};
+    ShortArgs a{p->rowptr, p->col, val, dense, out, p->chunks[which], (int)p->n_chunks[which], p->empty_rows,
+                (int)p->n_empty, (int)F, ldo, accumulate, row_div};
+    PieceArgs s{p->col_long, p->eperm, val, p->partial, p->item_begin, p->item_len, p->cls_list, p->cls_off,
+                p->max_cls_items, (int)F};
     FinalArgs f{p->long_rows, p->long_pbeg, p->partial, out, (int)p->n_long, (int)F, ldo, accumulate, row_div};
-    if (vec == 4) dispatch_shape<4>(nvec, a, s, f, st);
+    if (bits == 8) dispatch_shape_dq<8>(nvec, a, s, f, st);
+    else if (bits == 4) dispatch_shape_dq<4>(nvec, a, s, f, st);
+    else if (bits == 2) dispatch_shape_dq<2>(nvec, a, s, f, st);
+    else if (vec == 4) dispatch_shape<4>(nvec, a, s, f, st);
     else if (vec == 2) dispatch_shape<2>(nvec, a, s, f, st);
     else dispatch_shape<1>(nvec, a, s, f, st);
     SGNN_HIP_CHECK(hipGetLastError());
     return SGNN_OK;
+}
+
+extern "C" int sgnn_spmm_csr_f32(sgnn_spmm_plan *p, const float *val, const float *x, float *out, int64_t F,
+                                 int64_t ldx, int64_t ldo, int accumulate, const float *row_div,
+                                 sgnn_stream_t stream) {
+    SGNN_REQUIRE(p != nullptr, "plan is null");
+    SGNN_REQUIRE(ldx >= F, "leading dimension smaller than F (ldx=%lld F=%lld)", (long long)ldx, (long long)F);
+    SGNN_REQUIRE(x != nullptr || p->nnz == 0 || p->M == 0, "x is null");
+    DenseSrc d{x, ldx, nullptr, nullptr, nullptr, 0};
+    return spmm_run(p, val, d, 0, out, F, ldo, accumulate, row_div, (hipStream_t)stream);
+}
+
+extern "C" int sgnn_spmm_csr_dq_f32(sgnn_spmm_plan *p, const float *val, const uint8_t *q, const float *params,
+                                    const int32_t *row_slot, int bits, float *out, int64_t F, int64_t ldo,
+                                    int accumulate, const float *row_div, sgnn_stream_t stream) {
+    SGNN_REQUIRE(p != nullptr, "plan is null");
+    SGNN_REQUIRE(bits == 8 || bits == 4 || bits == 2, "bits=%d, expected 8, 4 or 2", bits);
+    SGNN_REQUIRE(F % 4 == 0, "the fused path needs F %% 4 == 0 (F=%lld): dequantize, then call sgnn_spmm_csr_f32", (long long)F);
+    SGNN_REQUIRE((q != nullptr && params != nullptr) || p->nnz == 0 || p->M == 0, "q / params is null");
+    SGNN_REQUIRE(aligned(q, 4) && aligned(params, 8), "q must be 4-byte and params 8-byte aligned");
+    DenseSrc d{nullptr, 0, q, params, row_slot, (int)F};
+    return spmm_run(p, val, d, bits, out, F, ldo, accumulate, row_div, (hipStream_t)stream);
 }

@@ -8,7 +8,7 @@ The reference computes an nnz-balanced OpenMP row split on first use and caches 
 getters/setters are still honoured so callers that inspect them keep working."""
 import torch
 
-from ..supergnn_ops import spmm
+from ..supergnn_ops import quant_segments, spmm
 
 
 def distribute_work_for_row(rowptr: torch.Tensor, value: torch.Tensor, num_threads_on_row: int) -> torch.Tensor:
@@ -71,3 +71,17 @@ def SPMM_backward(src, other: torch.Tensor, out: torch.Tensor) -> None:
         value_T = value_T.to(other.dtype)
     sparse_row = colptr.shape[0] - 1
     return spmm(colptr, row_T, value_T, other, out, sparse_row, row_splits, col_splits, plan=src.spmm_plan_T())
+
+
+def SPMM_forward_quantized(src, data_int8: torch.Tensor, quantized_params: torch.Tensor,
+                           work_range_per_proc: torch.Tensor, num_bits: int, out: torch.Tensor) -> None:
+    """out += A @ dequantize(data_int8), the remote / post-aggregation step of the forward pass with
+    the boundary rows still packed: replaces ``Quantizer_for_all_procs.dequantize_intX_to_fp32(...)``
+    followed by ``SPMM_forward(remote_adj_t, recv_buf, out)`` (super_gnn/aggregator.py:72-93) and
+    gives the same floats, without materialising ``recv_buf``."""
+    _, _, value = src.csr()
+    if value is not None:
+        value = value.to(torch.float32)
+    segs = quant_segments(work_range_per_proc, num_bits)
+    src.spmm_plan().run_quantized(value, data_int8, quantized_params, segs, num_bits, out, accumulate=True)
+    return None

@@ -34,7 +34,7 @@ from ._lib import check, lib
 __all__ = [
     "spmm", "quantize_tensor", "dequantize_tensor", "quantize_tensor_for_all_procs",
     "dequantize_tensor_for_all_procs", "quantize_tensor_v1", "dequantize_tensor_v1",
-    "SpmmPlan", "quant_segments",
+    "SpmmPlan", "quant_segments", "spmm_dequantized",
 ]
 
 
@@ -142,6 +142,36 @@ class SpmmPlan:
                                     F, F, F, int(bool(accumulate)), _ptr(s_div.dev) if s_div else None, _stream()))
         s_out.commit()
 
+    def run_quantized(self, value, data_int8, params, segs, bits, out, accumulate=True, row_div=None):
+        """out (+)= A @ dequantize(data_int8): the dense operand stays packed (row-group layout,
+        ``segs`` from quant_segments()) and is decoded inside the gather."""
+        _check_bits(bits)
+        _want(data_int8, torch.uint8, "data_int8")
+        _want(params, torch.float32, "quantized_params")
+        _want(out, torch.float32, "out")
+        if value is not None:
+            _want(value, torch.float32, "value")
+            if value.numel() != self.nnz:
+                raise ValueError(f"value has {value.numel()} entries, the matrix has {self.nnz}")
+        if out.dim() != 2 or out.shape[0] != self.M:
+            raise ValueError(f"out must be [{self.M}, F]")
+        F = out.shape[1]
+        if F % 4:
+            raise ValueError("the fused path needs a feature width divisible by 4")
+        if segs.n_rows != self.K:
+            raise ValueError(f"the segment table covers {segs.n_rows} rows, the sparse matrix has {self.K} columns")
+        if data_int8.numel() < segs.n_packed * F or params.numel() < self.K * 2:
+            raise ValueError("packed data / params smaller than the segment table requires")
+        if not (data_int8.is_cuda and params.is_cuda and out.is_cuda and (value is None or value.is_cuda)):
+            raise ValueError("the fused path takes GPU tensors only")
+        if not (data_int8.is_contiguous() and params.is_contiguous() and out.is_contiguous()):
+            raise ValueError("tensors must be contiguous")
+        if row_div is not None:
+            _want(row_div, torch.float32, "row_div")
+        slots = segs.row_slots(bits)
+        check(lib.sgnn_spmm_csr_dq_f32(self._h, _ptr(value), _ptr(data_int8), _ptr(params), _ptr(slots), bits,
+                                       _ptr(out), F, F, int(bool(accumulate)), _ptr(row_div), _stream()))
+
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
         if h:
@@ -211,6 +241,21 @@ class _Segments:
         self.seg = seg_host.to(dev)
         self.pseg = pseg_host.to(dev)
         self.pseg_host = pseg_host
+        self.seg_host = seg_host
+        self._slots = None
+
+    def row_slots(self, bits):
+        """Device table row -> position in the padded row space, or None when it is the identity
+        (every segment but the last holds a multiple of EPB rows)."""
+        epb = 8 // bits
+        sizes = (self.seg_host[1:] - self.seg_host[:-1])[:-1]
+        if self.P == 1 or bool((sizes % epb == 0).all()):
+            return None
+        if self._slots is None:
+            self._slots = torch.empty(self.n_rows, dtype=torch.int32, device=self.seg.device)
+            check(lib.sgnn_quant_row_slots(_ptr(self.seg), _ptr(self.pseg), self.P, bits, self.n_rows,
+                                           _ptr(self._slots), _stream()))
+        return self._slots
 
 
 def quant_segments(work_range, bits):
@@ -320,6 +365,20 @@ def dequantize_tensor_for_all_procs(input, output, dequantized_params, work_rang
     if work_range_per_proc.numel() != int(num_procs) + 1:
         raise ValueError("work_range_per_proc must have num_procs + 1 entries")
     _dequant_rows(input, output, dequantized_params, quant_segments(work_range_per_proc, bits), bits)
+
+
+def spmm_dequantized(rowptr, col, value, data_int8, quantized_params, work_range_per_proc, num_procs, bits, out,
+                     *, plan=None, accumulate=True, row_div=None):
+    """out (+)= A @ dequantize(data_int8) in one pass (no reference counterpart as a single call:
+    it fuses dequantize_tensor_for_all_procs with the spmm that follows it in
+    super_gnn/aggregator.py:72-93).  A has one column per quantized row."""
+    if work_range_per_proc.numel() != int(num_procs) + 1:
+        raise ValueError("work_range_per_proc must have num_procs + 1 entries")
+    segs = quant_segments(work_range_per_proc, bits)
+    if plan is None:
+        plan = _cached_plan(rowptr, col, segs.n_rows)
+    plan.run_quantized(value, data_int8, quantized_params, segs, bits, out, accumulate=accumulate, row_div=row_div)
+    return None
 
 
 # -------------------------------------------------------------------------------------------------

@@ -1,0 +1,136 @@
+"""GPU parity of the fused unpack+dequantize+SpMM path (remote boundary rows arrive packed).
+
+Checked three ways: (1) bit-identical to the separate GPU path "unpack+dequantize, then SpMM" with
+the same plan; (2) against the CPU oracle chain quant_rows -> dequant_rows -> spmm_accumulate within
+the SpMM tolerance; (3) the pre/post-aggregation data flow of super_gnn/aggregator.py:61-93 at a
+scaled-down size (local SpMM, then remote rows accumulated onto the same out)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from _util import random_csr, abs_sum64, assert_spmm_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(M, K, F, deg, bits, seg, seed, hubs=0):
+    import super_gnn_amd  # noqa: F401
+    from super_gnn_amd import supergnn_ops as ops
+    rowptr, col, val = random_csr(M, K, deg, seed=seed, empty_frac=0.1, hubs=hubs, hub_deg=min(K * 2, 1500))
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(K, F, generator=g)
+    x[::7] *= 30.0
+    seg_t = torch.tensor(seg, dtype=torch.int32)
+    P = seg_t.numel() - 1
+    npk = int(orc.packed_rows(seg, bits).sum())
+    q = torch.zeros(npk, F, dtype=torch.uint8, device="cuda")
+    params = torch.zeros(K, 2, device="cuda")
+    ops.quantize_tensor_for_all_procs(x.cuda(), q, params, seg_t, P, bits)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).cuda(), torch.from_numpy(col).cuda(), K)
+    return ops, plan, rowptr, col, val, x, seg_t, P, q, params
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+@pytest.mark.parametrize("M,K,F,deg,seg,hubs", [
+    (800, 600, 128, 9, [0, 600], 0),
+    (800, 600, 128, 9, [0, 600], 4),                  # long rows: class-partitioned pieces
+    (500, 403, 128, 7, [0, 5, 5, 130, 131, 403], 2),   # ragged segments: the row -> slot table is needed
+    (300, 256, 256, 6, [0, 100, 256], 0),             # full wavefront per row; segment sizes divisible by 4
+    (300, 250, 64, 6, [0, 33, 250], 1),               # 16-lane groups
+    (200, 180, 1024, 4, [0, 180], 0),                 # 4 words per lane
+    (150, 120, 100, 5, [0, 61, 120], 0),              # partly idle group
+    (120, 90, 8, 5, [0, 90], 0),
+])
+def test_fused_equals_separate_and_oracle(bits, M, K, F, deg, seg, hubs):
+    ops, plan, rowptr, col, val, x, seg_t, P, q, params = _setup(M, K, F, deg, bits, seg, seed=M + F + bits, hubs=hubs)
+    init = torch.randn(M, F, generator=torch.Generator().manual_seed(1))
+    vald = torch.from_numpy(val).cuda()
+    # separate GPU path
+    recv = torch.empty(K, F, device="cuda")
+    ops.dequantize_tensor_for_all_procs(q, recv, params, seg_t, P, bits)
+    out_sep = init.clone().cuda()
+    plan.run(vald, recv, out_sep, accumulate=True)
+    # fused
+    out_fused = init.clone().cuda()
+    ops.spmm_dequantized(None, None, vald, q, params, seg_t, P, bits, out_fused, plan=plan)
+    torch.cuda.synchronize()
+    assert torch.equal(out_fused, out_sep), "fused must equal dequantize-then-SpMM bit for bit"
+    # oracle chain on the CPU
+    q_ref, p_ref = orc.quant_rows(x.numpy(), seg, bits)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    d_ref = orc.dequant_rows(q_ref, p_ref, seg, bits, F)
+    want = init.numpy().copy()
+    orc.spmm_accumulate(rowptr, col, val, d_ref, want)
+    got = out_fused.cpu().numpy()
+    tol = 1e-6 + 1e-5 * np.abs(want)
+    bad = np.abs(got - want) > tol
+    if bad.any():  # long rows: adjudicate with the fp64 forward error bound
+        f64 = orc.spmm_f64(rowptr, col, val, d_ref, init.numpy())
+        S = orc.spmm_f64(rowptr, col, np.abs(val), np.abs(d_ref), np.abs(init.numpy()))
+        bound = (np.diff(rowptr)[:, None] + 1.0) * 2.0 ** -24 * S
+        bad &= np.abs(got - f64) > bound + 1e-6
+    assert not bad.any()
+    # overwrite mode and unit weights
+    out_o = torch.full((M, F), 9.0, device="cuda")
+    ops.spmm_dequantized(None, None, None, q, params, seg_t, P, bits, out_o, plan=plan, accumulate=False)
+    out_o2 = torch.full((M, F), 9.0, device="cuda")
+    plan.run(None, recv, out_o2, accumulate=False)
+    assert torch.equal(out_o, out_o2)
+
+
+def test_pre_post_aggregation_flow():
+    # local rows [0, K_local) are fp32; remote boundary rows arrive int2-packed in 8 segments
+    from super_gnn_amd import SparseTensor, SPMM_forward, SPMM_forward_quantized, synth
+    from super_gnn_amd.quantizer import Quantizer_for_all_procs
+    M, K_local, K_remote, F, bits = 20000, 20000, 5000, 128, 2
+    rp_l, col_l = synth.rmat_graph(M, 150000, seed=6)
+    rowptr_r, col_r, val_r = random_csr(M, K_remote, 4, seed=8, empty_frac=0.3, hubs=3, hub_deg=900)
+    g = torch.Generator().manual_seed(7)
+    x_local = torch.randn(K_local, F, generator=g)
+    x_remote = torch.randn(K_remote, F, generator=g)
+    wr = torch.tensor([0, 625, 1250, 1875, 2500, 3125, 3750, 4375, 5000], dtype=torch.int32)
+    qz = Quantizer_for_all_procs(8, bits)
+    npk = sum(qz.get_quantized_splits(625) for _ in range(8))
+    q = torch.zeros(npk, F, dtype=torch.uint8, device="cuda")
+    params = torch.zeros(K_remote, 2, device="cuda")
+    qz.quantize_fp32_to_intX(x_remote.cuda(), q, params, wr)
+    A_local = SparseTensor(rowptr=rp_l, col=col_l.to(torch.int64), value=torch.ones(col_l.numel()), sparse_sizes=(M, K_local), is_sorted=True).cuda()
+    A_remote = SparseTensor(rowptr=torch.from_numpy(rowptr_r), col=torch.from_numpy(col_r), value=torch.from_numpy(val_r),
+                            sparse_sizes=(M, K_remote), is_sorted=True).cuda()
+    # (A) the reference's sequence: local SpMM, dequantize into recv_buf, remote SpMM onto the same out
+    out_a = torch.zeros(M, F, device="cuda")
+    SPMM_forward(A_local, x_local.cuda(), out_a)
+    recv = torch.empty(K_remote, F, device="cuda")
+    qz.dequantize_intX_to_fp32(q, recv, params, wr)
+    SPMM_forward(A_remote, recv, out_a)
+    # (B) fused
+    out_b = torch.zeros(M, F, device="cuda")
+    SPMM_forward(A_local, x_local.cuda(), out_b)
+    SPMM_forward_quantized(A_remote, q, params, wr, bits, out_b)
+    assert torch.equal(out_a, out_b)
+    # and against the CPU oracle
+    want = np.zeros((M, F), np.float32)
+    orc.spmm_accumulate(rp_l.numpy(), col_l.numpy().astype(np.int64), np.ones(col_l.numel(), np.float32), x_local.numpy(), want)
+    q_ref, p_ref = orc.quant_rows(x_remote.numpy(), wr.numpy(), bits)
+    orc.spmm_accumulate(rowptr_r, col_r, val_r, orc.dequant_rows(q_ref, p_ref, wr.numpy(), bits, F), want)
+    got = out_b.cpu().numpy()
+    # one fp64 reference for the two-step sum: local part first, remote part accumulated onto it
+    ones = np.ones(col_l.numel(), np.float32)
+    cl = col_l.numpy().astype(np.int64)
+    d_ref = orc.dequant_rows(q_ref, p_ref, wr.numpy(), bits, F)
+    f64 = orc.spmm_f64(rp_l.numpy(), cl, ones, x_local.numpy()) + orc.spmm_f64(rowptr_r, col_r, val_r, d_ref)
+    S = abs_sum64(rp_l.numpy(), cl, ones, x_local.numpy()) + abs_sum64(rowptr_r, col_r, val_r, d_ref)
+    deg = np.diff(rp_l.numpy()) + np.diff(rowptr_r)
+    assert_spmm_close(got, want, f64, S, deg, what="pre/post flow")
+
+
+def test_fused_errors():
+    ops, plan, rowptr, col, val, x, seg_t, P, q, params = _setup(50, 40, 64, 3, 2, [0, 40], seed=3)
+    out = torch.zeros(50, 64, device="cuda")
+    with pytest.raises(ValueError):
+        ops.spmm_dequantized(None, None, None, q, params, seg_t, P, 3, out, plan=plan)
+    with pytest.raises(ValueError):
+        ops.spmm_dequantized(None, None, None, q, params, torch.tensor([0, 39], dtype=torch.int32), 1, 2, out, plan=plan)
+    with pytest.raises(ValueError):
+        ops.spmm_dequantized(None, None, None, q, params, seg_t, P, 2, torch.zeros(50, 62, device="cuda"), plan=plan)
