@@ -27,7 +27,12 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this file (see profiles/), scaled by what the same counters read for sgnn_stream_copy_f32 of a
 # known size.  Keyed by workload name; None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # spmm_piece_kernel: FETCH_SIZE 7062609 x 2.000 + WRITE_SIZE 860068 x 1.000 (KiB per launch)
+    "rmat_2450000n_62000000e_F128_gcn_weighted_sum": 15_345_000_000,
+    # quant_pack_rows16_kernel<2,...>: FETCH_SIZE 500044 x 2.000 + WRITE_SIZE 81291 x 1.000
+    "quant_pack_int2_1000000x256": 1_107_000_000,
+}
 
 
 def log(*a):
@@ -146,8 +151,14 @@ def main():
     ap.add_argument("--uniform-rows", type=int, default=0, help="diagnostic: replace the R-MAT graph by uniform random "
                     "rows of --uniform-degree neighbours over --nodes columns")
     ap.add_argument("--uniform-degree", type=int, default=25)
-    ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy"],
-                    help="rmat: headline SpMM (default); quant: int2 quantize+pack as the step; copy: streaming copy")
+    ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy", "prepost", "sbm"],
+                    help="rmat: headline SpMM (default); quant: int2 quantize+pack as the step; copy: streaming copy; "
+                         "prepost: one partition with packed remote rows, fused vs separate; sbm: dense-degree graph, F=602")
+    ap.add_argument("--local-nodes", type=int, default=8_000_000)
+    ap.add_argument("--remote-nodes", type=int, default=2_000_000)
+    ap.add_argument("--local-und-edges", type=int, default=160_000_000)
+    ap.add_argument("--remote-edges", type=int, default=80_000_000)
+    ap.add_argument("--sbm-nodes", type=int, default=233_000)
     ap.add_argument("--nodes", type=int, default=2_450_000)
     ap.add_argument("--und-edges", type=int, default=31_000_000)
     ap.add_argument("--feat", type=int, default=128)
@@ -276,7 +287,9 @@ def main():
         if dom == "spmm_short_kernel":
             dom_bytes = b_short
         elif dom == "spmm_piece_kernel":
-            dom_bytes = info["long_edges"] * (4 * F + 8) + info["pieces"] * 4 * F
+            # per edge: dense row + col + val (the per-unit figure of the gather model); the kernel's own
+            # bookkeeping (edge permutation, piece partial sums) is overhead, not algorithmic traffic
+            dom_bytes = info["long_edges"] * (4 * F + 8)
         else:
             dom_bytes = b_total
         ach = dom_bytes / dom_ms / 1e6
@@ -302,6 +315,102 @@ def main():
                                "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl),
                                "kernel": dom, "kernel_avg_ms": round(dom_ms, 5), "algorithmic_bytes": int(dom_bytes)},
                   "cpu_baseline": None if args.no_cpu else cpu_baseline_spmm(rowptr, col, w, x)}
+
+    # ---- one partition in pre/post-aggregation mode: remote rows arrive int2-packed -------------
+    if args.workload == "prepost":
+        F, bits = args.feat, args.bits
+        Ml, Kr = args.local_nodes, args.remote_nodes
+        t0 = time.perf_counter()
+        rp_l, col_l = synth.rmat_graph(Ml, args.local_und_edges, seed=6, device=dev)
+        g = torch.Generator(device=dev); g.manual_seed(7)
+        # remote edges: rows follow the local degree distribution, columns uniform over the boundary set
+        deg_l = (rp_l[1:] - rp_l[:-1]).to(torch.float32)
+        rows_r = torch.multinomial(deg_l + 0.05, args.remote_edges, replacement=True, generator=g)
+        cols_r = torch.randint(0, Kr, (args.remote_edges,), generator=g, device=dev)
+        rp_r, col_r = synth.csr_from_pairs(rows_r, cols_r, Ml, Kr, dedupe=True)
+        del rows_r, cols_r, deg_l
+        x_l = torch.randn(Ml, F, generator=g, device=dev)
+        x_r = torch.randn(Kr, F, generator=g, device=dev)
+        torch.cuda.synchronize()
+        log(f"[bench] prepost: local {Ml} rows / {col_l.numel()} edges, remote {Kr} cols / {col_r.numel()} edges, "
+            f"built in {time.perf_counter() - t0:.1f}s")
+        P = 8
+        wr = torch.tensor([Kr * i // P for i in range(P + 1)], dtype=torch.int32)
+        epb = 8 // bits
+        npk = sum((int(wr[i + 1] - wr[i]) + epb - 1) // epb for i in range(P))
+        q = torch.empty(npk, F, dtype=torch.uint8, device=dev)
+        prm = torch.empty(Kr, 2, device=dev)
+        ops.quantize_tensor_for_all_procs(x_r, q, prm, wr, P, bits)
+        del x_r
+        plan_l = ops.SpmmPlan(rp_l, col_l, Ml)
+        plan_r = ops.SpmmPlan(rp_r, col_r, Kr)
+        segs = ops.quant_segments(wr, bits)
+        out = torch.zeros(Ml, F, device=dev)
+        recv = torch.empty(Kr, F, device=dev)
+        ms_local = time_steps(lambda: plan_l.run(None, x_l, out, accumulate=True), args.steps, args.warmup)
+
+        def separate():
+            ops.dequantize_tensor_for_all_procs(q, recv, prm, wr, P, bits)
+            plan_r.run(None, recv, out, accumulate=True)
+
+        ms_sep = time_steps(separate, args.steps, args.warmup)
+        _lib.profile_start()
+        ms_fused = time_steps(lambda: plan_r.run_quantized(None, q, prm, segs, bits, out, accumulate=True), args.steps, args.warmup)
+        prof = _lib.profile_stop()
+        nl, nr = col_l.numel(), col_r.numel()
+        per_kernel = {k: round(v[1] / v[0], 5) for k, v in prof.items()}
+        dom = max(prof, key=lambda k: prof[k][1])
+        info_r = plan_r.info()
+        dom_edges = info_r["long_edges"] if "piece" in dom else nr - info_r["long_edges"]
+        dom_bytes = dom_edges * (F + 16)  # survey figure for a remote edge: one packed row of F bytes + params + col/val
+        dom_ms = prof[dom][1] / prof[dom][0]
+        extra.update({"local_spmm_ms": round(ms_local, 4), "remote_separate_ms": round(ms_sep, 4),
+                      "remote_fused_ms": round(ms_fused, 4), "fused_speedup_on_remote_step": round(ms_sep / ms_fused, 3),
+                      "local_GEdges_per_s": round(nl / ms_local / 1e6, 3), "kernel_avg_ms": per_kernel})
+        log(f"[bench] local SpMM {ms_local:.3f} ms; remote: separate {ms_sep:.3f} ms vs fused {ms_fused:.3f} ms")
+        total = ms_local + ms_fused
+        result = {"metric": "SpMM GEdges/s, pre/post-aggregation partition (local fp32 + int2-packed remote rows, fused)",
+                  "value": round((nl + nr) / total / 1e6, 4), "unit": "GEdges/s",
+                  "config": {"workload": f"prepost_{Ml}n_{nl}e_local_{Kr}c_{nr}e_remote_int{bits}_F{F}", "F": F, "bits": bits},
+                  "ms_per_step": total, "dtype": "f32",
+                  "roofline": {"bound": "hbm", "achieved": round(dom_bytes / dom_ms / 1e6, 1), "peak": HBM_PEAK_GBPS,
+                               "unit": "GB/s", "frac": round(dom_bytes / dom_ms / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None,
+                               "kernel": dom, "kernel_avg_ms": round(dom_ms, 5), "algorithmic_bytes": int(dom_bytes)},
+                  "cpu_baseline": None}
+
+    # ---- dense-degree community graph, wide odd feature rows --------------------------------------
+    if args.workload == "sbm":
+        F = 602
+        n = args.sbm_nodes // 50 * 50
+        t0 = time.perf_counter()
+        rowptr, col = synth.sbm_graph(n, 50, 0.03048, 0.001524, seed=3, device=dev)
+        g = torch.Generator(device=dev); g.manual_seed(4)
+        x = torch.rand(n, F, generator=g, device=dev) * 2 - 1
+        torch.cuda.synchronize()
+        nnz = col.numel()
+        log(f"[bench] sbm: {n} nodes, {nnz} edges (avg degree {nnz / n:.0f}), built in {time.perf_counter() - t0:.1f}s")
+        plan = ops.SpmmPlan(rowptr, col, n, long_row_threshold=args.long_threshold, piece_edges=args.piece_edges)
+        info = plan.info()
+        out = torch.zeros(n, F, device=dev)
+        _lib.profile_start()
+        ms = time_steps(lambda: plan.run(None, x, out, accumulate=True), args.steps, args.warmup)
+        prof = _lib.profile_stop()
+        per_kernel = {k: round(v[1] / v[0], 5) for k, v in prof.items()}
+        dom = max(prof, key=lambda k: prof[k][1])
+        dom_ms = prof[dom][1] / prof[dom][0]
+        dom_edges = info["long_edges"] if "piece" in dom else nnz - info["long_edges"]
+        dom_bytes = dom_edges * (4 * F + 4)
+        b_total = spmm_gather_bytes(nnz, n, F, weighted=False, accumulate=True, mean=False)
+        extra.update({"kernel_avg_ms": per_kernel, "plan": {k: info[k] for k in ("long_rows", "pieces", "long_edges")},
+                      "spmm_total_gather_GBps": round(b_total / ms / 1e6, 1)})
+        log(f"[bench] sbm sum: {ms:.3f} ms/step, {nnz / ms / 1e6:.2f} GEdges/s, {b_total / ms / 1e6:.0f} GB/s gather model, {per_kernel}")
+        result = {"metric": "SpMM GEdges/s (dense-degree community graph, F=602 fp32)", "value": round(nnz / ms / 1e6, 4),
+                  "unit": "GEdges/s", "config": {"workload": f"sbm_{n}n_{nnz}e_F{F}_sum", "F": F}, "ms_per_step": ms,
+                  "dtype": "f32",
+                  "roofline": {"bound": "hbm", "achieved": round(dom_bytes / dom_ms / 1e6, 1), "peak": HBM_PEAK_GBPS,
+                               "unit": "GB/s", "frac": round(dom_bytes / dom_ms / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None,
+                               "kernel": dom, "kernel_avg_ms": round(dom_ms, 5), "algorithmic_bytes": int(dom_bytes)},
+                  "cpu_baseline": None}
 
     line = {"metric": result["metric"], "value": result["value"], "unit": result["unit"], "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(result["ms_per_step"], 5),
