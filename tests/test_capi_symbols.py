@@ -16,7 +16,8 @@ def _declared():
 def test_header_declares_the_expected_entry_points():
     names = _declared()
     for must in ("sgnn_spmm_csr_f32", "sgnn_spmm_plan_create", "sgnn_quant_pack_rows_f32",
-                 "sgnn_unpack_dequant_rows_f32", "sgnn_quant_v1_f32", "sgnn_dequant_v1_f32", "sgnn_last_error"):
+                 "sgnn_unpack_dequant_rows_f32", "sgnn_quant_v1_f32", "sgnn_dequant_v1_f32", "sgnn_last_error",
+                 "sgnn_spmm_csr_dq_f32", "sgnn_quant_row_slots"):
         assert must in names
 
 
