@@ -12,26 +12,28 @@ from ..supergnn_ops import quant_segments, spmm
 
 
 def distribute_work_for_row(rowptr: torch.Tensor, value: torch.Tensor, num_threads_on_row: int) -> torch.Tensor:
-    """Greedy contiguous row split balanced by the per-row sum of ``value``
-    (super_gnn/ops/spmm_kernel.py:8-29), vectorised: the reference walks the rows in a Python loop.
-    Kept for interface parity; the GPU kernels do not consume it."""
+    """Greedy contiguous row split balanced by the per-row sum of ``value``: a range is closed at the
+    first row whose addition lifts the running sum above total // threads, and that row opens the
+    next range (super_gnn/ops/spmm_kernel.py:8-29).  The reference walks all rows in a Python loop;
+    this finds each cut with one binary search over the prefix sums.  Kept for interface parity: the
+    GPU kernels balance work through the SpMM plan instead and do not consume the split."""
     num_rows = rowptr.numel() - 1
     row_splits = torch.full((num_threads_on_row + 1,), num_rows, dtype=torch.int32)
     row_splits[0] = 0
-    if num_rows == 0:
+    if num_rows == 0 or value is None or value.numel() == 0:
         return row_splits
-    csum = torch.zeros(value.numel() + 1, dtype=torch.float64)
-    torch.cumsum(value.detach().to("cpu", torch.float64), 0, out=csum[1:])
-    rp = rowptr.detach().cpu()
-    flops = (csum[rp[1:]] - csum[rp[:-1]]).to(value.dtype)
-    target = flops.sum() // num_threads_on_row
-    cur, tid = flops.new_zeros(()), 0
-    for i, f in enumerate(flops.tolist()):
-        cur = cur + f
-        if cur > target and tid < num_threads_on_row:
-            row_splits[tid + 1] = i
-            tid += 1
-            cur = flops.new_tensor(f)
+    edge_prefix = torch.zeros(value.numel() + 1, dtype=torch.float64)
+    edge_prefix[1:] = torch.cumsum(value.detach().to("cpu", torch.float64), 0)
+    prefix = edge_prefix[rowptr.detach().cpu()]          # prefix[i] = sum of the first i rows
+    target = float(torch.div(prefix[-1], num_threads_on_row, rounding_mode="floor"))
+    start_sum, first_candidate = 0.0, 0                   # sum before the open range; earliest row that may close it
+    for t in range(1, num_threads_on_row + 1):
+        k = int(torch.searchsorted(prefix, torch.tensor(start_sum + target, dtype=torch.float64), right=True))
+        cut = max(k - 1, first_candidate)                 # first row i with prefix[i+1] - start_sum > target
+        if cut >= num_rows:
+            break
+        row_splits[t] = cut
+        start_sum, first_candidate = float(prefix[cut]), cut + 1
     row_splits[-1] = num_rows
     return row_splits
 

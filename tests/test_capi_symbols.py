@@ -63,3 +63,37 @@ def test_facade_helpers_match_reference_closed_forms():
     q = Quantizer_for_all_procs(4, 2)
     assert Quantizer_for_all_procs.ctx is q and q.get_quantized_splits(5) == 2 and q.get_quantized_splits(8) == 2
     assert Quantizer_for_all_procs(4, 8).get_quantized_splits(5) == 5
+
+
+def test_row_split_matches_the_reference_greedy_rule():
+    """distribute_work_for_row (super_gnn/ops/spmm_kernel.py:8-29) restated literally as a loop here,
+    against the binary-search version the package ships."""
+    import numpy as np
+    import torch
+    from super_gnn_amd.ops.spmm_kernel import distribute_work_for_row, disribute_work_for_col
+
+    def literal(rowptr, value, T):
+        flops = [float(value[rowptr[i]:rowptr[i + 1]].sum()) for i in range(len(rowptr) - 1)]
+        target = sum(flops) // T
+        splits = [len(flops)] * (T + 1)
+        splits[0] = 0
+        cur, tid = 0.0, 0
+        for i, f in enumerate(flops):
+            cur += f
+            if cur > target and tid < T:
+                splits[tid + 1] = i
+                tid += 1
+                cur = f
+        splits[-1] = len(flops)
+        return splits
+
+    rng = np.random.default_rng(0)
+    for M, T in [(50, 4), (200, 8), (7, 16), (1000, 3)]:
+        deg = rng.integers(0, 12, M)
+        deg[rng.integers(0, M, 3)] = 80  # rows heavier than the per-thread target
+        rowptr = np.concatenate([[0], np.cumsum(deg)])
+        value = np.ones(int(rowptr[-1]), dtype=np.float32)  # integer sums: no rounding ambiguity
+        got = distribute_work_for_row(torch.from_numpy(rowptr), torch.from_numpy(value), T).tolist()
+        assert got == literal(rowptr, value, T), (M, T)
+    assert disribute_work_for_col(torch.zeros(3, 128), 1).tolist() == [0, 128]
+    assert disribute_work_for_col(torch.zeros(3, 10), 4).tolist() == [0, 2, 4, 6, 10]
