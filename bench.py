@@ -268,7 +268,7 @@ def main():
         torch.cuda.synchronize()
         info = plan.info()
         extra["plan_build_ms"] = round((time.perf_counter() - t0) * 1e3, 1)
-        extra["plan"] = {k: info[k] for k in ("long_rows", "pieces", "long_edges", "long_row_threshold", "piece_edges")}
+        extra["plan"] = {k: info[k] for k in ("long_rows", "pieces", "long_edges", "long_row_threshold", "piece_edges", "partitioned")}
         log(f"[bench] plan: {extra['plan']} built in {extra['plan_build_ms']} ms")
         out = torch.zeros(M, F, device=dev)
         step = lambda: plan.run(w, x, out, accumulate=True)  # noqa: E731

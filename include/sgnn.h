@@ -45,9 +45,11 @@ int sgnn_version(void);
 
 /* Per-matrix schedule: 32-bit column indices, the row classes and their work lists.
  *   short rows : chunks of consecutive rows (~128 edges), one lane group per chunk;
- *   long rows  : edges regrouped by column class (a hash of col, 8 classes) and cut into pieces, one lane group per
- *                piece, workgroup i serving class i % 8 so that each XCD's L2 caches its own class
- *                of dense rows; partial sums land in a buffer owned by the plan;
+ *   long rows  : edges regrouped by column class (a hash of col, 8 classes) and cut into pieces, one
+ *                lane group per piece, workgroup i serving class i % 8 so that each XCD's L2 caches
+ *                its own class of dense rows; partial sums land in a buffer owned by the plan.  The
+ *                regrouping is skipped when column popularity is essentially uniform (it then only
+ *                costs): pieces are cut from the CSR order instead;
  *   empty rows : a list, used only by the modes that must write them.
  * Plays the role of the row_splits the reference computes once per matrix and caches on it
  * (super_gnn/ops/spmm_kernel.py:49-58, distribute_work_for_row :8-29).
@@ -69,8 +71,10 @@ int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int col_is_i64
 int sgnn_spmm_plan_destroy(sgnn_spmm_plan *plan);
 
 /* info[0]=M, [1]=K, [2]=nnz, [3]=#long rows, [4]=#pieces, [5]=edges in long rows,
- * [6]=long_row_threshold, [7]=piece_edges. */
-int sgnn_spmm_plan_info(const sgnn_spmm_plan *plan, int64_t info[8]);
+ * [6]=long_row_threshold, [7]=piece_edges, [8]=1 if the long rows were regrouped by column class,
+ * [9]=share of all edges that point at the 16384 most popular columns, in parts per million (0 when
+ * it was not measured). */
+int sgnn_spmm_plan_info(const sgnn_spmm_plan *plan, int64_t info[10]);
 
 /* out[M,F] (+)= A[M,K] * x[K,F], fp32, row-major, leading dimensions ldx / ldo (in floats).
  *

@@ -31,6 +31,8 @@ namespace sgnn {
 constexpr int kBlock = 256;
 constexpr int kDefaultLongThreshold = 128;  // rows with more edges go to the class-partitioned piece path
 constexpr int kDefaultPieceEdges = 32;      // minimum edges per piece of a long row
+constexpr int kPopularColumns = 16384;      // size of the "popular" column set the plan looks at
+constexpr double kPartitionMinShare = 0.02; // below this share of all edges (popularity ~uniform) leave the long rows as they are
 
 __host__ __device__ constexpr int unroll_of(int nv) { return nv == 1 ? 8 : nv == 2 ? 4 : nv == 3 ? 3 : 2; }
 
@@ -123,8 +125,8 @@ __device__ __forceinline__ void fma_row(float (&acc)[NV][VEC], float w, const Fe
 }
 
 // Accumulate the `deg` edges listed at colp into acc for one feature tile.  The weight of edge i is
-// val[eperm[i]] (val may be null = all ones).
-template <int VEC, int G, int NV, int BITS>
+// val[eperm[i]], or val[i] when eperm is null (val may be null = all ones).
+template <int VEC, int G, int NV, int BITS, bool PERM>
 __device__ __forceinline__ void gather_piece(float (&acc)[NV][VEC], const int32_t *__restrict__ colp,
                                              const int32_t *__restrict__ eperm, const float *__restrict__ val,
                                              int deg, const DenseSrc &dense, const int (&off)[NV],
@@ -135,7 +137,7 @@ __device__ __forceinline__ void gather_piece(float (&acc)[NV][VEC], const int32_
     float nw = 1.0f;
     if (lig < deg) {
         nc = __builtin_nontemporal_load(colp + lig);
-        if (val) nw = val[__builtin_nontemporal_load(eperm + lig)];
+        if (val) nw = PERM ? val[__builtin_nontemporal_load(eperm + lig)] : __builtin_nontemporal_load(val + lig);
     }
     for (int base = 0; base < deg; base += G) {
         const int myc = nc;
@@ -143,7 +145,7 @@ __device__ __forceinline__ void gather_piece(float (&acc)[NV][VEC], const int32_
         const int nidx = base + G + lig;
         if (nidx < deg) {
             nc = __builtin_nontemporal_load(colp + nidx);
-            if (val) nw = val[__builtin_nontemporal_load(eperm + nidx)];
+            if (val) nw = PERM ? val[__builtin_nontemporal_load(eperm + nidx)] : __builtin_nontemporal_load(val + nidx);
         }
         const int cnt = deg - base < G ? deg - base : G;
         for (int j = 0; j < cnt; j += U) {
@@ -348,7 +350,7 @@ __global__ __launch_bounds__(kBlock) void spmm_empty_rows_kernel(const int32_t *
 // rows of its own class and the eight 4 MB L2s hold eight DISJOINT sets of popular rows instead of
 // eight copies of the same set.
 // ------------------------------------------------------------------------------------------------
-template <int VEC, int G, int NV, int BITS>
+template <int VEC, int G, int NV, int BITS, bool PERM>
 __global__ __launch_bounds__(kBlock) void spmm_piece_kernel(
     const int32_t *__restrict__ col_long, const int32_t *__restrict__ eperm, const float *__restrict__ val,
     const DenseSrc dense, float *__restrict__ partial, const int32_t *__restrict__ item_begin,
@@ -378,7 +380,8 @@ __global__ __launch_bounds__(kBlock) void spmm_piece_kernel(
 #pragma unroll
             for (int k = 0; k < VEC; ++k) acc[v][k] = 0.0f;
         }
-        gather_piece<VEC, G, NV, BITS>(acc, col_long + b, eperm + b, val, len, dense, off, act, lig);
+        gather_piece<VEC, G, NV, BITS, PERM>(acc, col_long + b, PERM ? eperm + b : nullptr, (PERM || !val) ? val : val + b,
+                                             len, dense, off, act, lig);
 #pragma unroll
         for (int v = 0; v < NV; ++v)
             if (act[v]) vec_store<VEC>(partial + (int64_t)item * F + off[v], acc[v]);
@@ -517,6 +520,15 @@ __global__ __launch_bounds__(kBlock) void narrow_cols_kernel(const SrcT *__restr
     if (any_bad) atomicOr(bad, 1);
 }
 
+// How often each column occurs (its in-degree): decides at plan time whether regrouping the long
+// rows by column class can pay off.
+__global__ __launch_bounds__(kBlock) void column_popularity_kernel(const int32_t *__restrict__ col, int64_t n,
+                                                                   int *__restrict__ popularity) {
+    int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (; i < n; i += stride) atomicAdd(popularity + col[i], 1);
+}
+
 // ------------------------------------------------------------------------------------------------
 // Launch tables.
 // ------------------------------------------------------------------------------------------------
@@ -555,8 +567,12 @@ static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &
             // workgroup i serves class i % 8: grid = 8 * (workgroups of the fullest class)
             const uint32_t nb = (uint32_t)kNumXCD * (uint32_t)((s.max_cls_items + GPB - 1) / GPB);
             ProfScope prof(BITS == 0 ? K_SPMM_PIECE : K_FUSED_PIECE, st);
-            hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS>), dim3(nb), dim3(kBlock), 0, st, s.col_long, s.eperm,
-                               s.val, a.dense, s.partial, s.item_begin, s.item_len, s.cls_list, s.cls_off, s.F);
+            if (s.eperm)
+                hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS, true>), dim3(nb), dim3(kBlock), 0, st, s.col_long,
+                                   s.eperm, s.val, a.dense, s.partial, s.item_begin, s.item_len, s.cls_list, s.cls_off, s.F);
+            else
+                hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS, false>), dim3(nb), dim3(kBlock), 0, st, s.col_long,
+                                   s.eperm, s.val, a.dense, s.partial, s.item_begin, s.item_len, s.cls_list, s.cls_off, s.F);
         }
         const uint32_t nb = (uint32_t)((f.n_long + GPB - 1) / GPB);
         ProfScope prof(K_SPMM_LONG_FINAL, st);
@@ -609,6 +625,8 @@ struct sgnn_spmm_plan {
     int device = 0;
     int64_t M = 0, K = 0, nnz = 0;
     int long_thresh = 0, piece_edges = 0;
+    bool partitioned = false;   // long rows regrouped by column class
+    double top_share = 0.0;     // share of all edges that point at the kPopularColumns most popular columns
     int64_t *rowptr = nullptr;  // device, owned
     int32_t *col = nullptr;     // device, owned
     // long rows
@@ -671,7 +689,7 @@ extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     (void)hipFree(p->col);
     (void)hipFree(p->long_rows);
     (void)hipFree(p->long_pbeg);
-    (void)hipFree(p->col_long);
+    if (p->col_long != p->col) (void)hipFree(p->col_long);
     (void)hipFree(p->eperm);
     (void)hipFree(p->item_begin);
     (void)hipFree(p->item_len);
@@ -746,30 +764,78 @@ static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void
         if (h_bad) return fail(SGNN_ERR_RANGE, "a column index lies outside [0, %lld)", (long long)K);
     }
 
-    // ---- long rows: regroup by column class, cut into pieces ----------------------------------
+    // ---- long rows: regroup by column class (when popular columns exist), cut into pieces --------
     if (p->n_long > 0) {
         if ((rc = upload(&p->long_rows, long_rows, st)) != SGNN_OK) return rc;
-        int32_t *d_long_off = nullptr, *d_cls_count = nullptr;
-        if ((rc = upload(&d_long_off, long_off, st)) != SGNN_OK) return rc;
-        SGNN_HIP_CHECK(hipMalloc(&d_cls_count, sizeof(int32_t) * (size_t)p->n_long * kNumXCD));
-        SGNN_HIP_CHECK(hipMalloc(&p->col_long, sizeof(int32_t) * (size_t)p->long_edges));
-        SGNN_HIP_CHECK(hipMalloc(&p->eperm, sizeof(int32_t) * (size_t)p->long_edges));
-        hipLaunchKernelGGL(partition_long_rows_kernel, dim3((uint32_t)p->n_long), dim3(kBlock), 0, st, p->rowptr, p->col,
-                           p->long_rows, d_long_off, p->col_long, p->eperm, d_cls_count);
-        std::vector<int32_t> cls_count((size_t)p->n_long * kNumXCD);
-        hipError_t e1 = hipGetLastError();
-        hipError_t e2 = hipMemcpyAsync(cls_count.data(), d_cls_count, sizeof(int32_t) * cls_count.size(), hipMemcpyDeviceToHost, st);
-        hipError_t e3 = hipStreamSynchronize(st);
-        (void)hipFree(d_long_off);
-        (void)hipFree(d_cls_count);
-        SGNN_HIP_CHECK(e1);
-        SGNN_HIP_CHECK(e2);
-        SGNN_HIP_CHECK(e3);
+        // Regrouping lets each XCD's L2 keep its own slice of the popular dense rows; it pays when a
+        // modest set of columns receives a large share of the gathers (power-law graphs) and costs
+        // ~15% (smaller pieces, permuted val reads) when no column is popular.  Measure it.
+        const int part_env = env_int("SGNN_SPMM_PARTITION", -1);
+        if (part_env >= 0) {
+            p->partitioned = part_env != 0;
+        } else if (K <= kPopularColumns) {
+            p->partitioned = true;  // every dense row is "popular": eight disjoint slices beat eight full copies
+        } else {
+            int *pop = nullptr;
+            SGNN_HIP_CHECK(hipMalloc(&pop, sizeof(int) * (size_t)K));
+            SGNN_HIP_CHECK(hipMemsetAsync(pop, 0, sizeof(int) * (size_t)K, st));
+            const int nb = (int)std::min<int64_t>((nnz + kBlock - 1) / kBlock, 65536);
+            hipLaunchKernelGGL(column_popularity_kernel, dim3(nb), dim3(kBlock), 0, st, p->col, nnz, pop);
+            std::vector<int> h_pop((size_t)K);
+            hipError_t e1 = hipGetLastError();
+            hipError_t e2 = hipMemcpyAsync(h_pop.data(), pop, sizeof(int) * h_pop.size(), hipMemcpyDeviceToHost, st);
+            hipError_t e3 = hipStreamSynchronize(st);
+            (void)hipFree(pop);
+            SGNN_HIP_CHECK(e1);
+            SGNN_HIP_CHECK(e2);
+            SGNN_HIP_CHECK(e3);
+            std::nth_element(h_pop.begin(), h_pop.begin() + kPopularColumns, h_pop.end(), std::greater<int>());
+            int64_t top = 0;
+            for (int i = 0; i < kPopularColumns; ++i) top += h_pop[i];
+            p->top_share = (double)top / (double)nnz;
+            // a clearly popular set, or at least non-uniform popularity with enough reuse per column to matter
+            p->partitioned = p->top_share >= 0.2 || (p->top_share >= kPartitionMinShare && nnz >= 8 * K);
+        }
+        std::vector<int32_t> cls_count;
+        if (p->partitioned) {
+            int32_t *d_long_off = nullptr, *d_cls_count = nullptr;
+            if ((rc = upload(&d_long_off, long_off, st)) != SGNN_OK) return rc;
+            SGNN_HIP_CHECK(hipMalloc(&d_cls_count, sizeof(int32_t) * (size_t)p->n_long * kNumXCD));
+            SGNN_HIP_CHECK(hipMalloc(&p->col_long, sizeof(int32_t) * (size_t)p->long_edges));
+            SGNN_HIP_CHECK(hipMalloc(&p->eperm, sizeof(int32_t) * (size_t)p->long_edges));
+            hipLaunchKernelGGL(partition_long_rows_kernel, dim3((uint32_t)p->n_long), dim3(kBlock), 0, st, p->rowptr, p->col,
+                               p->long_rows, d_long_off, p->col_long, p->eperm, d_cls_count);
+            cls_count.resize((size_t)p->n_long * kNumXCD);
+            hipError_t e1 = hipGetLastError();
+            hipError_t e2 = hipMemcpyAsync(cls_count.data(), d_cls_count, sizeof(int32_t) * cls_count.size(), hipMemcpyDeviceToHost, st);
+            hipError_t e3 = hipStreamSynchronize(st);
+            (void)hipFree(d_long_off);
+            (void)hipFree(d_cls_count);
+            SGNN_HIP_CHECK(e1);
+            SGNN_HIP_CHECK(e2);
+            SGNN_HIP_CHECK(e3);
+        } else {
+            p->col_long = p->col;  // pieces index the CSR arrays directly; no permutation
+            p->eperm = nullptr;
+        }
 
         std::vector<int32_t> item_begin, item_len, long_pbeg, cls_off(kNumXCD + 1, 0);
         std::vector<std::vector<int32_t>> cls_items(kNumXCD);
         long_pbeg.push_back(0);
+        int rr = 0;  // round-robin class for unpartitioned pieces (balances the eight work lists)
         for (int64_t slot = 0; slot < p->n_long; ++slot) {
+            if (!p->partitioned) {
+                const int64_t b = h_rowptr[long_rows[slot]], n = h_rowptr[long_rows[slot] + 1] - b;
+                const int64_t len = std::max<int64_t>(std::max(p->piece_edges, 64), (n + 255) / 256);
+                for (int64_t o = 0; o < n; o += len) {
+                    cls_items[rr].push_back((int32_t)item_begin.size());
+                    rr = (rr + 1) % kNumXCD;
+                    item_begin.push_back((int32_t)(b + o));
+                    item_len.push_back((int32_t)std::min<int64_t>(len, n - o));
+                }
+                long_pbeg.push_back((int32_t)item_begin.size());
+                continue;
+            }
             int32_t base = long_off[slot];
             for (int c = 0; c < kNumXCD; ++c) {
                 const int32_t n = cls_count[slot * kNumXCD + c];
@@ -828,10 +894,11 @@ extern "C" int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int
     return SGNN_OK;
 }
 
-extern "C" int sgnn_spmm_plan_info(const sgnn_spmm_plan *p, int64_t info[8]) {
+extern "C" int sgnn_spmm_plan_info(const sgnn_spmm_plan *p, int64_t info[10]) {
     SGNN_REQUIRE(p != nullptr && info != nullptr, "null argument");
     info[0] = p->M; info[1] = p->K; info[2] = p->nnz; info[3] = p->n_long; info[4] = p->n_items;
     info[5] = p->long_edges; info[6] = p->long_thresh; info[7] = p->piece_edges;
+    info[8] = p->partitioned ? 1 : 0; info[9] = (int64_t)(p->top_share * 1e6);
     return SGNN_OK;
 }
 

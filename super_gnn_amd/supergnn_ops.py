@@ -109,9 +109,10 @@ class SpmmPlan:
         self.device = dev
 
     def info(self):
-        buf = (ctypes.c_int64 * 8)()
+        buf = (ctypes.c_int64 * 10)()
         check(lib.sgnn_spmm_plan_info(self._h, buf))
-        keys = ("M", "K", "nnz", "long_rows", "pieces", "long_edges", "long_row_threshold", "piece_edges")
+        keys = ("M", "K", "nnz", "long_rows", "pieces", "long_edges", "long_row_threshold", "piece_edges",
+                "partitioned", "top_share_ppm")
         return dict(zip(keys, list(buf)))
 
     def run(self, value, mat, out, accumulate=True, row_div=None):

@@ -227,3 +227,39 @@ def test_power_law_graph_weighted_and_mean():
     got_m, _ = _run_gpu(rowptr, col, None, x, z, accumulate=True, row_div=deg, col_dtype=torch.int32)
     _assert_close(got_m, want_m, orc.spmm_f64(rowptr, col, ones, x) / deg[:, None],
                   _abs_sum64(rowptr, col, ones, x) / deg[:, None], dg, what="rmat mean")
+
+
+@pytest.mark.parametrize("mode", ["0", "1", None])
+def test_long_row_modes_agree_and_auto_choice(mode, monkeypatch):
+    """Long rows are either regrouped by column class or cut in CSR order; both must meet the same
+    bar, and the automatic choice must regroup a power-law graph and leave a uniform one alone."""
+    from super_gnn_amd import synth
+    if mode is None:
+        monkeypatch.delenv("SGNN_SPMM_PARTITION", raising=False)
+    else:
+        monkeypatch.setenv("SGNN_SPMM_PARTITION", mode)
+    n = 40000
+    rp_t, col_t = synth.rmat_graph(n, 500000, seed=3)
+    rowptr, col = rp_t.numpy(), col_t.numpy().astype(np.int64)
+    rng = np.random.default_rng(0)
+    val = rng.random(col.shape[0], dtype=np.float32)
+    x = rng.standard_normal((n, 64), dtype=np.float32)
+    z = np.zeros((n, 64), np.float32)
+    want = z.copy(); orc.spmm_accumulate(rowptr, col, val, x, want)
+    got, plan = _run_gpu(rowptr, col, val, x, z, accumulate=True)
+    info = plan.info()
+    assert info["long_rows"] > 0
+    assert info["partitioned"] == (0 if mode == "0" else 1)
+    _assert_close(got, want, orc.spmm_f64(rowptr, col, val, x), _abs_sum64(rowptr, col, val, x), np.diff(rowptr), what=f"mode {mode}")
+    if mode is None:
+        # uniform popularity over many columns: left in CSR order
+        M, K = 3000, 2000000
+        rowptr_u = np.arange(M + 1, dtype=np.int64) * 600
+        col_u = np.sort(rng.integers(0, K, (M, 600)), axis=1).reshape(-1).astype(np.int64)
+        val_u = rng.random(col_u.shape[0], dtype=np.float32)
+        xu = rng.standard_normal((K, 4), dtype=np.float32)
+        zu = np.zeros((M, 4), np.float32)
+        wu = zu.copy(); orc.spmm_accumulate(rowptr_u, col_u, val_u, xu, wu)
+        gu, plan_u = _run_gpu(rowptr_u, col_u, val_u, xu, zu, accumulate=True)
+        assert plan_u.info()["partitioned"] == 0 and 0 < plan_u.info()["top_share_ppm"] < 100000
+        _assert_close(gu, wu, orc.spmm_f64(rowptr_u, col_u, val_u, xu), _abs_sum64(rowptr_u, col_u, val_u, xu), np.diff(rowptr_u), what="uniform")
