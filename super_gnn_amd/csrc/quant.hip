@@ -370,13 +370,18 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
         if (s == 0.0f) s = 1.0f;
         zp[rl] = mn;
         sc[rl] = s;
-        rinv[rl] = 1.0f / s;
+        rinv[rl] = __builtin_amdgcn_rcpf(s);  // hardware reciprocal, within 1 ulp of 1/s
         if (!(s >= 0x1p-100f && s <= 0x1p100f)) lane_exact = true;
         if (l16 == 0) *reinterpret_cast<float2 *>(params + row[rl] * 2) = make_float2(mn, s);
     }
 
-    // Codes: (x - zp) * RN(1/scale), accepted when provably equal to the IEEE quotient after
-    // rounding; otherwise this lane redoes its elements with the IEEE division.
+    // Codes.  The reference's code is RNE(RN((x - zp) / scale)).  The quotient is first formed as
+    // (x - zp) * rcp(scale) with the 1-ulp hardware reciprocal: the product is within 1.5 * 2^-23
+    // relative of the true quotient and the IEEE quotient within 2^-24, both are below 256, so the two
+    // differ by less than 2^-13.  If the product is further than 2^-13 from every half-integer,
+    // rounding it gives the same integer as rounding the IEEE quotient; a lane that sees an element
+    // inside that guard band (about 1 in 4000), or a scale whose reciprocal is not a normal number,
+    // redoes its elements with the IEEE division.  The stored bytes are always the exact formula's.
     const int shift = (EPB - 1 - (d % EPB)) * BITS;
     uint32_t words[RL][NV];
 #pragma unroll
@@ -389,7 +394,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
                 for (int e = 0; e < VEC; ++e) {
                     const float qf = (xv[rl][v][e] - zp[rl]) * rinv[rl];
                     const float ri = rintf(qf);
-                    if (!(fabsf(qf - ri) < 0.5f - 0x1p-14f)) lane_exact = true;
+                    if (!(fabsf(qf - ri) < 0.5f - 0x1p-13f)) lane_exact = true;
                     word |= (uint32_t)ri << (8 * e);
                 }
             }
