@@ -1,0 +1,146 @@
+"""The aggregation data flow of super_gnn/aggregator.py on one GPU: P partitions of one graph in one
+process, loop-back exchange.
+
+  * fp32 exchange: the concatenated partition outputs must equal the GLOBAL product A @ X of the
+    unpartitioned graph (CPU oracle), forward, and A^T @ G backward -- this pins the partition
+    builder, the splits and both exchange directions against something that knows nothing of them;
+  * int8/int4/int2 exchange: must equal the same flow computed on the CPU with the oracle's
+    quantize -> dequantize at every boundary crossing."""
+import numpy as np
+import pytest
+import scipy.sparse as sp
+import torch
+
+from oracle import oracle as orc
+from _util import abs_sum64, assert_spmm_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph(n=12000, und_edges=90000, seed=5):
+    from super_gnn_amd import synth
+    rowptr, col = synth.rmat_graph(n, und_edges, seed=seed)
+    w = synth.gcn_norm_weights(rowptr, col)
+    return rowptr, col, w
+
+
+def _csr_np(st):
+    rowptr, col, val = st.csr()
+    return rowptr.cpu().numpy().astype(np.int64), col.cpu().numpy().astype(np.int64), val.cpu().numpy().astype(np.float32)
+
+
+def _cpu_spmm(st, x, out):
+    rp, c, v = _csr_np(st)
+    if out.shape[0]:
+        orc.spmm_accumulate(rp, c, v, np.ascontiguousarray(x), out)
+
+
+@pytest.mark.parametrize("pre", [False, True])
+@pytest.mark.parametrize("P", [1, 4])
+def test_fp32_exchange_equals_global_product(pre, P):
+    from super_gnn_amd.aggregator import LoopbackWorld
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    rowptr, col, w = _graph()
+    n, F = rowptr.numel() - 1, 64
+    graphs = build_loopback_partitions(rowptr, col, w, P, F, num_bits=32, is_pre_delay=pre)
+    assert sum(g.local_adj_t.sparse_size(0) for g in graphs) == n
+    for g in graphs:  # every send segment is mirrored by the peer's recv segment
+        for r, h in enumerate(graphs):
+            assert g.comm_splits.send_splits[r] == h.comm_splits.recv_splits[graphs.index(g)]
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(n, F, generator=gen)
+    feats = [x[g.node_range[0]:g.node_range[1]].cuda().requires_grad_() for g in graphs]
+    world = LoopbackWorld(graphs, 32, pre)
+    outs = world.aggregate(feats)
+    got = torch.cat(outs).detach().cpu().numpy()
+    rp, c, v = rowptr.numpy(), col.numpy().astype(np.int64), w.numpy()
+    want = np.zeros((n, F), np.float32)
+    orc.spmm_accumulate(rp, c, v, x.numpy(), want)
+    assert_spmm_close(got, want, orc.spmm_f64(rp, c, v, x.numpy()), abs_sum64(rp, c, v, x.numpy()), np.diff(rp), what="forward")
+    # backward: d(sum(out * G))/dX = A^T G
+    G = torch.randn(n, F, generator=gen)
+    torch.autograd.backward(outs, [G[g.node_range[0]:g.node_range[1]].cuda() for g in graphs])
+    got_g = torch.cat([f.grad for f in feats]).cpu().numpy()
+    AT = sp.csr_matrix((v, c, rp), shape=(n, n)).T.tocsr(); AT.sort_indices()
+    rpt, ct, vt = AT.indptr.astype(np.int64), AT.indices.astype(np.int64), AT.data.astype(np.float32)
+    want_g = np.zeros((n, F), np.float32)
+    orc.spmm_accumulate(rpt, ct, vt, G.numpy(), want_g)
+    assert_spmm_close(got_g, want_g, orc.spmm_f64(rpt, ct, vt, G.numpy()), abs_sum64(rpt, ct, vt, G.numpy()), np.diff(rpt), what="backward")
+    if pre and P > 1:  # pre-aggregation must not send more rows than plain boundary exchange would
+        plain = build_loopback_partitions(rowptr, col, w, P, F, num_bits=32, is_pre_delay=False)
+        assert sum(sum(g.comm_splits.send_splits) for g in graphs) <= sum(sum(g.comm_splits.send_splits) for g in plain)
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+@pytest.mark.parametrize("pre", [False, True])
+def test_quantized_exchange_equals_cpu_flow(bits, pre):
+    from super_gnn_amd.aggregator import LoopbackWorld
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    rowptr, col, w = _graph(n=8000, und_edges=60000, seed=9)
+    n, F, P = rowptr.numel() - 1, 128, 4
+    graphs = build_loopback_partitions(rowptr, col, w, P, F, num_bits=bits, is_pre_delay=pre)
+    gen = torch.Generator().manual_seed(1)
+    x = torch.randn(n, F, generator=gen)
+    xs = [x[g.node_range[0]:g.node_range[1]] for g in graphs]
+    feats = [t.cuda().requires_grad_() for t in xs]
+    outs = LoopbackWorld(graphs, bits, pre).aggregate(feats)
+
+    def crossing(buf, splits):
+        """what a buffer looks like on the far side: quantize per segment, dequantize (oracle)"""
+        seg = np.concatenate([[0], np.cumsum(splits)]).astype(np.int32)
+        if buf.shape[0] == 0:
+            return buf
+        q, prm = orc.quant_rows(np.ascontiguousarray(buf), seg, bits)
+        return orc.dequant_rows(q, prm, seg, bits, buf.shape[1])
+
+    # forward on the CPU
+    sent = []
+    for g, xp in zip(graphs, xs):
+        ns = sum(g.comm_splits.send_splits)
+        sb = np.zeros((ns, F), np.float32)
+        if pre:
+            _cpu_spmm(g.adj_t_pre_post_aggr_to, xp.numpy(), sb)
+        elif ns:
+            sb = xp.numpy()[g.idx_nodes_send_to_others.cpu().numpy()]
+        sent.append(crossing(sb, g.comm_splits.send_splits))
+    want_outs = []
+    for r, (g, xp) in enumerate(zip(graphs, xs)):
+        segs = []
+        for p, h in enumerate(graphs):
+            o = np.concatenate([[0], np.cumsum(h.comm_splits.send_splits)])
+            segs.append(sent[p][o[r]:o[r + 1]])
+        recv = np.concatenate(segs) if segs else np.zeros((0, F), np.float32)
+        out = np.zeros((g.local_adj_t.sparse_size(0), F), np.float32)
+        _cpu_spmm(g.local_adj_t, xp.numpy(), out)
+        _cpu_spmm(g.adj_t_pre_post_aggr_from if pre else g.remote_adj_t, recv, out)
+        want_outs.append(out)
+    for r, (o, wnt) in enumerate(zip(outs, want_outs)):
+        got = o.detach().cpu().numpy()
+        assert np.all(np.abs(got - wnt) <= 1e-4 + 1e-4 * np.abs(wnt)), f"rank {r}"  # hub rows: summation order
+        assert (np.abs(got - wnt) <= 1e-6 + 1e-5 * np.abs(wnt)).mean() > 0.999
+    # backward runs, is finite, and is close to the unquantized gradient at the quantization error scale
+    G = torch.randn(n, F, generator=gen)
+    torch.autograd.backward(outs, [G[g.node_range[0]:g.node_range[1]].cuda() for g in graphs])
+    got_g = torch.cat([f.grad for f in feats]).cpu().numpy()
+    rp, c, v = rowptr.numpy(), col.numpy().astype(np.int64), w.numpy()
+    AT = sp.csr_matrix((v, c, rp), shape=(n, n)).T.tocsr()
+    exact_g = AT @ G.numpy()
+    assert np.isfinite(got_g).all()
+    rel = np.linalg.norm(got_g - exact_g) / np.linalg.norm(exact_g)
+    assert rel < {8: 0.01, 4: 0.1, 2: 0.5}[bits], rel
+
+
+def test_bf16_param_transport_matches_reference_wire_format():
+    # the reference ships (zero_point, scale) as bf16 (communicator.py:283-294)
+    from super_gnn_amd.aggregator import LoopbackWorld
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    rowptr, col, w = _graph(n=4000, und_edges=30000, seed=2)
+    n, F, P = rowptr.numel() - 1, 64, 2
+    graphs = build_loopback_partitions(rowptr, col, w, P, F, num_bits=8, is_pre_delay=False)
+    x = torch.randn(n, F, generator=torch.Generator().manual_seed(3))
+    feats = [x[g.node_range[0]:g.node_range[1]].cuda() for g in graphs]
+    o32 = torch.cat(LoopbackWorld(graphs, 8, False).aggregate(feats))
+    o16 = torch.cat(LoopbackWorld(graphs, 8, False, params_wire_dtype=torch.bfloat16).aggregate(feats))
+    prm = graphs[0].comm_buf_for_quantization.quantized_recv_params_buf_fp32
+    assert torch.equal(prm, prm.to(torch.bfloat16).to(torch.float32))  # what arrived is bf16-representable
+    assert not torch.equal(o32, o16) and torch.allclose(o32, o16, atol=0.05, rtol=0.05)
