@@ -151,7 +151,7 @@ def main():
     ap.add_argument("--uniform-rows", type=int, default=0, help="diagnostic: replace the R-MAT graph by uniform random "
                     "rows of --uniform-degree neighbours over --nodes columns")
     ap.add_argument("--uniform-degree", type=int, default=25)
-    ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy", "prepost", "sbm"],
+    ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy", "prepost", "sbm", "aggregate"],
                     help="rmat: headline SpMM (default); quant: int2 quantize+pack as the step; copy: streaming copy; "
                          "prepost: one partition with packed remote rows, fused vs separate; sbm: dense-degree graph, F=602")
     ap.add_argument("--local-nodes", type=int, default=8_000_000)
@@ -159,6 +159,9 @@ def main():
     ap.add_argument("--local-und-edges", type=int, default=160_000_000)
     ap.add_argument("--remote-edges", type=int, default=80_000_000)
     ap.add_argument("--sbm-nodes", type=int, default=233_000)
+    ap.add_argument("--parts", type=int, default=8, help="aggregate: number of vertex partitions simulated in this process")
+    ap.add_argument("--exchange-bits", type=int, default=2, help="aggregate: 32 (fp32 rows) or 8/4/2 (packed)")
+    ap.add_argument("--pre", type=int, default=1, help="aggregate: 1 = pre/post aggregation, 0 = plain boundary exchange")
     ap.add_argument("--nodes", type=int, default=2_450_000)
     ap.add_argument("--und-edges", type=int, default=31_000_000)
     ap.add_argument("--feat", type=int, default=128)
@@ -411,6 +414,38 @@ def main():
                                "unit": "GB/s", "frac": round(dom_bytes / dom_ms / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None,
                                "kernel": dom, "kernel_avg_ms": round(dom_ms, 5), "algorithmic_bytes": int(dom_bytes)},
                   "cpu_baseline": None}
+
+    # ---- one GraphSAGE-style aggregation (forward + backward) over P partitions of the headline graph ----
+    if args.workload == "aggregate":
+        from super_gnn_amd.aggregator import LoopbackWorld
+        from super_gnn_amd.data_manager import build_loopback_partitions
+        F = args.feat
+        rowptr, col, w, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
+        t0 = time.perf_counter()
+        graphs = build_loopback_partitions(rowptr, col, w, args.parts, F, num_bits=args.exchange_bits,
+                                           is_pre_delay=bool(args.pre), device=dev)
+        log(f"[bench] {args.parts} partitions built in {time.perf_counter() - t0:.1f}s; rows exchanged per direction: "
+            f"{sum(sum(g.comm_splits.send_splits) for g in graphs)}")
+        world = LoopbackWorld(graphs, args.exchange_bits, bool(args.pre))
+        feats = [x[g.node_range[0]:g.node_range[1]].clone().requires_grad_() for g in graphs]
+        grads = [torch.randn(g.node_range[1] - g.node_range[0], F, device=dev) for g in graphs]
+
+        def step():
+            outs = world.aggregate(feats)
+            torch.autograd.backward(outs, grads)
+            for f in feats:
+                f.grad = None
+
+        ms = time_steps(step, args.steps, args.warmup)
+        ms_fwd = time_steps(lambda: world.aggregate([f.detach() for f in feats]), args.steps, args.warmup)
+        nnz = col.numel()
+        extra.update({"forward_ms": round(ms_fwd, 4), "forward_backward_ms": round(ms, 4),
+                      "rows_exchanged": sum(sum(g.comm_splits.send_splits) for g in graphs)})
+        log(f"[bench] aggregate fwd {ms_fwd:.3f} ms, fwd+bwd {ms:.3f} ms ({2 * nnz / ms / 1e6:.2f} GEdges/s)")
+        result = {"metric": "aggregation layer GEdges/s (forward+backward, loop-back exchange)",
+                  "value": round(2 * nnz / ms / 1e6, 4), "unit": "GEdges/s",
+                  "config": {"workload": f"aggregate_rmat_{args.nodes}n_{nnz}e_F{F}_P{args.parts}_bits{args.exchange_bits}_pre{args.pre}"},
+                  "ms_per_step": ms, "dtype": "f32", "roofline": None, "cpu_baseline": None}
 
     line = {"metric": result["metric"], "value": result["value"], "unit": result["unit"], "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(result["ms_per_step"], 5),

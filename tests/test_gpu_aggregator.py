@@ -144,3 +144,50 @@ def test_bf16_param_transport_matches_reference_wire_format():
     prm = graphs[0].comm_buf_for_quantization.quantized_recv_params_buf_fp32
     assert torch.equal(prm, prm.to(torch.bfloat16).to(torch.float32))  # what arrived is bf16-representable
     assert not torch.equal(o32, o16) and torch.allclose(o32, o16, atol=0.05, rtol=0.05)
+
+
+def test_sage_model_is_partition_invariant_and_trains():
+    """A 3-layer GraphSAGE over 4 partitions (fp32 exchange) must produce the outputs and weight
+    gradients of the same model over the unpartitioned graph; with an int2 exchange it must still train."""
+    from super_gnn_amd.aggregator import LoopbackWorld
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    from super_gnn_amd.layers import LoopbackSAGE
+    rowptr, col, _ = _graph(n=6000, und_edges=40000, seed=4)
+    n, Fin, H, C = rowptr.numel() - 1, 64, 128, 8
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(n, Fin, generator=gen).cuda()
+    y = torch.randint(0, C, (n,), generator=gen).cuda()
+    torch.manual_seed(0)
+    model = LoopbackSAGE(Fin, H, C, num_layers=3, dropout=0.0).cuda()
+    model.reset_parameters()
+
+    def run(P, bits, pre):
+        graphs = build_loopback_partitions(rowptr, col, None, P, Fin, num_bits=bits, is_pre_delay=pre)
+        world = LoopbackWorld(graphs, bits, pre)
+        feats = [x[g.node_range[0]:g.node_range[1]] for g in graphs]
+        model.zero_grad()
+        out = torch.cat(model(world, feats))
+        loss = torch.nn.functional.nll_loss(out, y)
+        loss.backward()
+        return out.detach(), loss.item(), [p.grad.clone() for p in model.parameters()]
+
+    out1, loss1, g1 = run(1, 32, False)
+    for pre in (False, True):
+        out4, loss4, g4 = run(4, 32, pre)
+        assert torch.allclose(out1, out4, atol=2e-4, rtol=1e-3)
+        assert abs(loss1 - loss4) < 1e-4
+        for a, b in zip(g1, g4):
+            assert torch.allclose(a, b, atol=1e-4, rtol=1e-2)
+    # int2 exchange with pre/post aggregation: a few SGD steps reduce the loss
+    graphs = build_loopback_partitions(rowptr, col, None, 4, Fin, num_bits=2, is_pre_delay=True)
+    world = LoopbackWorld(graphs, 2, True)
+    feats = [x[g.node_range[0]:g.node_range[1]] for g in graphs]
+    opt = torch.optim.Adam(model.parameters(), lr=5e-3)
+    losses = []
+    for _ in range(12):
+        opt.zero_grad()
+        loss = torch.nn.functional.nll_loss(torch.cat(model(world, feats)), y)
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < losses[0] - 0.05, losses
