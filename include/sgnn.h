@@ -125,6 +125,26 @@ int sgnn_unpack_dequant_rows_f32(const uint8_t *q, float *x, const float *params
                                  const int32_t *seg, const int32_t *pseg, int P, int64_t n_rows,
                                  int64_t n_packed_rows, int64_t F, int bits, sgnn_stream_t stream);
 
+/* The same two kernels with the operands as they sit either side of the boundary exchange:
+ *   - row_index (i64[n_rows], device, nullable): row r of the quantizer's input is
+ *     x[row_index[r] * ldx ...] -- the index_select into send_buf that precedes quantization in
+ *     the plain (non pre-aggregated) mode, super_gnn/aggregator.py:48, folded into the load.
+ *     Entries must lie in [0, n_src_rows); an entry outside reads row 0 instead of faulting.
+ *     NULL: rows are x[r * ldx ...] and n_src_rows is ignored.
+ *   - params_bf16 = 1: params is bf16[n,2] instead of f32[n,2] -- the form in which the reference
+ *     ships (zero_point, scale), super_gnn/communicator.py:283-294 (copy_ to the bf16 buffer,
+ *     all_to_all, copy_ back).  Codes are computed from the fp32 values; only the stored pair is
+ *     rounded (to nearest even, NaN kept quiet), and the receiver widens it exactly. */
+int sgnn_quant_pack_rows_wire_f32(const float *x, int64_t ldx, const int64_t *row_index,
+                                  int64_t n_src_rows, uint8_t *q, void *params, int params_bf16,
+                                  const int32_t *seg, const int32_t *pseg, int P, int64_t n_rows,
+                                  int64_t n_packed_rows, int64_t F, int bits, sgnn_stream_t stream);
+
+int sgnn_unpack_dequant_rows_wire_f32(const uint8_t *q, float *x, const void *params,
+                                      int params_bf16, const int32_t *seg, const int32_t *pseg,
+                                      int P, int64_t n_rows, int64_t n_packed_rows, int64_t F,
+                                      int bits, sgnn_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Fused unpack + dequantize + SpMM (pre/post-aggregation mode)
  * ------------------------------------------------------------------------------------------- */
@@ -147,6 +167,15 @@ int sgnn_quant_row_slots(const int32_t *seg, const int32_t *pseg, int P, int bit
 int sgnn_spmm_csr_dq_f32(sgnn_spmm_plan *plan, const float *val, const uint8_t *q, const float *params,
                          const int32_t *row_slot, int bits, float *out, int64_t F, int64_t ldo,
                          int accumulate, const float *row_div, sgnn_stream_t stream);
+
+/* sgnn_spmm_csr_dq_f32 with params in either form (params_bf16: see
+ * sgnn_quant_pack_rows_wire_f32).  With a 0/1 selection matrix as A this is also the scatter of the
+ * plain mode's backward pass, local_grad.index_add_(0, idx, dequantize(q))
+ * (super_gnn/aggregator.py:159-175), summed in index order and free of atomics. */
+int sgnn_spmm_csr_dq_wire_f32(sgnn_spmm_plan *plan, const float *val, const uint8_t *q,
+                              const void *params, int params_bf16, const int32_t *row_slot, int bits,
+                              float *out, int64_t F, int64_t ldo, int accumulate,
+                              const float *row_div, sgnn_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Feature-packed mixed-bit quantization ("v1")

@@ -4,7 +4,8 @@ reference's own Python call signatures.  Importing this package loads libsgnn_hi
 it is absent -- there is no CPU fallback."""
 from . import _lib  # noqa: F401  (fails loudly when the HIP library is missing)
 from . import supergnn_ops  # noqa: F401
-from .ops.spmm_kernel import SPMM_backward, SPMM_forward, SPMM_forward_quantized  # noqa: F401
+from .ops.spmm_kernel import (SPMM_backward, SPMM_backward_quantized, SPMM_forward,  # noqa: F401
+                              SPMM_forward_quantized)
 from .quantizer import Quantizer_for_all_procs, QuantizerForMixedBits, QuantizerForPureBits  # noqa: F401
 from .sparse import SparseTensor  # noqa: F401
 

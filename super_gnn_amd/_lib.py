@@ -27,6 +27,9 @@ SIGNATURES = {
     "sgnn_unpack_dequant_rows_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
     "sgnn_quant_row_slots": (_int, [_vp, _vp, _int, _int, _i64, _vp, _vp]),
     "sgnn_spmm_csr_dq_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _i64, _i64, _int, _vp, _vp]),
+    "sgnn_quant_pack_rows_wire_f32": (_int, [_vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
+    "sgnn_unpack_dequant_rows_wire_f32": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
+    "sgnn_spmm_csr_dq_wire_f32": (_int, [_vp, _vp, _vp, _vp, _int, _vp, _int, _vp, _i64, _i64, _int, _vp, _vp]),
     "sgnn_quant_v1_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "sgnn_dequant_v1_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _vp]),
     "sgnn_profile_enable": (_int, [_int]),

@@ -12,17 +12,28 @@ Per partition and direction the steps and their order are the reference's:
                                            -> quantize+pack -> exchange (reverse direction)
                                            -> local transposed SpMM -> accumulate the returned rows
 
-Because the partitions share one process, the exchange is a set of device copies between their
-buffers, and the phases run for all partitions before the next phase starts.  With num_bits in
-{8,4,2} the receiver never materialises the fp32 rows: it feeds the packed bytes straight into the
-fused unpack+dequantize+SpMM kernel (forward), which is bit-identical to dequantizing first.
+What is folded together on the GPU (each fold gives the floats of the unfolded sequence):
+
+  * with num_bits in {8,4,2} the receiver never materialises fp32 rows: the packed bytes go straight
+    into the fused unpack+dequantize+SpMM kernel, forward (remote graph) and backward (transposed
+    pre-aggregation graph, or the 0/1 selection matrix that stands for ``index_add_``);
+  * in the plain mode the boundary rows are quantized straight out of the feature matrix
+    (``index_select`` folded into the quantizer's loads);
+  * (zero_point, scale) can be produced and consumed as bf16 pairs, the reference's wire format;
+  * "zero the buffer, then accumulate A @ x into it" is one overwriting SpMM (same floats: the sum
+    starts from 0 either way; rows without edges are written as zeros).
+
+Because the partitions share one process, every partition's buffers are slices of one arena per
+buffer kind, and the exchange is ONE row-permuting copy per buffer (send rows of all ranks -> recv
+rows of all ranks).  The send-side chain and the local SpMMs are issued on two streams.
 """
 from typing import List, Sequence
 
 import torch
 
-from .ops.spmm_kernel import SPMM_backward, SPMM_forward, SPMM_forward_quantized
+from .ops.spmm_kernel import (SPMM_backward, SPMM_backward_quantized, SPMM_forward, SPMM_forward_quantized)
 from .quantizer import Quantizer_for_all_procs
+from .sparse import SparseTensor
 
 
 def _cumulative(splits):
@@ -32,39 +43,95 @@ def _cumulative(splits):
     return out
 
 
-def _exchange(graphs, direction: str, quantized: bool, params_wire_dtype=None):
-    """Loop-back all-to-all.  forward: rank p's send segment for r -> rank r's recv segment from p.
-    backward: rank r's recv-side segment for p travels back into rank p's send-side segment for r
-    (the reference reuses the same buffers with the roles swapped, aggregator.py:113-118,153-166)."""
-    P = len(graphs)
-    for p in range(P):
-        gp = graphs[p]
-        s_off = _cumulative(gp.comm_splits.send_splits)
-        s_off_q = _cumulative(gp.comm_splits.send_splits_int2) if quantized else None
-        for r in range(P):
-            n = gp.comm_splits.send_splits[r]
-            if n == 0 or p == r:
+class _Arena(object):
+    """Buffers of all partitions for one feature width, and the row permutations of the exchange."""
+
+    def __init__(self, graphs, F, quantized, params_dtype, device):
+        self.F, self.quantized, self.params_dtype = F, quantized, params_dtype
+        self.send_tot = _cumulative([sum(g.comm_splits.send_splits) for g in graphs])
+        self.recv_tot = _cumulative([sum(g.comm_splits.recv_splits) for g in graphs])
+        n = self.send_tot[-1]
+        assert n == self.recv_tot[-1]
+        self.send = torch.zeros((n, F), dtype=torch.float32, device=device)
+        self.recv = torch.zeros((n, F), dtype=torch.float32, device=device)
+        self.perm = self._permutation(graphs, "send_splits", "recv_splits", self.send_tot, self.recv_tot, device)
+        self.inv_perm = torch.empty_like(self.perm)
+        self.inv_perm[self.perm] = torch.arange(n, device=device)
+        if not quantized:
+            return
+        self.qs_tot = _cumulative([sum(g.comm_splits.send_splits_int2) for g in graphs])
+        self.qr_tot = _cumulative([sum(g.comm_splits.recv_splits_int2) for g in graphs])
+        nq = self.qs_tot[-1]
+        self.send_q = torch.zeros((nq, F), dtype=torch.uint8, device=device)
+        self.recv_q = torch.zeros((nq, F), dtype=torch.uint8, device=device)
+        self.send_params = torch.zeros((n, 2), dtype=params_dtype, device=device)
+        self.recv_params = torch.zeros((n, 2), dtype=params_dtype, device=device)
+        self.perm_q = self._permutation(graphs, "send_splits_int2", "recv_splits_int2", self.qs_tot, self.qr_tot, device)
+        self.inv_perm_q = torch.empty_like(self.perm_q)
+        self.inv_perm_q[self.perm_q] = torch.arange(nq, device=device)
+        # one (zero_point, scale) pair moves as one machine word
+        word = torch.int64 if params_dtype == torch.float32 else torch.int32
+        self.send_params_w = self.send_params.view(word)
+        self.recv_params_w = self.recv_params.view(word)
+
+    def bind(self, graphs):
+        """Point every partition's buffer attributes at its slices of this arena."""
+        for p, g in enumerate(graphs):
+            s0, s1, r0, r1 = self.send_tot[p], self.send_tot[p + 1], self.recv_tot[p], self.recv_tot[p + 1]
+            g.comm_buf.send_buf, g.comm_buf.recv_buf = self.send[s0:s1], self.recv[r0:r1]
+            if not self.quantized:
                 continue
-            gr = graphs[r]
-            r_off = _cumulative(gr.comm_splits.recv_splits)
-            assert gr.comm_splits.recv_splits[p] == n
-            if not quantized:
-                a = gp.comm_buf.send_buf[s_off[r]:s_off[r + 1]]
-                b = gr.comm_buf.recv_buf[r_off[p]:r_off[p + 1]]
-                (b.copy_(a) if direction == "forward" else a.copy_(b))
-                continue
-            r_off_q = _cumulative(gr.comm_splits.recv_splits_int2)
-            qp, qr = gp.comm_buf_for_quantization, gr.comm_buf_for_quantization
-            da = qp.quantized_send_data_buf[s_off_q[r]:s_off_q[r + 1]]
-            db = qr.quantized_recv_data_buf[r_off_q[p]:r_off_q[p + 1]]
-            pa = qp.quantized_send_params_buf_fp32[s_off[r]:s_off[r + 1]]
-            pb = qr.quantized_recv_params_buf_fp32[r_off[p]:r_off[p + 1]]
-            src_d, dst_d, src_p, dst_p = (da, db, pa, pb) if direction == "forward" else (db, da, pb, pa)
-            dst_d.copy_(src_d)
-            if params_wire_dtype is not None:  # the reference ships params as bf16 (communicator.py:283-294)
-                dst_p.copy_(src_p.to(params_wire_dtype).to(torch.float32))
+            q = g.comm_buf_for_quantization
+            q.quantized_send_data_buf = self.send_q[self.qs_tot[p]:self.qs_tot[p + 1]]
+            q.quantized_recv_data_buf = self.recv_q[self.qr_tot[p]:self.qr_tot[p + 1]]
+            q.send_params, q.recv_params = self.send_params[s0:s1], self.recv_params[r0:r1]
+            if self.params_dtype == torch.float32:
+                q.quantized_send_params_buf_fp32, q.quantized_recv_params_buf_fp32 = q.send_params, q.recv_params
             else:
-                dst_p.copy_(src_p)
+                q.quantized_send_params_buf_bf16, q.quantized_recv_params_buf_bf16 = q.send_params, q.recv_params
+
+    @staticmethod
+    def _permutation(graphs, send_name, recv_name, send_tot, recv_tot, device):
+        """perm[j] = row of the send arena that lands in row j of the recv arena (all_to_all_single
+        semantics: rank p's segment for r becomes rank r's segment from p)."""
+        P = len(graphs)
+        perm = torch.empty(recv_tot[-1], dtype=torch.int64)
+        send_cum = [_cumulative(getattr(g.comm_splits, send_name)) for g in graphs]
+        for r, g in enumerate(graphs):
+            recv_cum = _cumulative(getattr(g.comm_splits, recv_name))
+            for p in range(P):
+                n = recv_cum[p + 1] - recv_cum[p]
+                assert n == send_cum[p][r + 1] - send_cum[p][r]
+                if n:
+                    begin = send_tot[p] + send_cum[p][r]
+                    perm[recv_tot[r] + recv_cum[p]:recv_tot[r] + recv_cum[p + 1]] = torch.arange(begin, begin + n)
+        return perm.to(device)
+
+    def exchange(self, direction, quantized):
+        if direction == "forward":
+            if quantized:
+                torch.index_select(self.send_q, 0, self.perm_q, out=self.recv_q)
+                torch.index_select(self.send_params_w, 0, self.perm, out=self.recv_params_w)
+            else:
+                torch.index_select(self.send, 0, self.perm, out=self.recv)
+        else:  # the same buffers with the roles swapped (aggregator.py:113-118,153-166)
+            if quantized:
+                torch.index_select(self.recv_q, 0, self.inv_perm_q, out=self.send_q)
+                torch.index_select(self.recv_params_w, 0, self.inv_perm, out=self.send_params_w)
+            else:
+                torch.index_select(self.recv, 0, self.inv_perm, out=self.send)
+
+
+def _scatter_matrix(g, n_local):
+    """0/1 matrix S[n_local, n_send] with S[idx[i], i] = 1, so that ``S @ rows`` is
+    ``index_add_(0, idx, rows)`` (aggregator.py:173-175) summed in index order without atomics."""
+    m = getattr(g, "_scatter_adj_t", None)
+    if m is None:
+        idx = g.idx_nodes_send_to_others
+        m = SparseTensor(row=idx.cpu(), col=torch.arange(idx.numel()), value=torch.ones(idx.numel()),
+                         sparse_sizes=(n_local, idx.numel())).to(idx.device)
+        g._scatter_adj_t = m
+    return m
 
 
 class LoopbackAggregator(torch.autograd.Function):
@@ -76,40 +143,47 @@ class LoopbackAggregator(torch.autograd.Function):
         graphs, bits, pre = world.graphs, world.num_bits, world.is_pre_delay
         quantized = bits in (2, 4, 8)
         F = feats[0].shape[-1]
+        arena = world.arena(F, feats[0].device)
         qz = Quantizer_for_all_procs(len(graphs), bits) if quantized else None
-        for g, x in zip(graphs, feats):
-            g.comm_buf.resize_buffer(g.comm_splits, F, bits)
-            if quantized:
-                g.comm_buf_for_quantization.resize_buffer(g.comm_splits, F, bits)
-            send_buf = g.comm_buf.send_buf
-            send_buf.zero_()                                              # aggregator.py:41
-            if send_buf.shape[0]:
+        fused = quantized and F % 4 == 0
+        feats = [x.contiguous() for x in feats]
+        main = torch.cuda.current_stream()
+        side = world.side_stream(feats[0].device)
+        side.wait_stream(main)
+        with torch.cuda.stream(side):                                     # send-side chain + exchange
+            for g, x in zip(graphs, feats):
+                send_buf = g.comm_buf.send_buf
+                if not send_buf.shape[0]:
+                    continue
+                q = g.comm_buf_for_quantization
                 if pre:
-                    SPMM_forward(g.adj_t_pre_post_aggr_to, x, send_buf)   # aggregator.py:46
-                else:
+                    SPMM_forward(g.adj_t_pre_post_aggr_to, x, send_buf, accumulate=False)   # aggregator.py:41,46
+                elif not quantized:
                     torch.index_select(x, 0, g.idx_nodes_send_to_others, out=send_buf)   # aggregator.py:48
                 if quantized:                                             # communicator.py:269
-                    q = g.comm_buf_for_quantization
-                    qz.quantize_fp32_to_intX(send_buf, q.quantized_send_data_buf, q.quantized_send_params_buf_fp32,
-                                             q.quantized_work_range_per_proc)
-        _exchange(graphs, "forward", quantized, world.params_wire_dtype)
+                    qz.quantize_fp32_to_intX(x if not pre else send_buf, q.quantized_send_data_buf, q.send_params,
+                                             q.quantized_work_range_per_proc,
+                                             row_index=None if pre else g.idx_nodes_send_to_others)
+            arena.exchange("forward", quantized)
         outs = []
-        for g, x in zip(graphs, feats):
-            out = torch.zeros((g.local_adj_t.sparse_size(0), F), dtype=torch.float32, device=x.device)
-            SPMM_forward(g.local_adj_t, x, out)                           # aggregator.py:62-65
-            remote = g.adj_t_pre_post_aggr_from if pre else g.remote_adj_t
-            if remote.sparse_size(1):
-                if quantized and F % 4 == 0:
-                    q = g.comm_buf_for_quantization                       # fused: aggregator.py:72-93 in one pass
-                    SPMM_forward_quantized(remote, q.quantized_recv_data_buf, q.quantized_recv_params_buf_fp32,
-                                           q.dequantized_work_range_per_proc, bits, out)
-                else:
-                    if quantized:
-                        q = g.comm_buf_for_quantization
-                        qz.dequantize_intX_to_fp32(q.quantized_recv_data_buf, g.comm_buf.recv_buf,
-                                                   q.quantized_recv_params_buf_fp32, q.dequantized_work_range_per_proc)
-                    SPMM_forward(remote, g.comm_buf.recv_buf, out)         # aggregator.py:90/92
+        for g, x in zip(graphs, feats):                                   # overlaps the chain above
+            out = torch.empty((g.local_adj_t.sparse_size(0), F), dtype=torch.float32, device=x.device)
+            SPMM_forward(g.local_adj_t, x, out, accumulate=False)         # aggregator.py:57,62-65
             outs.append(out)
+        main.wait_stream(side)
+        for g, out in zip(graphs, outs):
+            remote = g.adj_t_pre_post_aggr_from if pre else g.remote_adj_t
+            if not remote.sparse_size(1):
+                continue
+            q = g.comm_buf_for_quantization
+            if fused:                                                     # aggregator.py:72-93 in one pass
+                SPMM_forward_quantized(remote, q.quantized_recv_data_buf, q.recv_params,
+                                       q.dequantized_work_range_per_proc, bits, out)
+            else:
+                if quantized:
+                    qz.dequantize_intX_to_fp32(q.quantized_recv_data_buf, g.comm_buf.recv_buf, q.recv_params,
+                                               q.dequantized_work_range_per_proc)
+                SPMM_forward(remote, g.comm_buf.recv_buf, out)             # aggregator.py:90/92
         ctx.world = world
         return tuple(outs)
 
@@ -119,51 +193,88 @@ class LoopbackAggregator(torch.autograd.Function):
         graphs, bits, pre = world.graphs, world.num_bits, world.is_pre_delay
         quantized = bits in (2, 4, 8)
         F = grads[0].shape[-1]
+        arena = world.arena(F, grads[0].device)
         qz = Quantizer_for_all_procs(len(graphs), bits) if quantized else None
-        for g, go in zip(graphs, grads):
-            go = go.contiguous()
-            g.comm_buf.resize_buffer(g.comm_splits, F, bits)
-            if quantized:
-                g.comm_buf_for_quantization.resize_buffer(g.comm_splits, F, bits)
-            recv_buf = g.comm_buf.recv_buf
-            recv_buf.zero_()                                              # aggregator.py:122
-            if recv_buf.shape[0]:
+        fused = quantized and F % 4 == 0
+        grads = [go.contiguous() for go in grads]
+        main = torch.cuda.current_stream()
+        side = world.side_stream(grads[0].device)
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            for g, go in zip(graphs, grads):
+                recv_buf = g.comm_buf.recv_buf
+                if not recv_buf.shape[0]:
+                    continue
                 remote = g.adj_t_pre_post_aggr_from if pre else g.remote_adj_t
-                SPMM_backward(remote, go, recv_buf)                       # aggregator.py:125/127
+                SPMM_backward(remote, go, recv_buf, accumulate=False)     # aggregator.py:122,125/127
                 if quantized:                                             # the reverse trip is quantized too
                     q = g.comm_buf_for_quantization
-                    qz.quantize_fp32_to_intX(recv_buf, q.quantized_recv_data_buf, q.quantized_recv_params_buf_fp32,
+                    qz.quantize_fp32_to_intX(recv_buf, q.quantized_recv_data_buf, q.recv_params,
                                              q.dequantized_work_range_per_proc)
-        _exchange(graphs, "backward", quantized, world.params_wire_dtype)
+            arena.exchange("backward", quantized)
         outs = []
         for g, go in zip(graphs, grads):
-            go = go.contiguous()
-            local_grad = torch.zeros((g.local_adj_t.sparse_size(1), F), dtype=torch.float32, device=go.device)
-            SPMM_backward(g.local_adj_t, go, local_grad)                  # aggregator.py:145-148
-            send_buf = g.comm_buf.send_buf
-            if send_buf.shape[0]:
-                if quantized:                                             # aggregator.py:159-164
-                    q = g.comm_buf_for_quantization
-                    qz.dequantize_intX_to_fp32(q.quantized_send_data_buf, send_buf, q.quantized_send_params_buf_fp32,
-                                               q.quantized_work_range_per_proc)
-                if pre:
-                    SPMM_backward(g.adj_t_pre_post_aggr_to, send_buf, local_grad)          # aggregator.py:171
-                else:
-                    local_grad.index_add_(0, g.idx_nodes_send_to_others, send_buf)           # aggregator.py:173-175
+            local_grad = torch.empty((g.local_adj_t.sparse_size(1), F), dtype=torch.float32, device=go.device)
+            SPMM_backward(g.local_adj_t, go, local_grad, accumulate=False)   # aggregator.py:140,145-148
             outs.append(local_grad)
+        main.wait_stream(side)
+        for g, local_grad in zip(graphs, outs):
+            send_buf = g.comm_buf.send_buf
+            if not send_buf.shape[0]:
+                continue
+            q = g.comm_buf_for_quantization
+            if quantized and not fused:                                   # aggregator.py:159-164
+                qz.dequantize_intX_to_fp32(q.quantized_send_data_buf, send_buf, q.send_params,
+                                           q.quantized_work_range_per_proc)
+            if pre:                                                       # aggregator.py:171
+                if fused:
+                    SPMM_backward_quantized(g.adj_t_pre_post_aggr_to, q.quantized_send_data_buf, q.send_params,
+                                            q.quantized_work_range_per_proc, bits, local_grad)
+                else:
+                    SPMM_backward(g.adj_t_pre_post_aggr_to, send_buf, local_grad)
+            else:                                                         # aggregator.py:173-175
+                scatter = _scatter_matrix(g, local_grad.shape[0])
+                if fused:
+                    SPMM_forward_quantized(scatter, q.quantized_send_data_buf, q.send_params,
+                                           q.quantized_work_range_per_proc, bits, local_grad)
+                else:
+                    SPMM_forward(scatter, send_buf, local_grad)
         return (None,) + tuple(outs)
 
 
 class LoopbackWorld(object):
     """The P partitions of one graph plus the aggregation settings the reference passes per call
-    (num_bits, is_pre_delay).  ``params_wire_dtype=torch.bfloat16`` reproduces the reference's bf16
-    transport of (zero_point, scale) (communicator.py:283-294); None keeps them fp32."""
+    (num_bits, is_pre_delay).  ``params_wire_dtype=torch.bfloat16`` keeps (zero_point, scale) in the
+    reference's bf16 wire format (communicator.py:283-294) from the quantizer to the consumer; None
+    keeps them fp32."""
 
     def __init__(self, graphs: Sequence[object], num_bits: int, is_pre_delay: bool, params_wire_dtype=None) -> None:
         self.graphs = list(graphs)
         self.num_bits = int(num_bits)
         self.is_pre_delay = bool(is_pre_delay)
+        if params_wire_dtype not in (None, torch.float32, torch.bfloat16):
+            raise ValueError("params_wire_dtype must be None, torch.float32 or torch.bfloat16")
         self.params_wire_dtype = params_wire_dtype
+        self._arenas = {}
+        self._current = None
+        self._side = None
+
+    def arena(self, F, device):
+        """Buffers are kept per feature width; the partitions' buffer attributes are views of the
+        arena requested last (a layer sequence that alternates widths switches views)."""
+        a = self._arenas.get(F)
+        if a is None:
+            a = _Arena(self.graphs, F, self.num_bits in (2, 4, 8), self.params_wire_dtype or torch.float32, device)
+            self._arenas[F] = a
+        if self._current is not a:
+            a.bind(self.graphs)
+            self._current = a
+        return a
+
+    def side_stream(self, device):
+        if self._side is None:
+            self._side = torch.cuda.Stream(device=device)   # default priority
+        return self._side
 
     def aggregate(self, feats: Sequence[torch.Tensor]) -> List[torch.Tensor]:
         return list(LoopbackAggregator.apply(self, *feats))

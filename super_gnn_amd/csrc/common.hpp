@@ -95,6 +95,56 @@ __device__ __forceinline__ void vec_load(float (&r)[VEC], const float *p) {
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Operands of the quantize / dequantize kernels as they sit either side of the boundary exchange.
+// ------------------------------------------------------------------------------------------------
+
+// fp32 rows to quantize: row r is x[(index ? index[r] : r) * ld ...].  With an index the kernel
+// gathers the boundary rows straight out of the feature matrix (the reference first copies them into
+// send_buf, super_gnn/aggregator.py:48).  An index outside [0, n_src) reads row 0 instead of faulting.
+struct RowSrc {
+    const float *x;
+    int64_t ld;
+    const int64_t *index;
+    int64_t n_src;
+};
+__device__ __forceinline__ const float *row_ptr(const RowSrc &s, int64_t r) {
+    if (s.index) {
+        r = s.index[r];
+        if ((uint64_t)r >= (uint64_t)s.n_src) r = 0;
+    }
+    return s.x + r * s.ld;
+}
+
+// (zero_point, scale) per row, either fp32[n,2] or -- the form the reference puts on the wire,
+// super_gnn/communicator.py:283-294 -- bf16[n,2].  Codes are always computed from the fp32 values;
+// the bf16 form only changes what is stored and what the receiver multiplies by.
+struct ParamBuf {
+    void *p;
+    int bf16;
+};
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {  // round to nearest even, NaN -> quiet NaN
+    const uint32_t u = __float_as_uint(f);
+    if (f != f) return 0x7fc0u | ((u >> 16) & 0x8000u);
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ void store_params(const ParamBuf &b, int64_t row, float zp, float sc) {
+    if (b.bf16) reinterpret_cast<uint32_t *>(b.p)[row] = f32_to_bf16_bits(zp) | (f32_to_bf16_bits(sc) << 16);
+    else reinterpret_cast<float2 *>(b.p)[row] = make_float2(zp, sc);
+}
+template <bool BF16>
+__device__ __forceinline__ float2 load_params_as(const void *p, int64_t row) {
+    if constexpr (BF16) {
+        const uint32_t w = reinterpret_cast<const uint32_t *>(p)[row];
+        return make_float2(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u));
+    } else {
+        return reinterpret_cast<const float2 *>(p)[row];
+    }
+}
+__device__ __forceinline__ float2 load_params(const ParamBuf &b, int64_t row) {
+    return b.bf16 ? load_params_as<true>(b.p, row) : load_params_as<false>(b.p, row);
+}
+
 template <int VEC>
 __device__ __forceinline__ void vec_load_nt(float (&r)[VEC], const float *p) {
     if constexpr (VEC == 4) {

@@ -101,7 +101,7 @@ __device__ __forceinline__ uint32_t quant_code(float x, float zp, float sc) {
 // ------------------------------------------------------------------------------------------------
 template <int BITS, int VEC, int G, int NV, bool kForceExactDivision>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
-    const float *__restrict__ x, uint8_t *__restrict__ q, float *__restrict__ params,
+    const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
     constexpr int EPB = 8 / BITS;
     constexpr int R = kRowsPerGroup;
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (!valid[r]) continue;
-        const float *xr = x + row[r] * F;
+        const float *xr = row_ptr(xs, row[r]);
 #pragma unroll
         for (int v = 0; v < NV; ++v)
             if (act[v]) vec_load_nt<VEC>(xv[r][v], xr + off[v]);
@@ -193,7 +193,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
         if (s == 0.0f) s = 1.0f;
         zp[r] = mn;
         sc[r] = s;
-        if (lig == 0) *reinterpret_cast<float2 *>(params + row[r] * 2) = make_float2(mn, s);
+        if (lig == 0) store_params(pb, row[r], mn, s);
     }
 
     // Codes.  The reference's code is RNE(RN((x - zp) / scale)).  A correctly rounded fp32 division
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
 // ------------------------------------------------------------------------------------------------
 template <int BITS, int NV, int RL, bool kForceExactDivision>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
-    const float *__restrict__ x, uint8_t *__restrict__ q, float *__restrict__ params,
+    const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
     constexpr int EPB = 8 / BITS;
     constexpr int VEC = 4;
@@ -319,7 +319,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
 #pragma unroll
     for (int rl = 0; rl < RL; ++rl) {
         if (!valid[rl]) continue;
-        const float *xr = x + row[rl] * F;
+        const float *xr = row_ptr(xs, row[rl]);
 #pragma unroll
         for (int v = 0; v < NV; ++v)
             if (act[v]) vec_load_nt<VEC>(xv[rl][v], xr + off[v]);
@@ -372,7 +372,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
         sc[rl] = s;
         rinv[rl] = __builtin_amdgcn_rcpf(s);  // hardware reciprocal, within 1 ulp of 1/s
         if (!(s >= 0x1p-100f && s <= 0x1p100f)) lane_exact = true;
-        if (l16 == 0) *reinterpret_cast<float2 *>(params + row[rl] * 2) = make_float2(mn, s);
+        if (l16 == 0) store_params(pb, row[rl], mn, s);
     }
 
     // Codes.  The reference's code is RNE(RN((x - zp) / scale)).  The quotient is first formed as
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
 // ------------------------------------------------------------------------------------------------
 template <int BITS, int VEC, int G, int NV>
 __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_kernel(
-    const uint8_t *__restrict__ q, float *__restrict__ x, const float *__restrict__ params,
+    const uint8_t *__restrict__ q, float *__restrict__ x, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
     constexpr int EPB = 8 / BITS;
     constexpr int R = kRowsPerGroup;
@@ -460,7 +460,7 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_kernel(
             zp[k] = 0.0f;
             sc[k] = 0.0f;
             if (row0 + k < rend) {
-                const float2 ps = *reinterpret_cast<const float2 *>(params + (row0 + k) * 2);
+                const float2 ps = load_params(pb, row0 + k);
                 zp[k] = ps.x;
                 sc[k] = ps.y;
             }
@@ -495,7 +495,7 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_kernel(
 // ------------------------------------------------------------------------------------------------
 template <int BITS, int NV, int RL>
 __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows16_kernel(
-    const uint8_t *__restrict__ q, float *__restrict__ x, const float *__restrict__ params,
+    const uint8_t *__restrict__ q, float *__restrict__ x, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
     constexpr int EPB = 8 / BITS;
     constexpr int VEC = 4;
@@ -522,7 +522,7 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows16_kernel(
             valid[rl] = row[rl] < seg[p + 1];
         }
         if (valid[rl]) {
-            ps[rl] = *reinterpret_cast<const float2 *>(params + row[rl] * 2);
+            ps[rl] = load_params(pb, row[rl]);
             const uint8_t *qr = q + (int64_t)g * F;
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
@@ -553,7 +553,7 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows16_kernel(
 // ------------------------------------------------------------------------------------------------
 template <int BITS>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows_wide_kernel(
-    const float *__restrict__ x, uint8_t *__restrict__ q, float *__restrict__ params,
+    const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F) {
     constexpr int EPB = 8 / BITS;
     const int lane = threadIdx.x & 63;
@@ -568,7 +568,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_wide_kernel(
         zp[k] = 0.0f;
         sc[k] = 1.0f;
         if (row0 + k >= rend) continue;
-        const float *xr = x + (row0 + k) * F;
+        const float *xr = row_ptr(xs, row0 + k);
         float mn = INFINITY, mx = -INFINITY;
         int key = INT_MAX;
         for (int j = lane; j < F; j += 64) {
@@ -589,21 +589,21 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_wide_kernel(
         if (s == 0.0f) s = 1.0f;
         zp[k] = mn;
         sc[k] = s;
-        if (lane == 0) { params[(row0 + k) * 2] = mn; params[(row0 + k) * 2 + 1] = s; }
+        if (lane == 0) store_params(pb, row0 + k, mn, s);
     }
     uint8_t *qr = q + (int64_t)gp * F;
     for (int j = lane; j < F; j += 64) {
         uint32_t byte = 0;
 #pragma unroll
         for (int k = 0; k < EPB; ++k)
-            if (row0 + k < rend) byte |= quant_code(x[(row0 + k) * F + j], zp[k], sc[k]) << ((EPB - 1 - k) * BITS);
+            if (row0 + k < rend) byte |= quant_code(row_ptr(xs, row0 + k)[j], zp[k], sc[k]) << ((EPB - 1 - k) * BITS);
         qr[j] = (uint8_t)byte;
     }
 }
 
 template <int BITS>
 __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_wide_kernel(
-    const uint8_t *__restrict__ q, float *__restrict__ x, const float *__restrict__ params,
+    const uint8_t *__restrict__ q, float *__restrict__ x, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F) {
     constexpr int EPB = 8 / BITS;
     constexpr uint32_t MASK = (1u << BITS) - 1u;
@@ -617,7 +617,8 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_wide_kernel(
 #pragma unroll
     for (int k = 0; k < EPB; ++k) {
         if (row0 + k >= rend) continue;
-        const float zp = params[(row0 + k) * 2], sc = params[(row0 + k) * 2 + 1];
+        const float2 ps = load_params(pb, row0 + k);
+        const float zp = ps.x, sc = ps.y;
         for (int j = lane; j < F; j += 64)
             x[(row0 + k) * F + j] = fmaf((float)((qr[j] >> ((EPB - 1 - k) * BITS)) & MASK), sc, zp);
     }
@@ -707,8 +708,9 @@ __global__ __launch_bounds__(kQBlock) void row_slots_kernel(const int32_t *__res
 // Launch tables.
 // ------------------------------------------------------------------------------------------------
 struct RowsArgs {
-    const float *x_in; uint8_t *q_out; float *params_out;            // quantize
-    const uint8_t *q_in; float *x_out; const float *params_in;        // dequantize
+    RowSrc x_in; uint8_t *q_out;                                     // quantize
+    const uint8_t *q_in; float *x_out;                               // dequantize
+    ParamBuf params;                                                 // written by quantize, read by dequantize
     const int32_t *seg; const int32_t *pseg; int P; int n_packed; int F; bool quantize;
     bool layout16;        // diagnostic switch: one fp32 row per 16 lanes (default) vs per lane group
     bool exact_division;  // diagnostic: IEEE division for every element (the results are identical either way)
@@ -723,13 +725,13 @@ static void launch_rows(const RowsArgs &a, hipStream_t st) {
     ProfScope prof(a.quantize ? K_QUANT_PACK_ROWS : K_UNPACK_DEQUANT_ROWS, st);
     if (a.quantize && a.exact_division)
         hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
-                           a.q_out, a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                           a.q_out, a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
     else if (a.quantize)
         hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV, false>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
-                           a.q_out, a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                           a.q_out, a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
     else
         hipLaunchKernelGGL((unpack_dequant_rows_kernel<BITS, VEC, G, NV>), dim3(nb), dim3(kQBlock), 0, st, a.q_in,
-                           a.x_out, a.params_in, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                           a.x_out, a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
 }
 
 template <int BITS, int NV>
@@ -742,10 +744,10 @@ static void launch_quant16(const RowsArgs &a, hipStream_t st) {
     ProfScope prof(K_QUANT_PACK_ROWS, st);
     if (a.exact_division)
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
-                           a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                           a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
     else
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
-                           a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                           a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
 }
 
 template <int BITS, int NV>
@@ -757,7 +759,7 @@ static void launch_dequant16(const RowsArgs &a, hipStream_t st) {
     const int nb = (n_units + kQBlock / 64 - 1) / (kQBlock / 64);
     ProfScope prof(K_UNPACK_DEQUANT_ROWS, st);
     hipLaunchKernelGGL((unpack_dequant_rows16_kernel<BITS, NV, RL>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, a.x_out,
-                       a.params_in, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                       a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
 }
 
 template <int BITS>
@@ -766,10 +768,10 @@ static void launch_rows_wide(const RowsArgs &a, hipStream_t st) {
     ProfScope prof(a.quantize ? K_QUANT_PACK_ROWS : K_UNPACK_DEQUANT_ROWS, st);
     if (a.quantize)
         hipLaunchKernelGGL((quant_pack_rows_wide_kernel<BITS>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
-                           a.params_out, a.seg, a.pseg, a.P, a.n_packed, a.F);
+                           a.params, a.seg, a.pseg, a.P, a.n_packed, a.F);
     else
         hipLaunchKernelGGL((unpack_dequant_rows_wide_kernel<BITS>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, a.x_out,
-                           a.params_in, a.seg, a.pseg, a.P, a.n_packed, a.F);
+                           a.params, a.seg, a.pseg, a.P, a.n_packed, a.F);
 }
 
 template <int BITS, int VEC>
@@ -821,13 +823,13 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
     SGNN_REQUIRE(n_rows >= 0 && a.n_packed >= 0, "negative row count");
     if (n_rows == 0 || a.n_packed == 0) return SGNN_OK;
     SGNN_REQUIRE(fp32_ptr && u8_ptr && a.seg && a.pseg, "null pointer argument");
-    SGNN_REQUIRE(a.quantize ? a.params_out != nullptr : a.params_in != nullptr, "params is null");
+    SGNN_REQUIRE(a.params.p != nullptr, "params is null");
     SGNN_REQUIRE((int64_t)a.n_packed * (8 / bits) < (int64_t)INT32_MAX, "too many rows for 32-bit row units");
+    const int64_t ld = a.quantize ? a.x_in.ld : (int64_t)a.F;
     int vec = 1;
-    if (a.F % 4 == 0 && aligned(fp32_ptr, 16) && aligned(u8_ptr, 4)) vec = 4;
-    else if (a.F % 2 == 0 && aligned(fp32_ptr, 8) && aligned(u8_ptr, 2)) vec = 2;
-    const void *pp = a.quantize ? (const void *)a.params_out : (const void *)a.params_in;
-    SGNN_REQUIRE(aligned(pp, 8), "params must be 8-byte aligned");
+    if (a.F % 4 == 0 && ld % 4 == 0 && aligned(fp32_ptr, 16) && aligned(u8_ptr, 4)) vec = 4;
+    else if (a.F % 2 == 0 && ld % 2 == 0 && aligned(fp32_ptr, 8) && aligned(u8_ptr, 2)) vec = 2;
+    SGNN_REQUIRE(aligned(a.params.p, a.params.bf16 ? 4 : 8), "params must be %d-byte aligned", a.params.bf16 ? 4 : 8);
     if (bits == 8) dispatch_rows<8>(vec, a, st);
     else if (bits == 4) dispatch_rows<4>(vec, a, st);
     else dispatch_rows<2>(vec, a, st);
@@ -869,27 +871,58 @@ extern "C" int sgnn_quant_row_slots(const int32_t *seg, const int32_t *pseg, int
     return SGNN_OK;
 }
 
-extern "C" int sgnn_quant_pack_rows_f32(const float *x, uint8_t *q, float *params, const int32_t *seg,
-                                        const int32_t *pseg, int P, int64_t n_rows, int64_t n_packed_rows,
-                                        int64_t F, int bits, sgnn_stream_t stream) {
+static int quant_pack_rows_impl(const RowSrc &src, uint8_t *q, void *params, int params_bf16, const int32_t *seg,
+                                const int32_t *pseg, int P, int64_t n_rows, int64_t n_packed_rows, int64_t F, int bits,
+                                sgnn_stream_t stream) {
     SGNN_REQUIRE(F > 0 && F < (1 << 24) && n_packed_rows < INT32_MAX, "size out of range");
+    SGNN_REQUIRE(src.ld >= F, "row stride %lld is smaller than the feature width %lld", (long long)src.ld, (long long)F);
+    SGNN_REQUIRE(src.index == nullptr || src.n_src > 0 || n_rows == 0, "row index given but the source has no rows");
+    SGNN_REQUIRE(params_bf16 == 0 || params_bf16 == 1, "params_bf16=%d, expected 0 or 1", params_bf16);
     RowsArgs a{};
-    a.x_in = x; a.q_out = q; a.params_out = params; a.seg = seg; a.pseg = pseg; a.P = P;
+    a.x_in = src; a.q_out = q; a.params = ParamBuf{params, params_bf16}; a.seg = seg; a.pseg = pseg; a.P = P;
     a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = true;
     { const char *e = getenv("SGNN_QUANT_EXACT_DIV"); a.exact_division = e && e[0] == '1'; }
     { const char *e = getenv("SGNN_QUANT_LAYOUT16"); a.layout16 = !(e && e[0] == '0'); }
+    return run_rows(a, bits, n_rows, src.x, q, (hipStream_t)stream);
+}
+
+static int unpack_dequant_rows_impl(const uint8_t *q, float *x, const void *params, int params_bf16,
+                                    const int32_t *seg, const int32_t *pseg, int P, int64_t n_rows,
+                                    int64_t n_packed_rows, int64_t F, int bits, sgnn_stream_t stream) {
+    SGNN_REQUIRE(F > 0 && F < (1 << 24) && n_packed_rows < INT32_MAX, "size out of range");
+    SGNN_REQUIRE(params_bf16 == 0 || params_bf16 == 1, "params_bf16=%d, expected 0 or 1", params_bf16);
+    RowsArgs a{};
+    a.q_in = q; a.x_out = x; a.params = ParamBuf{const_cast<void *>(params), params_bf16}; a.seg = seg; a.pseg = pseg;
+    a.P = P; a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = false;
+    { const char *e = getenv("SGNN_QUANT_LAYOUT16"); a.layout16 = !(e && e[0] == '0'); }
     return run_rows(a, bits, n_rows, x, q, (hipStream_t)stream);
+}
+
+extern "C" int sgnn_quant_pack_rows_f32(const float *x, uint8_t *q, float *params, const int32_t *seg,
+                                        const int32_t *pseg, int P, int64_t n_rows, int64_t n_packed_rows,
+                                        int64_t F, int bits, sgnn_stream_t stream) {
+    return quant_pack_rows_impl(RowSrc{x, F, nullptr, n_rows}, q, params, 0, seg, pseg, P, n_rows, n_packed_rows, F,
+                                bits, stream);
+}
+
+extern "C" int sgnn_quant_pack_rows_wire_f32(const float *x, int64_t ldx, const int64_t *row_index, int64_t n_src_rows,
+                                             uint8_t *q, void *params, int params_bf16, const int32_t *seg,
+                                             const int32_t *pseg, int P, int64_t n_rows, int64_t n_packed_rows,
+                                             int64_t F, int bits, sgnn_stream_t stream) {
+    return quant_pack_rows_impl(RowSrc{x, ldx, row_index, row_index ? n_src_rows : n_rows}, q, params, params_bf16,
+                                seg, pseg, P, n_rows, n_packed_rows, F, bits, stream);
 }
 
 extern "C" int sgnn_unpack_dequant_rows_f32(const uint8_t *q, float *x, const float *params, const int32_t *seg,
                                             const int32_t *pseg, int P, int64_t n_rows, int64_t n_packed_rows,
                                             int64_t F, int bits, sgnn_stream_t stream) {
-    SGNN_REQUIRE(F > 0 && F < (1 << 24) && n_packed_rows < INT32_MAX, "size out of range");
-    RowsArgs a{};
-    a.q_in = q; a.x_out = x; a.params_in = params; a.seg = seg; a.pseg = pseg; a.P = P;
-    a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = false;
-    { const char *e = getenv("SGNN_QUANT_LAYOUT16"); a.layout16 = !(e && e[0] == '0'); }
-    return run_rows(a, bits, n_rows, x, q, (hipStream_t)stream);
+    return unpack_dequant_rows_impl(q, x, params, 0, seg, pseg, P, n_rows, n_packed_rows, F, bits, stream);
+}
+
+extern "C" int sgnn_unpack_dequant_rows_wire_f32(const uint8_t *q, float *x, const void *params, int params_bf16,
+                                                 const int32_t *seg, const int32_t *pseg, int P, int64_t n_rows,
+                                                 int64_t n_packed_rows, int64_t F, int bits, sgnn_stream_t stream) {
+    return unpack_dequant_rows_impl(q, x, params, params_bf16, seg, pseg, P, n_rows, n_packed_rows, F, bits, stream);
 }
 
 extern "C" int sgnn_quant_v1_f32(const float *x, uint8_t *q, const int64_t *range, float *params, int64_t n,

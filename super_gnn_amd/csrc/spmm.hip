@@ -56,12 +56,15 @@ __device__ __forceinline__ int64_t uniform64(int64_t v) {
 }
 
 // The dense operand of the product: fp32 rows (BITS == 0), or rows that arrive quantized and
-// bit-packed in the row-group layout (BITS in {8, 4, 2}; see quant.hip) and are decoded on the fly.
+// bit-packed in the row-group layout (see quant.hip) and are decoded on the fly.  For those the
+// template parameter BITS is a format code: the low four bits are the code width (8, 4 or 2) and
+// kBf16Params is added when (zero_point, scale) are bf16 pairs instead of fp32 pairs.
+constexpr int kBf16Params = 16;
 struct DenseSrc {
     const float *x;        // fp32: [K, ldx]
     int64_t ldx;
     const uint8_t *q;      // quantized: packed rows of qF bytes
-    const float *params;   // quantized: (zero_point, scale) per dense row
+    ParamBuf params;       // quantized: (zero_point, scale) per dense row, fp32 or bf16 pairs
     const int32_t *slot;   // quantized: dense row -> index in the padded row space (null = identity)
     int qF;
 };
@@ -86,12 +89,13 @@ __device__ __forceinline__ void fetch_row(Fetched<VEC, NV, BITS> &r, const Dense
         for (int v = 0; v < NV; ++v)
             if (act[v]) vec_load<VEC>(r.f[v], xr + off[v]);
     } else {
-        constexpr int EPB = 8 / BITS;
+        constexpr int NB = BITS & 15;
+        constexpr int EPB = 8 / NB;
         const int sl = d.slot ? d.slot[c] : c;
-        const float2 ps = *reinterpret_cast<const float2 *>(d.params + (int64_t)c * 2);
+        const float2 ps = load_params_as<(BITS & kBf16Params) != 0>(d.params.p, c);
         r.zp = ps.x;
         r.sc = ps.y;
-        r.shift = (EPB - 1 - (sl % EPB)) * BITS;
+        r.shift = (EPB - 1 - (sl % EPB)) * NB;
         const uint8_t *qr = d.q + (int64_t)(sl / EPB) * d.qF;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
@@ -116,7 +120,7 @@ __device__ __forceinline__ void fma_row(float (&acc)[NV][VEC], float w, const Fe
             if constexpr (BITS == 0) {
                 xv = r.f[v][k];
             } else {
-                const uint32_t code = (r.w[v] >> (8 * k + r.shift)) & ((1u << BITS) - 1u);
+                const uint32_t code = (r.w[v] >> (8 * k + r.shift)) & ((1u << (BITS & 15)) - 1u);
                 xv = fmaf((float)code, r.sc, r.zp);
             }
             acc[v][k] = fmaf(w, xv, acc[v][k]);
@@ -952,7 +956,11 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     PieceArgs s{p->col_long, p->eperm, val, p->partial, p->item_begin, p->item_len, p->cls_list, p->cls_off,
                 p->max_cls_items, (int)F};
     FinalArgs f{p->long_rows, p->long_pbeg, p->partial, out, (int)p->n_long, (int)F, ldo, accumulate, row_div};
-    if (bits == 8) dispatch_shape_dq<8>(nvec, a, s, f, st);
+    if (bits != 0 && dense.params.bf16) {
+        if (bits == 8) dispatch_shape_dq<8 + kBf16Params>(nvec, a, s, f, st);
+        else if (bits == 4) dispatch_shape_dq<4 + kBf16Params>(nvec, a, s, f, st);
+        else dispatch_shape_dq<2 + kBf16Params>(nvec, a, s, f, st);
+    } else if (bits == 8) dispatch_shape_dq<8>(nvec, a, s, f, st);
     else if (bits == 4) dispatch_shape_dq<4>(nvec, a, s, f, st);
     else if (bits == 2) dispatch_shape_dq<2>(nvec, a, s, f, st);
     else if (vec == 4) dispatch_shape<4>(nvec, a, s, f, st);
@@ -968,18 +976,32 @@ extern "C" int sgnn_spmm_csr_f32(sgnn_spmm_plan *p, const float *val, const floa
     SGNN_REQUIRE(p != nullptr, "plan is null");
     SGNN_REQUIRE(ldx >= F, "leading dimension smaller than F (ldx=%lld F=%lld)", (long long)ldx, (long long)F);
     SGNN_REQUIRE(x != nullptr || p->nnz == 0 || p->M == 0, "x is null");
-    DenseSrc d{x, ldx, nullptr, nullptr, nullptr, 0};
+    DenseSrc d{x, ldx, nullptr, ParamBuf{nullptr, 0}, nullptr, 0};
     return spmm_run(p, val, d, 0, out, F, ldo, accumulate, row_div, (hipStream_t)stream);
+}
+
+static int spmm_dq_impl(sgnn_spmm_plan *p, const float *val, const uint8_t *q, const void *params, int params_bf16,
+                       const int32_t *row_slot, int bits, float *out, int64_t F, int64_t ldo, int accumulate,
+                       const float *row_div, sgnn_stream_t stream) {
+    SGNN_REQUIRE(p != nullptr, "plan is null");
+    SGNN_REQUIRE(bits == 8 || bits == 4 || bits == 2, "bits=%d, expected 8, 4 or 2", bits);
+    SGNN_REQUIRE(params_bf16 == 0 || params_bf16 == 1, "params_bf16=%d, expected 0 or 1", params_bf16);
+    SGNN_REQUIRE(F % 4 == 0, "the fused path needs F %% 4 == 0 (F=%lld): dequantize, then call sgnn_spmm_csr_f32", (long long)F);
+    SGNN_REQUIRE((q != nullptr && params != nullptr) || p->nnz == 0 || p->M == 0, "q / params is null");
+    SGNN_REQUIRE(aligned(q, 4) && aligned(params, params_bf16 ? 4 : 8), "q must be 4-byte and params %d-byte aligned",
+                 params_bf16 ? 4 : 8);
+    DenseSrc d{nullptr, 0, q, ParamBuf{const_cast<void *>(params), params_bf16}, row_slot, (int)F};
+    return spmm_run(p, val, d, bits, out, F, ldo, accumulate, row_div, (hipStream_t)stream);
 }
 
 extern "C" int sgnn_spmm_csr_dq_f32(sgnn_spmm_plan *p, const float *val, const uint8_t *q, const float *params,
                                     const int32_t *row_slot, int bits, float *out, int64_t F, int64_t ldo,
                                     int accumulate, const float *row_div, sgnn_stream_t stream) {
-    SGNN_REQUIRE(p != nullptr, "plan is null");
-    SGNN_REQUIRE(bits == 8 || bits == 4 || bits == 2, "bits=%d, expected 8, 4 or 2", bits);
-    SGNN_REQUIRE(F % 4 == 0, "the fused path needs F %% 4 == 0 (F=%lld): dequantize, then call sgnn_spmm_csr_f32", (long long)F);
-    SGNN_REQUIRE((q != nullptr && params != nullptr) || p->nnz == 0 || p->M == 0, "q / params is null");
-    SGNN_REQUIRE(aligned(q, 4) && aligned(params, 8), "q must be 4-byte and params 8-byte aligned");
-    DenseSrc d{nullptr, 0, q, params, row_slot, (int)F};
-    return spmm_run(p, val, d, bits, out, F, ldo, accumulate, row_div, (hipStream_t)stream);
+    return spmm_dq_impl(p, val, q, params, 0, row_slot, bits, out, F, ldo, accumulate, row_div, stream);
+}
+
+extern "C" int sgnn_spmm_csr_dq_wire_f32(sgnn_spmm_plan *p, const float *val, const uint8_t *q, const void *params,
+                                         int params_bf16, const int32_t *row_slot, int bits, float *out, int64_t F,
+                                         int64_t ldo, int accumulate, const float *row_div, sgnn_stream_t stream) {
+    return spmm_dq_impl(p, val, q, params, params_bf16, row_slot, bits, out, F, ldo, accumulate, row_div, stream);
 }

@@ -50,7 +50,10 @@ def disribute_work_for_col(other: torch.Tensor, num_threads_on_col: int) -> torc
     return col_splits
 
 
-def SPMM_forward(src, other: torch.Tensor, out: torch.Tensor) -> None:
+def SPMM_forward(src, other: torch.Tensor, out: torch.Tensor, accumulate=None) -> None:
+    """``accumulate=None`` follows the reference (out += A @ other except on its overwrite branch);
+    ``False`` writes out = A @ other, which equals zero-filling out and accumulating, bit for bit,
+    without the fill and the read-back."""
     rowptr, col, value = src.csr()
     col_splits = disribute_work_for_col(other, 1)
     row_splits, _ = src.get_work_range()
@@ -58,11 +61,11 @@ def SPMM_forward(src, other: torch.Tensor, out: torch.Tensor) -> None:
     if value is not None:
         value = value.to(other.dtype)
     sparse_row = rowptr.shape[0] - 1
-    spmm(rowptr, col, value, other, out, sparse_row, row_splits, col_splits, plan=src.spmm_plan())
+    spmm(rowptr, col, value, other, out, sparse_row, row_splits, col_splits, plan=src.spmm_plan(), accumulate=accumulate)
     return None
 
 
-def SPMM_backward(src, other: torch.Tensor, out: torch.Tensor) -> None:
+def SPMM_backward(src, other: torch.Tensor, out: torch.Tensor, accumulate=None) -> None:
     colptr = src.storage.colptr()
     row_T = src.storage.row_T()
     value_T = src.storage.value_T()
@@ -72,7 +75,8 @@ def SPMM_backward(src, other: torch.Tensor, out: torch.Tensor) -> None:
     if value_T is not None:
         value_T = value_T.to(other.dtype)
     sparse_row = colptr.shape[0] - 1
-    return spmm(colptr, row_T, value_T, other, out, sparse_row, row_splits, col_splits, plan=src.spmm_plan_T())
+    return spmm(colptr, row_T, value_T, other, out, sparse_row, row_splits, col_splits, plan=src.spmm_plan_T(),
+                accumulate=accumulate)
 
 
 def SPMM_forward_quantized(src, data_int8: torch.Tensor, quantized_params: torch.Tensor,
@@ -86,4 +90,18 @@ def SPMM_forward_quantized(src, data_int8: torch.Tensor, quantized_params: torch
         value = value.to(torch.float32)
     segs = quant_segments(work_range_per_proc, num_bits)
     src.spmm_plan().run_quantized(value, data_int8, quantized_params, segs, num_bits, out, accumulate=True)
+    return None
+
+
+def SPMM_backward_quantized(src, data_int8: torch.Tensor, quantized_params: torch.Tensor,
+                            work_range_per_proc: torch.Tensor, num_bits: int, out: torch.Tensor) -> None:
+    """out += A^T @ dequantize(data_int8): the last step of the backward pass in pre/post-aggregation
+    mode with the returned gradient rows still packed; replaces ``dequantize_intX_to_fp32(...)``
+    followed by ``SPMM_backward(adj_t_pre_post_aggr_to, send_buf, local_grad)``
+    (super_gnn/aggregator.py:159-171) and gives the same floats."""
+    value_T = src.storage.value_T()
+    if value_T is not None:
+        value_T = value_T.to(torch.float32)
+    segs = quant_segments(work_range_per_proc, num_bits)
+    src.spmm_plan_T().run_quantized(value_T, data_int8, quantized_params, segs, num_bits, out, accumulate=True)
     return None

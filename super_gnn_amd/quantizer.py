@@ -70,9 +70,13 @@ class Quantizer_for_all_procs(object):
         self.num_bits = num_bits
         type(self).ctx = self
 
-    def quantize_fp32_to_intX(self, data_fp32, data_int8, quantized_params, quantized_work_range_per_proc):
+    def quantize_fp32_to_intX(self, data_fp32, data_int8, quantized_params, quantized_work_range_per_proc,
+                              row_index=None):
+        """``quantized_params`` may be fp32 or bf16 pairs; with ``row_index`` the rows quantized are
+        ``data_fp32[row_index]`` (see supergnn_ops.quantize_tensor_for_all_procs)."""
         _ops.quantize_tensor_for_all_procs(
-            data_fp32, data_int8, quantized_params, quantized_work_range_per_proc, self.world_size, self.num_bits)
+            data_fp32, data_int8, quantized_params, quantized_work_range_per_proc, self.world_size, self.num_bits,
+            row_index=row_index)
 
     def dequantize_intX_to_fp32(self, data_int8, data_fp32, quantized_params, dequantized_work_range_per_proc):
         _ops.dequantize_tensor_for_all_procs(

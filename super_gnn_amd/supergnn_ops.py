@@ -148,7 +148,7 @@ class SpmmPlan:
         ``segs`` from quant_segments()) and is decoded inside the gather."""
         _check_bits(bits)
         _want(data_int8, torch.uint8, "data_int8")
-        _want(params, torch.float32, "quantized_params")
+        bf16 = _params_kind(params, "quantized_params")
         _want(out, torch.float32, "out")
         if value is not None:
             _want(value, torch.float32, "value")
@@ -170,8 +170,12 @@ class SpmmPlan:
         if row_div is not None:
             _want(row_div, torch.float32, "row_div")
         slots = segs.row_slots(bits)
-        check(lib.sgnn_spmm_csr_dq_f32(self._h, _ptr(value), _ptr(data_int8), _ptr(params), _ptr(slots), bits,
-                                       _ptr(out), F, F, int(bool(accumulate)), _ptr(row_div), _stream()))
+        if bf16:
+            check(lib.sgnn_spmm_csr_dq_wire_f32(self._h, _ptr(value), _ptr(data_int8), _ptr(params), 1, _ptr(slots), bits,
+                                                _ptr(out), F, F, int(bool(accumulate)), _ptr(row_div), _stream()))
+        else:
+            check(lib.sgnn_spmm_csr_dq_f32(self._h, _ptr(value), _ptr(data_int8), _ptr(params), _ptr(slots), bits,
+                                           _ptr(out), F, F, int(bool(accumulate)), _ptr(row_div), _stream()))
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
@@ -279,12 +283,37 @@ def _check_bits(bits):
         raise ValueError(f"bits={bits}: only 8, 4 and 2 pack into bytes")  # TORCH_CHECK(8 % bits == 0), quantization_arm.cpp:438
 
 
-def _quant_rows(inp, out_u8, params, segs, bits):
+def _params_kind(params, name):
+    """0 for fp32 (zero_point, scale) pairs, 1 for the bf16 pairs the reference puts on the wire
+    (super_gnn/communicator.py:283-294)."""
+    if params.dtype == torch.float32:
+        return 0
+    if params.dtype == torch.bfloat16:
+        return 1
+    raise TypeError(f"{name} must be torch.float32 or torch.bfloat16, got {params.dtype}")
+
+
+def _checked_row_index(row_index, n_src):
+    """An int64 GPU index tensor whose range has been checked once (cached on the tensor object)."""
+    _want(row_index, torch.int64, "row_index")
+    if row_index.dim() != 1 or not row_index.is_contiguous():
+        raise ValueError("row_index must be a contiguous 1-D tensor")
+    seen = row_index.__dict__.get("_sgnn_index_ok")
+    if seen != (row_index._version, int(n_src)):
+        if row_index.numel() and (int(row_index.min()) < 0 or int(row_index.max()) >= n_src):
+            raise IndexError(f"row_index out of range for a source of {n_src} rows")
+        row_index.__dict__["_sgnn_index_ok"] = (row_index._version, int(n_src))
+    return row_index
+
+
+def _quant_rows(inp, out_u8, params, segs, bits, row_index=None):
     _want(inp, torch.float32, "input")
     _want(out_u8, torch.uint8, "output")
-    _want(params, torch.float32, "quantized_params")
+    bf16 = _params_kind(params, "quantized_params")
     if inp.dim() != 2:
         raise ValueError("input must be [rows, features]")
+    if row_index is not None:
+        return _quant_gathered_rows(inp, row_index, out_u8, params, bf16, segs, bits)
     n, F = inp.shape
     if segs.n_rows != n:
         raise ValueError(f"segment table ends at row {segs.n_rows}, input has {n} rows")
@@ -296,16 +325,40 @@ def _quant_rows(inp, out_u8, params, segs, bits):
     s_in = _Staged(inp, dev)
     s_q = _Staged(out_u8, dev, writeback=True)
     s_p = _Staged(params, dev, writeback=True)
-    check(lib.sgnn_quant_pack_rows_f32(_ptr(s_in.dev), _ptr(s_q.dev), _ptr(s_p.dev), _ptr(segs.seg), _ptr(segs.pseg),
-                                       segs.P, n, segs.n_packed, F, bits, _stream()))
+    if bf16:
+        check(lib.sgnn_quant_pack_rows_wire_f32(_ptr(s_in.dev), F, None, n, _ptr(s_q.dev), _ptr(s_p.dev), 1, _ptr(segs.seg),
+                                                _ptr(segs.pseg), segs.P, n, segs.n_packed, F, bits, _stream()))
+    else:
+        check(lib.sgnn_quant_pack_rows_f32(_ptr(s_in.dev), _ptr(s_q.dev), _ptr(s_p.dev), _ptr(segs.seg), _ptr(segs.pseg),
+                                           segs.P, n, segs.n_packed, F, bits, _stream()))
     s_q.commit()
     s_p.commit()
+
+
+def _quant_gathered_rows(src, row_index, out_u8, params, bf16, segs, bits):
+    """Quantize rows src[row_index[r]] without materialising them (GPU tensors only)."""
+    if not (src.is_cuda and row_index.is_cuda and out_u8.is_cuda and params.is_cuda):
+        raise ValueError("the gathering quantizer takes GPU tensors only")
+    if src.stride(1) != 1 or not (out_u8.is_contiguous() and params.is_contiguous()):
+        raise ValueError("input rows must be dense (unit stride) and outputs contiguous")
+    n_src, F = src.shape
+    n = row_index.numel()
+    _checked_row_index(row_index, n_src)
+    if segs.n_rows != n:
+        raise ValueError(f"segment table ends at row {segs.n_rows}, row_index has {n} entries")
+    if out_u8.numel() < segs.n_packed * F:
+        raise ValueError(f"output holds {out_u8.numel()} bytes, {segs.n_packed * F} needed")
+    if params.numel() < n * 2:
+        raise ValueError(f"quantized_params holds {params.numel()} elements, {n * 2} needed")
+    check(lib.sgnn_quant_pack_rows_wire_f32(_ptr(src), src.stride(0), _ptr(row_index), n_src, _ptr(out_u8), _ptr(params),
+                                            bf16, _ptr(segs.seg), _ptr(segs.pseg), segs.P, n, segs.n_packed, F, bits,
+                                            _stream()))
 
 
 def _dequant_rows(inp_u8, out, params, segs, bits):
     _want(inp_u8, torch.uint8, "input")
     _want(out, torch.float32, "output")
-    _want(params, torch.float32, "dequantized_params")
+    bf16 = _params_kind(params, "dequantized_params")
     if out.dim() != 2:
         raise ValueError("output must be [rows, features]")
     n, F = out.shape
@@ -319,8 +372,12 @@ def _dequant_rows(inp_u8, out, params, segs, bits):
     s_q = _Staged(inp_u8, dev)
     s_p = _Staged(params, dev)
     s_out = _Staged(out, dev, writeback=True)
-    check(lib.sgnn_unpack_dequant_rows_f32(_ptr(s_q.dev), _ptr(s_out.dev), _ptr(s_p.dev), _ptr(segs.seg),
-                                           _ptr(segs.pseg), segs.P, n, segs.n_packed, F, bits, _stream()))
+    if bf16:
+        check(lib.sgnn_unpack_dequant_rows_wire_f32(_ptr(s_q.dev), _ptr(s_out.dev), _ptr(s_p.dev), 1, _ptr(segs.seg),
+                                                    _ptr(segs.pseg), segs.P, n, segs.n_packed, F, bits, _stream()))
+    else:
+        check(lib.sgnn_unpack_dequant_rows_f32(_ptr(s_q.dev), _ptr(s_out.dev), _ptr(s_p.dev), _ptr(segs.seg),
+                                               _ptr(segs.pseg), segs.P, n, segs.n_packed, F, bits, _stream()))
     s_out.commit()
 
 
@@ -350,14 +407,21 @@ def dequantize_tensor(input, output, quantized_params, bits):
     _dequant_rows(input, output, quantized_params, _single_segment(output.shape[0], bits), bits)
 
 
-def quantize_tensor_for_all_procs(input, output, quantized_params, work_range_per_proc, num_procs, bits):
+def quantize_tensor_for_all_procs(input, output, quantized_params, work_range_per_proc, num_procs, bits,
+                                  row_index=None):
     """quantize_tensor_for_all_procs (quantization_arm.cpp:496-578): segment p = rows
     [work_range[p], work_range[p+1]) is packed on its own, starting at packed row
-    sum_{q<p} ceil(n_q / EPB)."""
+    sum_{q<p} ceil(n_q / EPB).
+
+    Beyond the reference's arguments: ``quantized_params`` may be a bfloat16 tensor (the (zero_point,
+    scale) pairs are then stored in the wire format of super_gnn/communicator.py:283-294, codes still
+    computed from the fp32 values), and ``row_index`` (int64, GPU) makes row r of the quantizer's
+    input ``input[row_index[r]]`` -- the index_select into send_buf of super_gnn/aggregator.py:48
+    folded into the quantizer."""
     _check_bits(bits)
     if work_range_per_proc.numel() != int(num_procs) + 1:
         raise ValueError("work_range_per_proc must have num_procs + 1 entries")
-    _quant_rows(input, output, quantized_params, quant_segments(work_range_per_proc, bits), bits)
+    _quant_rows(input, output, quantized_params, quant_segments(work_range_per_proc, bits), bits, row_index=row_index)
 
 
 def dequantize_tensor_for_all_procs(input, output, dequantized_params, work_range_per_proc, num_procs, bits):

@@ -130,20 +130,89 @@ def test_quantized_exchange_equals_cpu_flow(bits, pre):
     assert rel < {8: 0.01, 4: 0.1, 2: 0.5}[bits], rel
 
 
-def test_bf16_param_transport_matches_reference_wire_format():
-    # the reference ships (zero_point, scale) as bf16 (communicator.py:283-294)
+@pytest.mark.parametrize("bits,pre", [(8, False), (2, False), (4, True), (2, True)])
+def test_bf16_param_transport_matches_reference_wire_format(bits, pre):
+    """With bf16 params the world must give exactly the floats of the reference's sequence
+    (communicator.py:269-294, aggregator.py:72-93): quantize with fp32 params, copy_ to bf16, move,
+    copy_ back to fp32, dequantize, SpMM -- rebuilt here from the unfused GPU operators."""
+    from super_gnn_amd import Quantizer_for_all_procs, SPMM_forward
     from super_gnn_amd.aggregator import LoopbackWorld
     from super_gnn_amd.data_manager import build_loopback_partitions
     rowptr, col, w = _graph(n=4000, und_edges=30000, seed=2)
-    n, F, P = rowptr.numel() - 1, 64, 2
-    graphs = build_loopback_partitions(rowptr, col, w, P, F, num_bits=8, is_pre_delay=False)
+    n, F, P = rowptr.numel() - 1, 64, 3
+    graphs = build_loopback_partitions(rowptr, col, w, P, F, num_bits=bits, is_pre_delay=pre)
     x = torch.randn(n, F, generator=torch.Generator().manual_seed(3))
     feats = [x[g.node_range[0]:g.node_range[1]].cuda() for g in graphs]
-    o32 = torch.cat(LoopbackWorld(graphs, 8, False).aggregate(feats))
-    o16 = torch.cat(LoopbackWorld(graphs, 8, False, params_wire_dtype=torch.bfloat16).aggregate(feats))
-    prm = graphs[0].comm_buf_for_quantization.quantized_recv_params_buf_fp32
-    assert torch.equal(prm, prm.to(torch.bfloat16).to(torch.float32))  # what arrived is bf16-representable
-    assert not torch.equal(o32, o16) and torch.allclose(o32, o16, atol=0.05, rtol=0.05)
+    o32 = LoopbackWorld(graphs, bits, pre).aggregate(feats)
+    world16 = LoopbackWorld(graphs, bits, pre, params_wire_dtype=torch.bfloat16)
+    o16 = world16.aggregate(feats)
+    prm = graphs[0].comm_buf_for_quantization.quantized_recv_params_buf_bf16
+    assert prm.dtype == torch.bfloat16 and prm.shape[0] == sum(graphs[0].comm_splits.recv_splits)
+
+    qz = Quantizer_for_all_procs(P, bits)
+    crossed = []   # per sender: its send rows after quantize -> bf16 params -> dequantize
+    for g, xp in zip(graphs, feats):
+        ns = sum(g.comm_splits.send_splits)
+        sb = torch.zeros((ns, F), device="cuda")
+        if pre:
+            SPMM_forward(g.adj_t_pre_post_aggr_to, xp, sb)
+        elif ns:
+            sb = xp[g.idx_nodes_send_to_others].contiguous()
+        wr = torch.tensor([0] + list(np.cumsum(g.comm_splits.send_splits)), dtype=torch.int32)
+        q = torch.zeros((sum(g.comm_splits.send_splits_int2), F), dtype=torch.uint8, device="cuda")
+        p32 = torch.zeros((ns, 2), device="cuda")
+        back = torch.zeros_like(sb)
+        if ns:
+            qz.quantize_fp32_to_intX(sb, q, p32, wr)
+            p_wire = p32.to(torch.bfloat16).to(torch.float32)
+            qz.dequantize_intX_to_fp32(q, back, p_wire, wr)
+        crossed.append(back)
+    for r, (g, xp) in enumerate(zip(graphs, feats)):
+        segs = []
+        for p, h in enumerate(graphs):
+            o = np.concatenate([[0], np.cumsum(h.comm_splits.send_splits)])
+            segs.append(crossed[p][o[r]:o[r + 1]])
+        recv = torch.cat(segs).contiguous()
+        out = torch.zeros((g.local_adj_t.sparse_size(0), F), device="cuda")
+        SPMM_forward(g.local_adj_t, xp, out)
+        if recv.shape[0]:
+            SPMM_forward(g.adj_t_pre_post_aggr_from if pre else g.remote_adj_t, recv, out)
+        assert torch.equal(out, o16[r]), f"rank {r}"
+    a, b = torch.cat(o32), torch.cat(o16)
+    assert not torch.equal(a, b) and torch.allclose(a, b, atol=0.1, rtol=0.1)
+
+
+def test_backward_is_deterministic_and_matches_unfused_scatter():
+    """Plain mode, int8: the fused dequantize+scatter of the returned gradient rows equals
+    dequantize followed by a sequential index_add (reference: aggregator.py:159-175), run to run."""
+    from super_gnn_amd.aggregator import LoopbackWorld
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    rowptr, col, w = _graph(n=5000, und_edges=40000, seed=12)
+    n, F, P = rowptr.numel() - 1, 32, 4
+    graphs = build_loopback_partitions(rowptr, col, w, P, F, num_bits=8, is_pre_delay=False)
+    gen = torch.Generator().manual_seed(5)
+    x, G = torch.randn(n, F, generator=gen), torch.randn(n, F, generator=gen)
+    world = LoopbackWorld(graphs, 8, False)
+    runs = []
+    for _ in range(2):
+        feats = [x[g.node_range[0]:g.node_range[1]].cuda().requires_grad_() for g in graphs]
+        outs = world.aggregate(feats)
+        torch.autograd.backward(outs, [G[g.node_range[0]:g.node_range[1]].cuda() for g in graphs])
+        runs.append(torch.cat([f.grad for f in feats]))
+    assert torch.equal(runs[0], runs[1])
+    # rebuild partition 0's gradient from what the exchange left in its buffers
+    from super_gnn_amd import Quantizer_for_all_procs, SPMM_backward
+    g = graphs[0]
+    q = g.comm_buf_for_quantization
+    rows = torch.zeros_like(g.comm_buf.send_buf)
+    Quantizer_for_all_procs(P, 8).dequantize_intX_to_fp32(q.quantized_send_data_buf, rows, q.send_params,
+                                                          q.quantized_work_range_per_proc)
+    want = torch.zeros((g.node_range[1] - g.node_range[0], F), device="cuda")
+    SPMM_backward(g.local_adj_t, G[g.node_range[0]:g.node_range[1]].cuda(), want)
+    want = want.cpu()
+    for i, node in enumerate(g.idx_nodes_send_to_others.cpu().tolist()):   # index order, one add per row
+        want[node] += rows[i].cpu()
+    assert torch.equal(runs[0][:want.shape[0]].cpu(), want)
 
 
 def test_sage_model_is_partition_invariant_and_trains():

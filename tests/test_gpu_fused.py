@@ -134,3 +134,22 @@ def test_fused_errors():
         ops.spmm_dequantized(None, None, None, q, params, torch.tensor([0, 39], dtype=torch.int32), 1, 2, out, plan=plan)
     with pytest.raises(ValueError):
         ops.spmm_dequantized(None, None, None, q, params, seg_t, P, 2, torch.zeros(50, 62, device="cuda"), plan=plan)
+
+
+@pytest.mark.parametrize("bits", [8, 2])
+@pytest.mark.parametrize("hubs", [0, 6])
+def test_fused_with_bf16_params_equals_widened_params(bits, hubs):
+    """params handed over as bf16 pairs == the same pairs widened to fp32 first (bitwise)."""
+    M, K, F = 3000, 2000, 128
+    seg = [0, 513, 1200, K]
+    ops, plan, rowptr, col, val, x, seg_t, P, q, params = _setup(M, K, F, 9, bits, seg, seed=31 + bits, hubs=hubs)
+    p16 = params.to(torch.bfloat16)
+    v = torch.from_numpy(val).cuda()
+    segs = ops.quant_segments(seg_t, bits)
+    a = torch.randn(M, F, generator=torch.Generator().manual_seed(1)).cuda()
+    b = a.clone()
+    plan.run_quantized(v, q, p16, segs, bits, a, accumulate=True)
+    plan.run_quantized(v, q, p16.to(torch.float32), segs, bits, b, accumulate=True)
+    assert torch.equal(a, b)
+    with pytest.raises(TypeError):
+        plan.run_quantized(v, q, params.to(torch.float16), segs, bits, a, accumulate=True)

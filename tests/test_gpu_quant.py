@@ -269,3 +269,57 @@ def test_fast_quotient_equals_ieee_division(bits):
     xs = x[: na + 8].cpu().numpy()
     q_ref, p_ref = orc.quant_rows(xs, [0, na + 8], bits)
     assert np.array_equal(outs[0][0][: (na + 8) // epb].cpu().numpy(), q_ref)
+
+
+# ------------------------------------------------------------------------------------------------
+# wire-side variants: gathered input rows, bf16 (zero_point, scale)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("bits", [8, 4, 2])
+@pytest.mark.parametrize("F", [128, 256, 100, 37, 1200])
+def test_gathering_quantizer_equals_index_select_then_quantize(bits, F):
+    from super_gnn_amd import supergnn_ops as ops
+    gen = torch.Generator().manual_seed(bits * 1000 + F)
+    src = torch.randn(5000, F, generator=gen).cuda()
+    idx = torch.randint(0, 5000, (3001,), generator=gen).cuda()
+    wr = torch.tensor([0, 700, 700, 1999, 3001], dtype=torch.int32)
+    npk = sum(-(-int(b - a) // (8 // bits)) for a, b in zip(wr[:-1], wr[1:]))
+    q_a = torch.zeros((npk, F), dtype=torch.uint8, device="cuda"); p_a = torch.zeros((3001, 2), device="cuda")
+    q_b = torch.zeros_like(q_a); p_b = torch.zeros_like(p_a)
+    ops.quantize_tensor_for_all_procs(src[idx].contiguous(), q_a, p_a, wr, 4, bits)
+    ops.quantize_tensor_for_all_procs(src, q_b, p_b, wr, 4, bits, row_index=idx)
+    assert torch.equal(q_a, q_b) and torch.equal(p_a, p_b)
+    # strided source (a column window of a wider matrix)
+    wide = torch.randn(5000, F + 8, generator=gen).cuda()
+    view = wide[:, 4:4 + F]
+    q_c = torch.zeros_like(q_a); p_c = torch.zeros_like(p_a)
+    ops.quantize_tensor_for_all_procs(view, q_c, p_c, wr, 4, bits, row_index=idx)
+    ops.quantize_tensor_for_all_procs(view[idx].contiguous(), q_a, p_a, wr, 4, bits)
+    assert torch.equal(q_a, q_c) and torch.equal(p_a, p_c)
+    with pytest.raises(IndexError):
+        ops.quantize_tensor_for_all_procs(src, q_b, p_b, wr, 4, bits, row_index=idx + 4000)
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+@pytest.mark.parametrize("F", [128, 64, 602, 1200])
+def test_bf16_params_equal_torch_casts(bits, F):
+    """bf16 params out of the quantizer == torch's fp32->bf16 copy of the fp32 params (codes
+    unchanged); dequantizing with bf16 params == dequantizing with their exact fp32 widening."""
+    from super_gnn_amd import supergnn_ops as ops
+    gen = torch.Generator().manual_seed(bits + F)
+    n = 2049
+    x = (torch.randn(n, F, generator=gen) * torch.logspace(-20, 20, n).unsqueeze(1)).cuda()
+    x[5] = 0.0; x[6] = -0.0; x[7, 0] = float("nan"); x[8] = 3.0e38; x[8, 1] = -3.0e38
+    wr = torch.tensor([0, 1000, n], dtype=torch.int32)
+    npk = sum(-(-int(b - a) // (8 // bits)) for a, b in zip(wr[:-1], wr[1:]))
+    q32 = torch.zeros((npk, F), dtype=torch.uint8, device="cuda"); p32 = torch.zeros((n, 2), device="cuda")
+    q16 = torch.zeros_like(q32); p16 = torch.zeros((n, 2), dtype=torch.bfloat16, device="cuda")
+    ops.quantize_tensor_for_all_procs(x, q32, p32, wr, 2, bits)
+    ops.quantize_tensor_for_all_procs(x, q16, p16, wr, 2, bits)
+    assert torch.equal(q32, q16)
+    want16 = p32.to(torch.bfloat16)
+    assert torch.equal(p16.view(torch.int16)[~want16.isnan()], want16.view(torch.int16)[~want16.isnan()])
+    assert torch.equal(p16.isnan(), want16.isnan())
+    a = torch.zeros((n, F), device="cuda"); b = torch.zeros((n, F), device="cuda")
+    ops.dequantize_tensor_for_all_procs(q16, a, p16, wr, 2, bits)
+    ops.dequantize_tensor_for_all_procs(q16, b, p16.to(torch.float32), wr, 2, bits)
+    assert torch.equal(a.nan_to_num(1.5, 2.5, 3.5), b.nan_to_num(1.5, 2.5, 3.5))
