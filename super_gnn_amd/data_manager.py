@@ -4,14 +4,21 @@ builder that cuts ONE global graph into P vertex partitions inside a single proc
 aggregation data flow of ``super_gnn/aggregator.py`` can run on one GPU with a loop-back exchange.
 
 The reference builds these objects per MPI rank from ParMETIS partition files with handshakes between
-ranks (DataProcessor.py:17-123, :258-281); here every partition is built from the global CSR directly.
-The pre/post-aggregation split uses a simple per-rank-pair vertex cover (all sources or all
-destinations of the pair's boundary edges, whichever is fewer) instead of the reference's minimum
-vertex cover: any vertex cover yields a correct data flow; only the communication volume differs."""
+ranks (DataLoader.py:17-278, DataProcessor.py:17-541); here every partition is built from the global
+CSR directly, and ``load_loopback_partitions`` reads the reference's per-rank files back into that
+global CSR first.  The pre/post-aggregation split follows the reference: per ordered rank pair a
+minimum vertex cover of the pair's bipartite boundary graph decides, edge by edge, whether the source
+row is shipped (source in the cover: post-aggregation at the receiver) or a partial sum per
+destination is (pre-aggregation at the sender) (DataProcessor.py:266-289, VertexCoverFinder.py:686-753);
+the cover comes from a Hopcroft-Karp maximum matching plus Koenig's construction."""
 import math
+import os
 from typing import List, Optional
 
+import numpy as np
+import scipy.sparse as sp
 import torch
+from scipy.sparse.csgraph import maximum_bipartite_matching
 from torch import Tensor
 
 from .sparse import SparseTensor
@@ -111,18 +118,69 @@ def _coo_to_sparse(row, col, val, sizes, device):
     return SparseTensor(row=row, col=col, value=val, sparse_sizes=sizes).to(device)
 
 
+def minimum_vertex_cover(src: np.ndarray, dst: np.ndarray):
+    """Minimum vertex cover of the bipartite graph with edges (src[i], dst[i]); sources and
+    destinations are separate id spaces.  Returns boolean masks (src_in_cover, dst_in_cover) over the
+    *edges' endpoints*: every edge has src_in_cover[i] or dst_in_cover[i], and the number of distinct
+    covered endpoints equals the size of a maximum matching (Koenig's theorem).  Same role as
+    VertexCoverFinder.find_minimum_vertex_cover (super_gnn/data_manager/VertexCoverFinder.py:697-753)."""
+    if src.size == 0:
+        return np.zeros(0, bool), np.zeros(0, bool)
+    us, ui = np.unique(src, return_inverse=True)
+    vs, vi = np.unique(dst, return_inverse=True)
+    nu, nv = us.size, vs.size
+    g = sp.csr_matrix((np.ones(src.size, np.int8), (ui, vi)), shape=(nu, nv))
+    g.sum_duplicates()
+    match_u = maximum_bipartite_matching(g, perm_type="column")      # for each u: matched v or -1
+    match_v = np.full(nv, -1, np.int64)
+    match_v[match_u[match_u >= 0]] = np.nonzero(match_u >= 0)[0]
+    # Z = vertices reachable from unmatched u by alternating paths (free edge u->v, matched edge v->u)
+    zu = match_u < 0
+    zv = np.zeros(nv, bool)
+    frontier = np.nonzero(zu)[0]
+    indptr, indices = g.indptr, g.indices
+    while frontier.size:
+        counts = indptr[frontier + 1] - indptr[frontier]
+        starts = np.repeat(indptr[frontier], counts)
+        offs = np.arange(counts.sum()) - np.repeat(np.cumsum(counts) - counts, counts)
+        nbr = np.unique(indices[starts + offs])
+        nbr = nbr[~zv[nbr]]
+        zv[nbr] = True
+        nxt = match_v[nbr]
+        nxt = nxt[nxt >= 0]
+        nxt = nxt[~zu[nxt]]
+        zu[nxt] = True
+        frontier = nxt
+    cover_u, cover_v = ~zu, zv                                        # (U \ Z) + (V & Z)
+    return cover_u[ui], cover_v[vi]
+
+
 def build_loopback_partitions(rowptr: Tensor, col: Tensor, value: Optional[Tensor], num_parts: int, feat_len: int,
-                              num_bits: int = 32, is_pre_delay: bool = False, device="cuda") -> List[object]:
+                              num_bits: int = 32, is_pre_delay: bool = False, device="cuda",
+                              bounds: Optional[Tensor] = None, cover: str = "minimum") -> List[object]:
     """Cut the global graph (CSR over destination rows, i.e. the transposed adjacency the reference
-    calls ``adj_t``) into ``num_parts`` contiguous vertex ranges and build each partition's graph
-    object, comm splits and buffers.  Returns a list of DistributedGraph / DistributedGraphForPre,
-    each with an extra attribute ``node_range = (begin, end)``."""
+    calls ``adj_t``) into ``num_parts`` contiguous vertex ranges (``bounds``: the reference's
+    begin_node_on_each_partition, default equal ranges) and build each partition's graph object, comm
+    splits and buffers.  Returns a list of DistributedGraph / DistributedGraphForPre, each with an
+    extra attribute ``node_range = (begin, end)``.
+
+    ``cover`` (pre/post mode only): "minimum" = minimum vertex cover per rank pair (the reference's
+    rule), "side" = all sources or all destinations of the pair, whichever is fewer.  Within a segment
+    the message rows are ordered by the global id of the node they stand for, as in the reference
+    (DataProcessor.py:306-318)."""
     rowptr = rowptr.detach().cpu().to(torch.int64)
     col = col.detach().cpu().to(torch.int64)
     N = rowptr.numel() - 1
     P = int(num_parts)
     val = value.detach().cpu().to(torch.float32) if value is not None else torch.ones(col.numel())
-    bounds = torch.tensor([N * p // P for p in range(P + 1)], dtype=torch.int64)
+    if bounds is None:
+        bounds = torch.tensor([N * p // P for p in range(P + 1)], dtype=torch.int64)
+    else:
+        bounds = torch.as_tensor(bounds, dtype=torch.int64)
+        if bounds.numel() != P + 1 or int(bounds[0]) != 0 or int(bounds[-1]) != N or bool((bounds[1:] < bounds[:-1]).any()):
+            raise ValueError("bounds must be P + 1 non-decreasing node offsets from 0 to the node count")
+    if cover not in ("minimum", "side"):
+        raise ValueError("cover must be 'minimum' or 'side'")
     deg = rowptr[1:] - rowptr[:-1]
     row = torch.repeat_interleave(torch.arange(N), deg)
     owner_of = lambda ids: torch.searchsorted(bounds, ids, right=True) - 1  # noqa: E731
@@ -138,7 +196,7 @@ def build_loopback_partitions(rowptr: Tensor, col: Tensor, value: Optional[Tenso
                       "local": (rr[is_local], cc[is_local] - b, ww[is_local]),
                       "remote": (rr[~is_local], cc[~is_local], ww[~is_local])})
 
-    # boundary blocks: blocks[p][r] = (rows (rows at the receiver r), cols (source nodes local to p), weights)
+    # boundary blocks per ordered pair p -> r (p owns the sources, r the destinations)
     seg_rows = [[0] * P for _ in range(P)]          # rows exchanged p -> r
     to_blocks = [[None] * P for _ in range(P)]      # at the sender p: (seg_row, local_src, w)
     from_blocks = [[None] * P for _ in range(P)]    # at the receiver r: (local_dst, seg_row, w)
@@ -152,21 +210,36 @@ def build_loopback_partitions(rowptr: Tensor, col: Tensor, value: Optional[Tenso
             m = own == p
             if not bool(m.any()):
                 continue
-            vv, uu, wwp = v[m], u_glob[m] - int(bounds[p]), w[m]
-            src_nodes, src_inv = torch.unique(uu, return_inverse=True)
-            dst_nodes, dst_inv = torch.unique(vv, return_inverse=True)
-            if not is_pre_delay or src_nodes.numel() <= dst_nodes.numel():
-                # post-aggregation: ship the source rows, apply the edges at the receiver
-                n = src_nodes.numel()
-                to_blocks[p][r] = (torch.arange(n), src_nodes, torch.ones(n))
-                from_blocks[p][r] = (vv, src_inv, wwp)
-                send_idx[p][r] = src_nodes
+            vv, uu, wwp = v[m], u_glob[m] - int(bounds[p]), w[m]     # dst local to r, src local to p
+            if not is_pre_delay:
+                post = torch.ones(vv.numel(), dtype=torch.bool)
+            elif cover == "side":
+                n_src, n_dst = torch.unique(uu).numel(), torch.unique(vv).numel()
+                post = torch.full((vv.numel(),), n_src <= n_dst, dtype=torch.bool)
             else:
-                # pre-aggregation: ship one partial sum per destination node
-                n = dst_nodes.numel()
-                to_blocks[p][r] = (dst_inv, uu, wwp)
-                from_blocks[p][r] = (dst_nodes, torch.arange(n), torch.ones(n))
-            seg_rows[p][r] = n
+                src_in_cover, _ = minimum_vertex_cover(uu.numpy(), vv.numpy())
+                post = torch.from_numpy(src_in_cover)                 # DataProcessor.py:283-287
+            # message rows: one per shipped source node (post) and one per pre-aggregated destination,
+            # ordered by global id (sources of p and destinations of r live in disjoint id ranges)
+            post_nodes = torch.unique(uu[post]) + int(bounds[p])
+            pre_nodes = torch.unique(vv[~post]) + int(bounds[r])
+            keys = torch.cat([post_nodes, pre_nodes])
+            order = torch.argsort(keys)
+            slot_of = torch.empty_like(order)
+            slot_of[order] = torch.arange(order.numel())
+            post_slot, pre_slot = slot_of[:post_nodes.numel()], slot_of[post_nodes.numel():]
+            e_post_slot = post_slot[torch.searchsorted(post_nodes, uu[post] + int(bounds[p]))]
+            e_pre_slot = pre_slot[torch.searchsorted(pre_nodes, vv[~post] + int(bounds[r]))]
+            n_post, n_pre = post_nodes.numel(), pre_nodes.numel()
+            to_blocks[p][r] = (torch.cat([post_slot, e_pre_slot]),
+                               torch.cat([post_nodes - int(bounds[p]), uu[~post]]),
+                               torch.cat([torch.ones(n_post), wwp[~post]]))
+            from_blocks[p][r] = (torch.cat([vv[post], pre_nodes - int(bounds[r])]),
+                                 torch.cat([e_post_slot, pre_slot]),
+                                 torch.cat([wwp[post], torch.ones(n_pre)]))
+            if not is_pre_delay:
+                send_idx[p][r] = post_nodes - int(bounds[p])
+            seg_rows[p][r] = n_post + n_pre
 
     graphs = []
     for r in range(P):
@@ -208,3 +281,103 @@ def build_loopback_partitions(rowptr: Tensor, col: Tensor, value: Optional[Tenso
         g.node_range = parts[r]["range"]
         graphs.append(g)
     return graphs
+
+
+# ------------------------------------------------------------------------------------------------
+# The reference's on-disk partition format (one set of files per rank, written by its
+# graph_partition scripts and read by super_gnn/data_manager/DataLoader.py:17-68)
+# ------------------------------------------------------------------------------------------------
+def _rank_file(input_dir, graph_name, rank, what):
+    return os.path.join(input_dir, "p{:0>3d}-{}_{}.npy".format(rank, graph_name, what))
+
+
+def load_graph_structures(input_dir, graph_name, rank):
+    """(local_nodes_list [n,>=1] with the global id in column 0, local_edges_list [2,E] = (src, dst)
+    both local ids, remote_edges_list [2,E'] = (global src id, local dst id),
+    begin_node_on_each_partition [P+1], num_local_nodes) -- DataLoader.py:17-46."""
+    nodes = np.load(_rank_file(input_dir, graph_name, rank, "nodes"))
+    local_edges = np.load(_rank_file(input_dir, graph_name, rank, "local_edges"))
+    remote_edges = np.load(_rank_file(input_dir, graph_name, rank, "remote_edges"))
+    begins = np.loadtxt(os.path.join(input_dir, "begin_node_on_each_partition.txt"), dtype=np.int64, delimiter=" ")
+    num_local = int(nodes[-1][0] - nodes[0][0] + 1)
+    return (torch.from_numpy(nodes), torch.from_numpy(local_edges), torch.from_numpy(remote_edges),
+            torch.from_numpy(np.atleast_1d(begins)), num_local)
+
+
+def load_nodes_labels(input_dir, graph_name, rank):
+    return torch.from_numpy(np.load(_rank_file(input_dir, graph_name, rank, "nodes_label")))   # DataLoader.py:49-54
+
+
+def load_nodes_features(input_dir, graph_name, rank):
+    feat = np.load(_rank_file(input_dir, graph_name, rank, "nodes_feat"))                      # DataLoader.py:57-62
+    if feat.dtype == np.float16:
+        feat = feat.astype(np.float32)
+    return torch.from_numpy(feat)
+
+
+def load_dataset_mask(input_dir, graph_name, rank):
+    return tuple(torch.from_numpy(np.load(_rank_file(input_dir, graph_name, rank, "nodes_%s_idx" % k)))
+                 for k in ("train", "valid", "test"))                                        # DataLoader.py:65-68
+
+
+def load_loopback_partitions(input_dir, graph_name, world_size, feat_len, num_bits=32, is_pre_delay=False,
+                             device="cuda", cover="minimum"):
+    """Read every rank's files and build the P partitions in this process.  Returns
+    (graphs, data) where data[p] is the dict the reference's load_data returns per rank
+    (DataLoader.py:213-278): nodes_features, nodes_labels, nodes_{train,valid,test}_masks, plus graph.
+    Edge weights are ones, as in DataProcessor.transform_edge_index_to_sparse_tensor (:108-123)."""
+    P = int(world_size)
+    srcs, dsts, begins = [], [], None
+    for rank in range(P):
+        nodes, local_edges, remote_edges, b, n_local = load_graph_structures(input_dir, graph_name, rank)
+        if begins is None:
+            begins = b.to(torch.int64)
+            if begins.numel() != P + 1:
+                raise ValueError("begin_node_on_each_partition.txt lists %d ranges, world_size is %d" % (begins.numel() - 1, P))
+        first = int(nodes[0][0])
+        if first != int(begins[rank]) or n_local != int(begins[rank + 1] - begins[rank]):
+            raise ValueError("rank %d: node list does not match begin_node_on_each_partition.txt" % rank)
+        srcs += [local_edges[0].to(torch.int64) + first, remote_edges[0].to(torch.int64)]
+        dsts += [local_edges[1].to(torch.int64) + first, remote_edges[1].to(torch.int64) + first]
+    src, dst = torch.cat(srcs), torch.cat(dsts)
+    N = int(begins[-1])
+    order = torch.argsort(dst * N + src)                 # CSR over destinations, columns ascending
+    src, dst = src[order], dst[order]
+    rowptr = torch.zeros(N + 1, dtype=torch.int64)
+    rowptr[1:] = torch.cumsum(torch.bincount(dst, minlength=N), 0)
+    graphs = build_loopback_partitions(rowptr, src, None, P, feat_len, num_bits=num_bits, is_pre_delay=is_pre_delay,
+                                       device=device, bounds=begins, cover=cover)
+    data = []
+    for rank, g in enumerate(graphs):
+        train, valid, test = load_dataset_mask(input_dir, graph_name, rank)
+        data.append({"graph": g, "nodes_features": load_nodes_features(input_dir, graph_name, rank),
+                     "nodes_labels": load_nodes_labels(input_dir, graph_name, rank),
+                     "nodes_train_masks": train, "nodes_valid_masks": valid, "nodes_test_masks": test})
+    return graphs, data
+
+
+def save_partition_files(output_dir, graph_name, rowptr, col, bounds, feat, label, train_idx, valid_idx, test_idx):
+    """Write a global graph (CSR over destinations) as the reference's per-rank files, for the given
+    contiguous node ranges: the layout load_graph_structures reads.  train/valid/test_idx are global
+    node ids; each rank stores its own, localized."""
+    os.makedirs(output_dir, exist_ok=True)
+    rowptr = torch.as_tensor(rowptr, dtype=torch.int64).cpu()
+    col = torch.as_tensor(col, dtype=torch.int64).cpu()
+    bounds = torch.as_tensor(bounds, dtype=torch.int64).cpu()
+    N = rowptr.numel() - 1
+    row = torch.repeat_interleave(torch.arange(N), rowptr[1:] - rowptr[:-1])
+    np.savetxt(os.path.join(output_dir, "begin_node_on_each_partition.txt"), bounds.numpy()[None, :], fmt="%d", delimiter=" ")
+    for rank in range(bounds.numel() - 1):
+        b, e = int(bounds[rank]), int(bounds[rank + 1])
+        sel = slice(int(rowptr[b]), int(rowptr[e]))
+        src, dst = col[sel], row[sel] - b
+        local = (src >= b) & (src < e)
+        ids = torch.arange(b, e)
+        np.save(_rank_file(output_dir, graph_name, rank, "nodes"), torch.stack([ids, ids - b], 1).numpy())
+        np.save(_rank_file(output_dir, graph_name, rank, "local_edges"), torch.stack([src[local] - b, dst[local]]).numpy())
+        np.save(_rank_file(output_dir, graph_name, rank, "remote_edges"), torch.stack([src[~local], dst[~local]]).numpy())
+        np.save(_rank_file(output_dir, graph_name, rank, "nodes_feat"), torch.as_tensor(feat)[b:e].cpu().numpy())
+        np.save(_rank_file(output_dir, graph_name, rank, "nodes_label"), torch.as_tensor(label)[b:e].cpu().numpy())
+        for name, idx in (("train", train_idx), ("valid", valid_idx), ("test", test_idx)):
+            idx = torch.as_tensor(idx, dtype=torch.int64).cpu()
+            np.save(_rank_file(output_dir, graph_name, rank, "nodes_%s_idx" % name), (idx[(idx >= b) & (idx < e)] - b).numpy())

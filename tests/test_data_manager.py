@@ -1,0 +1,138 @@
+"""Host-side partition logic (no GPU): minimum vertex cover, the pre/post split, and the reference's
+on-disk partition format (super_gnn/data_manager/DataLoader.py:17-68) written and read back."""
+import itertools
+
+import numpy as np
+import scipy.sparse as sp
+import torch
+
+from super_gnn_amd.data_manager import (build_loopback_partitions, load_loopback_partitions, minimum_vertex_cover,
+                                        save_partition_files)
+from super_gnn_amd.synth import rmat_graph
+
+
+def _brute_force_cover_size(src, dst):
+    us, vs = np.unique(src), np.unique(dst)
+    verts = [("u", u) for u in us] + [("v", v) for v in vs]
+    for k in range(len(verts) + 1):
+        for pick in itertools.combinations(verts, k):
+            chosen = set(pick)
+            if all(("u", s) in chosen or ("v", d) in chosen for s, d in zip(src, dst)):
+                return k
+    raise AssertionError
+
+
+def test_minimum_vertex_cover_against_brute_force():
+    rng = np.random.default_rng(0)
+    for trial in range(60):
+        nu, nv, ne = rng.integers(1, 6), rng.integers(1, 6), rng.integers(1, 12)
+        src, dst = rng.integers(0, nu, ne), rng.integers(0, nv, ne) + 100
+        cu, cv = minimum_vertex_cover(src, dst)
+        assert np.all(cu | cv), "not a cover"
+        size = np.unique(src[cu]).size + np.unique(dst[cv]).size
+        assert size == _brute_force_cover_size(src, dst), (trial, src, dst)
+        # membership is a property of the node, not of the edge
+        for s in np.unique(src):
+            assert np.unique(cu[src == s]).size == 1
+        for d in np.unique(dst):
+            assert np.unique(cv[dst == d]).size == 1
+
+
+def test_minimum_vertex_cover_size_equals_maximum_matching():
+    from scipy.sparse.csgraph import maximum_bipartite_matching
+    rng = np.random.default_rng(1)
+    src = (rng.zipf(1.6, 40000) % 3000).astype(np.int64)
+    dst = (rng.zipf(1.4, 40000) % 5000).astype(np.int64)
+    cu, cv = minimum_vertex_cover(src, dst)
+    assert np.all(cu | cv)
+    g = sp.csr_matrix((np.ones(src.size), (src, dst)), shape=(3000, 5000))
+    matching = (maximum_bipartite_matching(g, perm_type="column") >= 0).sum()
+    assert np.unique(src[cu]).size + np.unique(dst[cv]).size == matching
+    assert matching <= min(np.unique(src).size, np.unique(dst).size)
+    assert minimum_vertex_cover(np.zeros(0, np.int64), np.zeros(0, np.int64))[0].size == 0
+
+
+def _scipy(m):
+    rowptr, col, val = m.csr()
+    return sp.csr_matrix((val.cpu().numpy(), col.cpu().numpy(), rowptr.cpu().numpy()), shape=tuple(m.sparse_sizes()))
+
+
+def _flow(graphs, x, pre):
+    """The aggregation data flow with scipy products and a loop-back exchange."""
+    P = len(graphs)
+    sent = []
+    for g in graphs:
+        xp = x[g.node_range[0]:g.node_range[1]]
+        sent.append(_scipy(g.adj_t_pre_post_aggr_to) @ xp if pre else xp[g.idx_nodes_send_to_others.cpu().numpy()])
+    outs = []
+    for r, g in enumerate(graphs):
+        segs = []
+        for p, h in enumerate(graphs):
+            o = np.concatenate([[0], np.cumsum(h.comm_splits.send_splits)])
+            segs.append(sent[p][o[r]:o[r + 1]])
+            assert segs[-1].shape[0] == g.comm_splits.recv_splits[p]
+        recv = np.concatenate(segs)
+        xp = x[g.node_range[0]:g.node_range[1]]
+        outs.append(_scipy(g.local_adj_t) @ xp + _scipy(g.adj_t_pre_post_aggr_from if pre else g.remote_adj_t) @ recv)
+    return np.concatenate(outs)
+
+
+def _graph(n=3000, e=20000, seed=0):
+    rowptr, col = rmat_graph(n, e, seed=seed)
+    w = torch.rand(col.numel(), generator=torch.Generator().manual_seed(seed)) + 0.5
+    return rowptr, col, w
+
+
+def test_partition_flow_equals_global_product_on_cpu():
+    rowptr, col, w = _graph()
+    n = rowptr.numel() - 1
+    A = sp.csr_matrix((w.numpy().astype(np.float64), col.numpy(), rowptr.numpy()), shape=(n, n))
+    x = np.random.default_rng(0).standard_normal((n, 8))
+    want = A @ x
+    bounds = torch.tensor([0, 100, 100, 1700, n])        # uneven, one empty partition
+    for pre, cover in ((False, "minimum"), (True, "minimum"), (True, "side")):
+        for b in (None, bounds):
+            graphs = build_loopback_partitions(rowptr, col, w, 4, 8, num_bits=32, is_pre_delay=pre, device="cpu",
+                                               bounds=b, cover=cover)
+            got = _flow(graphs, x, pre)
+            assert np.allclose(got, want, rtol=1e-5, atol=1e-5), (pre, cover)
+    rows = {}
+    for cover in ("minimum", "side"):
+        graphs = build_loopback_partitions(rowptr, col, w, 4, 8, num_bits=32, is_pre_delay=True, device="cpu", cover=cover)
+        rows[cover] = sum(sum(g.comm_splits.send_splits) for g in graphs)
+    plain = build_loopback_partitions(rowptr, col, w, 4, 8, num_bits=32, is_pre_delay=False, device="cpu")
+    rows["plain"] = sum(sum(g.comm_splits.send_splits) for g in plain)
+    assert rows["minimum"] <= rows["side"] <= rows["plain"], rows
+    assert rows["minimum"] < rows["plain"]
+
+
+def test_reference_partition_files_round_trip(tmp_path):
+    rowptr, col, _ = _graph(n=2000, e=12000, seed=3)
+    n = rowptr.numel() - 1
+    gen = torch.Generator().manual_seed(0)
+    feat = torch.randn(n, 16, generator=gen).to(torch.float16)
+    label = torch.randint(0, 7, (n,), generator=gen)
+    perm = torch.randperm(n, generator=gen)
+    train, valid, test = perm[:1000].sort().values, perm[1000:1500].sort().values, perm[1500:].sort().values
+    bounds = torch.tensor([0, 600, 1300, n])
+    save_partition_files(str(tmp_path), "toy", rowptr, col, bounds, feat, label, train, valid, test)
+    assert (tmp_path / "p002-toy_remote_edges.npy").exists() and (tmp_path / "begin_node_on_each_partition.txt").exists()
+    for pre in (False, True):
+        graphs, data = load_loopback_partitions(str(tmp_path), "toy", 3, 16, num_bits=2, is_pre_delay=pre, device="cpu")
+        direct = build_loopback_partitions(rowptr, col, None, 3, 16, num_bits=2, is_pre_delay=pre, device="cpu", bounds=bounds)
+        for g, d in zip(graphs, direct):
+            assert g.node_range == d.node_range
+            assert g.comm_splits.send_splits == d.comm_splits.send_splits
+            assert g.comm_splits.recv_splits_int2 == d.comm_splits.recv_splits_int2
+            names = ("local_adj_t", "adj_t_pre_post_aggr_from", "adj_t_pre_post_aggr_to") if pre else ("local_adj_t", "remote_adj_t")
+            for name in names:
+                a, b = _scipy(getattr(g, name)), _scipy(getattr(d, name))
+                assert a.shape == b.shape and (a != b).nnz == 0
+            assert torch.equal(g.in_degrees, d.in_degrees)
+        for rank, rec in enumerate(data):
+            b, e = int(bounds[rank]), int(bounds[rank + 1])
+            assert rec["nodes_features"].dtype == torch.float32                     # fp16 files are widened
+            assert torch.equal(rec["nodes_features"], feat[b:e].to(torch.float32))
+            assert torch.equal(rec["nodes_labels"], label[b:e])
+            assert torch.equal(rec["nodes_train_masks"] + b, train[(train >= b) & (train < e)])
+            assert rec["graph"] is graphs[rank]
