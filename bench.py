@@ -151,7 +151,7 @@ def main():
     ap.add_argument("--uniform-rows", type=int, default=0, help="diagnostic: replace the R-MAT graph by uniform random "
                     "rows of --uniform-degree neighbours over --nodes columns")
     ap.add_argument("--uniform-degree", type=int, default=25)
-    ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy", "prepost", "sbm", "aggregate"],
+    ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy", "prepost", "sbm", "aggregate", "sage"],
                     help="rmat: headline SpMM (default); quant: int2 quantize+pack as the step; copy: streaming copy; "
                          "prepost: one partition with packed remote rows, fused vs separate; sbm: dense-degree graph, F=602")
     ap.add_argument("--local-nodes", type=int, default=8_000_000)
@@ -159,6 +159,8 @@ def main():
     ap.add_argument("--local-und-edges", type=int, default=160_000_000)
     ap.add_argument("--remote-edges", type=int, default=80_000_000)
     ap.add_argument("--sbm-nodes", type=int, default=233_000)
+    ap.add_argument("--hidden", type=int, default=256, help="sage: hidden width")
+    ap.add_argument("--classes", type=int, default=47, help="sage: output classes")
     ap.add_argument("--parts", type=int, default=8, help="aggregate: number of vertex partitions simulated in this process")
     ap.add_argument("--exchange-bits", type=int, default=2, help="aggregate: 32 (fp32 rows) or 8/4/2 (packed)")
     ap.add_argument("--pre", type=int, default=1, help="aggregate: 1 = pre/post aggregation, 0 = plain boundary exchange")
@@ -445,6 +447,40 @@ def main():
         result = {"metric": "aggregation layer GEdges/s (forward+backward, loop-back exchange)",
                   "value": round(2 * nnz / ms / 1e6, 4), "unit": "GEdges/s",
                   "config": {"workload": f"aggregate_rmat_{args.nodes}n_{nnz}e_F{F}_P{args.parts}_bits{args.exchange_bits}_pre{args.pre}"},
+                  "ms_per_step": ms, "dtype": "f32", "roofline": None, "cpu_baseline": None}
+
+    # ---- one training epoch of a 3-layer GraphSAGE over P partitions (examples/graphsage/sage.py:213-232) ----
+    if args.workload == "sage":
+        from super_gnn_amd.aggregator import LoopbackWorld
+        from super_gnn_amd.data_manager import build_loopback_partitions
+        from super_gnn_amd.layers import LoopbackSAGE
+        F, H, C = args.feat, args.hidden, args.classes
+        rowptr, col, _, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
+        graphs = build_loopback_partitions(rowptr, col, None, args.parts, max(F, H, C), num_bits=args.exchange_bits,
+                                           is_pre_delay=bool(args.pre), device=dev)
+        world = LoopbackWorld(graphs, args.exchange_bits, bool(args.pre),
+                              params_wire_dtype=torch.bfloat16 if args.exchange_bits in (2, 4, 8) else None)
+        torch.manual_seed(0)
+        model = LoopbackSAGE(F, H, C, num_layers=3, dropout=0.5).to(dev)
+        model.reset_parameters()
+        opt = torch.optim.Adam(model.parameters(), lr=0.01)
+        feats = [x[g.node_range[0]:g.node_range[1]] for g in graphs]
+        labels = torch.randint(0, C, (rowptr.numel() - 1,), device=dev)
+
+        def epoch():
+            model.train()
+            opt.zero_grad()
+            out = torch.cat(model(world, feats))
+            loss = torch.nn.functional.nll_loss(out, labels)
+            loss.backward()
+            opt.step()
+
+        ms = time_steps(epoch, args.steps, args.warmup)
+        nnz = col.numel()
+        log(f"[bench] sage epoch {ms:.3f} ms (3 layers {F}-{H}-{H}-{C}, P={args.parts}, bits={args.exchange_bits}, pre={args.pre})")
+        result = {"metric": "GraphSAGE training epoch time (3 layers, full graph, loop-back exchange)",
+                  "value": round(1000.0 / ms, 4), "unit": "epochs/s",
+                  "config": {"workload": f"sage_rmat_{args.nodes}n_{nnz}e_F{F}_H{H}_C{C}_P{args.parts}_bits{args.exchange_bits}_pre{args.pre}"},
                   "ms_per_step": ms, "dtype": "f32", "roofline": None, "cpu_baseline": None}
 
     line = {"metric": result["metric"], "value": result["value"], "unit": result["unit"], "n_gpus": 1,
