@@ -489,62 +489,62 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
-// Unpack + dequantize, one fp32 row per 16 lanes (float4 lanes, F <= 1024): the mirror image of
-// quant_pack_rows16_kernel.  Every lane reads the packed words of its own row's packed row (the DPP
-// rows that share a packed row read the same words), extracts its row's code and writes its row.
+// Unpack + dequantize over the flat output (F % 4 == 0, any F): the fp32 output is one contiguous
+// array of n*F/4 float4, and every wavefront store covers 64 consecutive float4 = 1 KB of it,
+// whatever the row width (a 512-byte row: two rows per store; a 4-KB row: a quarter row).  A lane
+// derives (row, column) from its flat index, fetches the packed word that holds its four codes and
+// the row's params, and writes.  Rows that share a packed word re-read it from the cache.  Waves are
+// short (R stores each) and carry no loop: measured on MI355X this shape streams writes faster than
+// longer-lived or persistent waves.
 // ------------------------------------------------------------------------------------------------
-template <int BITS, int NV, int RL>
-__global__ __launch_bounds__(kQBlock) void unpack_dequant_rows16_kernel(
-    const uint8_t *__restrict__ q, float *__restrict__ x, const ParamBuf pb,
-    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
+template <int BITS, int R, bool POW2, bool SEGMENTED>
+__global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_kernel(
+    const uint8_t *__restrict__ q, float *__restrict__ x, const ParamBuf pb, const int32_t *__restrict__ seg,
+    const int32_t *__restrict__ pseg, int P, int G /* float4 per row */, int g_shift, int64_t n_vec) {
     constexpr int EPB = 8 / BITS;
-    constexpr int VEC = 4;
     constexpr uint32_t MASK = (1u << BITS) - 1u;
-    const int lane = threadIdx.x & 63, d = lane >> 4, l16 = lane & 15;
-    const int unit = blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
-    if (unit >= n_units) return;
-    const int shift = (EPB - 1 - (d % EPB)) * BITS;
-
-    int64_t row[RL];
-    bool valid[RL];
-    uint32_t words[RL][NV];
-    float2 ps[RL];
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
+    const int64_t base = wave * (R * 64) + lane;
+    uint32_t word[R];
+    float2 ps[R];
+    int shift[R];
 #pragma unroll
-    for (int rl = 0; rl < RL; ++rl) {
-        const int pr = (unit * RL + rl) * 4 + d;
-        const int g = pr / EPB, k = pr % EPB;
-        valid[rl] = false;
-        row[rl] = 0;
-        ps[rl] = make_float2(0.0f, 0.0f);
-        if (g < n_packed) {
-            const int p = P == 1 ? 0 : find_segment(pseg, P, g);
-            row[rl] = (int64_t)seg[p] + (int64_t)(g - pseg[p]) * EPB + k;
-            valid[rl] = row[rl] < seg[p + 1];
+    for (int u = 0; u < R; ++u) {
+        const int64_t i = base + u * 64;
+        word[u] = 0;
+        ps[u] = make_float2(0.0f, 0.0f);
+        shift[u] = 0;
+        if (i >= n_vec) continue;
+        int row, c;
+        if constexpr (POW2) {
+            row = (int)(i >> g_shift);
+            c = (int)(i & (G - 1));
+        } else {
+            row = (int)(i / G);
+            c = (int)(i - (int64_t)row * G);
         }
-        if (valid[rl]) {
-            ps[rl] = load_params(pb, row[rl]);
-            const uint8_t *qr = q + (int64_t)g * F;
-#pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                const int off = (v * 16 + l16) * VEC;
-                if (off < F) words[rl][v] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(qr + off));
+        int slot = row;
+        if constexpr (SEGMENTED) {  // sub-byte codes and more than one segment: segments start on packed-row boundaries
+            int lo = 0, hi = P - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (seg[mid + 1] > row) hi = mid; else lo = mid + 1;
             }
+            slot = pseg[lo] * EPB + (row - seg[lo]);
         }
+        ps[u] = load_params(pb, row);
+        shift[u] = (EPB - 1 - (slot % EPB)) * BITS;
+        word[u] = reinterpret_cast<const uint32_t *>(q)[(int64_t)(slot / EPB) * G + c];  // cacheable on purpose
     }
 #pragma unroll
-    for (int rl = 0; rl < RL; ++rl) {
-        if (!valid[rl]) continue;
-        float *xr = x + row[rl] * F;
+    for (int u = 0; u < R; ++u) {
+        const int64_t i = base + u * 64;
+        if (i >= n_vec) continue;
+        float o[4];
 #pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int off = (v * 16 + l16) * VEC;
-            if (off >= F) continue;
-            float o[VEC];
-#pragma unroll
-            for (int e = 0; e < VEC; ++e)
-                o[e] = fmaf((float)((words[rl][v] >> (8 * e + shift)) & MASK), ps[rl].y, ps[rl].x);
-            vec_store_nt<VEC>(xr + off, o);
-        }
+        for (int e = 0; e < 4; ++e) o[e] = fmaf((float)((word[u] >> (8 * e + shift[u])) & MASK), ps[u].y, ps[u].x);
+        vec_store_nt<4>(x + i * 4, o);
     }
 }
 
@@ -713,6 +713,7 @@ struct RowsArgs {
     ParamBuf params;                                                 // written by quantize, read by dequantize
     const int32_t *seg; const int32_t *pseg; int P; int n_packed; int F; bool quantize;
     bool layout16;        // diagnostic switch: one fp32 row per 16 lanes (default) vs per lane group
+    bool flat;            // dequantize over the flat output (default) vs the row-tiled kernels
     bool exact_division;  // diagnostic: IEEE division for every element (the results are identical either way)
 };
 
@@ -750,16 +751,36 @@ static void launch_quant16(const RowsArgs &a, hipStream_t st) {
                            a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
 }
 
-template <int BITS, int NV>
-static void launch_dequant16(const RowsArgs &a, hipStream_t st) {
-    constexpr int RL = NV >= 4 ? 1 : 4 / NV;
-    constexpr int EPB = 8 / BITS;
-    const int64_t padded = (int64_t)a.n_packed * EPB;
-    const int n_units = (int)((padded + 4 * RL - 1) / (4 * RL));
-    const int nb = (n_units + kQBlock / 64 - 1) / (kQBlock / 64);
+template <int BITS, int R>
+static void launch_dequant_flat_r(const RowsArgs &a, int64_t n_rows, hipStream_t st) {
+    const int G = a.F / 4;
+    const int64_t n_vec = n_rows * G;
+    const int64_t n_waves = (n_vec + R * 64 - 1) / (R * 64);
+    const unsigned nb = (unsigned)((n_waves + kQBlock / 64 - 1) / (kQBlock / 64));
+    const bool pow2 = (G & (G - 1)) == 0;
+    int g_shift = 0;
+    while ((1 << g_shift) < G) ++g_shift;
+    const bool segmented = BITS != 8 && a.P > 1;
     ProfScope prof(K_UNPACK_DEQUANT_ROWS, st);
-    hipLaunchKernelGGL((unpack_dequant_rows16_kernel<BITS, NV, RL>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, a.x_out,
-                       a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+#define SGNN_FLAT(POW2, SEGM)                                                                                        \
+    hipLaunchKernelGGL((unpack_dequant_flat_kernel<BITS, R, POW2, SEGM>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, \
+                       a.x_out, a.params, a.seg, a.pseg, a.P, G, g_shift, n_vec)
+    if (pow2 && segmented) SGNN_FLAT(true, true);
+    else if (pow2) SGNN_FLAT(true, false);
+    else if (segmented) SGNN_FLAT(false, true);
+    else SGNN_FLAT(false, false);
+#undef SGNN_FLAT
+}
+
+// Measured on MI355X (1 M x 256, 2 M x 128, 1 M x 64, 400 k x 600): ordinary (cacheable) loads of the
+// packed words beat non-temporal ones by 15-40 % (rows that share a word hit in cache, and the
+// write stream is not disturbed), and the shortest waves win: one 1-KB store per wave for sub-byte
+// codes on power-of-two widths, two otherwise.
+template <int BITS>
+static void launch_dequant_flat(const RowsArgs &a, int64_t n_rows, hipStream_t st) {
+    const int G = a.F / 4;
+    if (BITS != 8 && (G & (G - 1)) == 0) launch_dequant_flat_r<BITS, 1>(a, n_rows, st);
+    else launch_dequant_flat_r<BITS, 2>(a, n_rows, st);
 }
 
 template <int BITS>
@@ -783,15 +804,6 @@ static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
             if (nvec <= 64) return launch_quant16<BITS, 4>(a, st);
             if (nvec <= 128) return launch_quant16<BITS, 8>(a, st);
             if (nvec <= 256) return launch_quant16<BITS, 16>(a, st);
-        }
-        // Measured on MI355X: at int2 one packed word feeds four fp32 rows and the group-per-packed-row
-        // kernel (one load, four whole-row stores) wins; at int4 / int8 the row-per-16-lanes kernel does.
-        if (!a.quantize && a.layout16 && BITS != 2) {
-            if (nvec <= 16) return launch_dequant16<BITS, 1>(a, st);
-            if (nvec <= 32) return launch_dequant16<BITS, 2>(a, st);
-            if (nvec <= 64) return launch_dequant16<BITS, 4>(a, st);
-            if (nvec <= 128) return launch_dequant16<BITS, 8>(a, st);
-            if (nvec <= 256) return launch_dequant16<BITS, 16>(a, st);
         }
     }
     if (nvec <= 16) return launch_rows<BITS, VEC, 16, 1>(a, st);
@@ -830,7 +842,11 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
     if (a.F % 4 == 0 && ld % 4 == 0 && aligned(fp32_ptr, 16) && aligned(u8_ptr, 4)) vec = 4;
     else if (a.F % 2 == 0 && ld % 2 == 0 && aligned(fp32_ptr, 8) && aligned(u8_ptr, 2)) vec = 2;
     SGNN_REQUIRE(aligned(a.params.p, a.params.bf16 ? 4 : 8), "params must be %d-byte aligned", a.params.bf16 ? 4 : 8);
-    if (bits == 8) dispatch_rows<8>(vec, a, st);
+    if (!a.quantize && vec == 4 && a.flat) {
+        if (bits == 8) launch_dequant_flat<8>(a, n_rows, st);
+        else if (bits == 4) launch_dequant_flat<4>(a, n_rows, st);
+        else launch_dequant_flat<2>(a, n_rows, st);
+    } else if (bits == 8) dispatch_rows<8>(vec, a, st);
     else if (bits == 4) dispatch_rows<4>(vec, a, st);
     else dispatch_rows<2>(vec, a, st);
     SGNN_HIP_CHECK(hipGetLastError());
@@ -895,6 +911,7 @@ static int unpack_dequant_rows_impl(const uint8_t *q, float *x, const void *para
     a.q_in = q; a.x_out = x; a.params = ParamBuf{const_cast<void *>(params), params_bf16}; a.seg = seg; a.pseg = pseg;
     a.P = P; a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = false;
     { const char *e = getenv("SGNN_QUANT_LAYOUT16"); a.layout16 = !(e && e[0] == '0'); }
+    { const char *e = getenv("SGNN_DEQUANT_FLAT"); a.flat = !(e && e[0] == '0'); }
     return run_rows(a, bits, n_rows, x, q, (hipStream_t)stream);
 }
 

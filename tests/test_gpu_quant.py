@@ -323,3 +323,27 @@ def test_bf16_params_equal_torch_casts(bits, F):
     ops.dequantize_tensor_for_all_procs(q16, a, p16, wr, 2, bits)
     ops.dequantize_tensor_for_all_procs(q16, b, p16.to(torch.float32), wr, 2, bits)
     assert torch.equal(a.nan_to_num(1.5, 2.5, 3.5), b.nan_to_num(1.5, 2.5, 3.5))
+
+
+@pytest.mark.parametrize("bits", [8, 4, 2])
+@pytest.mark.parametrize("F", [4, 64, 100, 128, 256, 600, 1028, 2052])
+def test_flat_and_row_tiled_dequantizers_agree(bits, F, monkeypatch):
+    """The flat-output kernel (default) and the row-tiled kernels are two decompositions of the same
+    arithmetic: same bits out, ragged multi-segment tables included."""
+    from super_gnn_amd import supergnn_ops as ops
+    gen = torch.Generator().manual_seed(bits * 7 + F)
+    n = 3001
+    x = torch.randn(n, F, generator=gen).cuda()
+    for wr in ([0, n], [0, 1, 2, 2, 777, 2998, n]):
+        wr_t = torch.tensor(wr, dtype=torch.int32)
+        P = len(wr) - 1
+        npk = sum(-(-(b - a) // (8 // bits)) for a, b in zip(wr[:-1], wr[1:]))
+        q = torch.zeros((npk, F), dtype=torch.uint8, device="cuda"); prm = torch.zeros((n, 2), device="cuda")
+        ops.quantize_tensor_for_all_procs(x, q, prm, wr_t, P, bits)
+        outs = []
+        for flat in ("1", "0"):
+            monkeypatch.setenv("SGNN_DEQUANT_FLAT", flat)
+            o = torch.full((n, F), 7.0, device="cuda")
+            ops.dequantize_tensor_for_all_procs(q, o, prm, wr_t, P, bits)
+            outs.append(o)
+        assert torch.equal(outs[0], outs[1])
