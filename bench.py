@@ -65,6 +65,27 @@ def time_steps(fn, steps, warmup):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def time_reps_events(fn, reps, warmup, flush=None):
+    """Per-repetition device times (ms) from event pairs on the current stream; ``flush`` (a
+    callable that overwrites a buffer larger than L2 + Infinity Cache) runs before each repetition,
+    outside the timed pair."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    times = []
+    for _ in range(reps):
+        if flush is not None:
+            flush()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        times.append(a.elapsed_time(b))
+    times.sort()
+    return {"median_ms": round(times[len(times) // 2], 4), "min_ms": round(times[0], 4)}
+
+
 def build_headline_graph(nodes, und_edges, F, device):
     import torch
     from super_gnn_amd import synth
@@ -151,7 +172,7 @@ def main():
     ap.add_argument("--uniform-rows", type=int, default=0, help="diagnostic: replace the R-MAT graph by uniform random "
                     "rows of --uniform-degree neighbours over --nodes columns")
     ap.add_argument("--uniform-degree", type=int, default=25)
-    ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy", "prepost", "sbm", "aggregate", "sage"],
+    ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy", "prepost", "sbm", "aggregate", "sage", "small"],
                     help="rmat: headline SpMM (default); quant: int2 quantize+pack as the step; copy: streaming copy; "
                          "prepost: one partition with packed remote rows, fused vs separate; sbm: dense-degree graph, F=602")
     ap.add_argument("--local-nodes", type=int, default=8_000_000)
@@ -307,6 +328,12 @@ def main():
             extra["spmm_mean_GEdges_per_s"] = round(nnz / ms_mean / 1e6, 3)
             extra["spmm_mean_gather_GBps"] = round(spmm_gather_bytes(nnz, M, F, False, True, True) / ms_mean / 1e6, 1)
             del out2
+        if not args.no_extras:
+            scratch = torch.empty(192 * 1024 * 1024, device=dev)   # 768 MB > 8 x 4 MB L2 + 256 MB Infinity Cache
+            extra["spmm_warm"] = time_reps_events(step, 20, 5)
+            extra["spmm_cache_flushed"] = time_reps_events(step, 20, 2, flush=lambda: scratch.fill_(1.0))
+            log(f"[bench] weighted sum per repetition: warm {extra['spmm_warm']}, caches flushed before each {extra['spmm_cache_flushed']}")
+            del scratch
         extra["spmm_total_gather_GBps"] = round(b_total / ms / 1e6, 1)
         extra["spmm_total_frac_of_hbm_peak"] = round(b_total / ms / 1e6 / HBM_PEAK_GBPS, 4)
         extra["spmm_GFLOPs"] = round(2.0 * nnz * F / ms / 1e6, 1)
@@ -320,6 +347,45 @@ def main():
                                "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl),
                                "kernel": dom, "kernel_avg_ms": round(dom_ms, 5), "algorithmic_bytes": int(dom_bytes)},
                   "cpu_baseline": None if args.no_cpu else cpu_baseline_spmm(rowptr, col, w, x)}
+
+    # ---- the small CPU-runnable configuration: cache-resident, so GEdges/s only -----------------
+    if args.workload == "small":
+        N, F = 10_000, 128
+        g = torch.Generator().manual_seed(0)
+        col = torch.randint(0, N, (N, 16), generator=g)
+        col = torch.sort(torch.cat([col, torch.arange(N).unsqueeze(1)], dim=1), dim=1).values.reshape(-1)
+        rowptr = 17 * torch.arange(N + 1, dtype=torch.int64)
+        x = torch.randn(N, F, generator=g)
+        w = torch.ones(col.numel())
+        d_rowptr, d_col, d_w, d_x = rowptr.to(dev), col.to(torch.int32).to(dev), w.to(dev), x.to(dev)
+        plan = ops.SpmmPlan(d_rowptr, d_col, N)
+        out = torch.zeros(N, F, device=dev)
+        step = lambda: plan.run(d_w, d_x, out, accumulate=True)  # noqa: E731
+        _lib.profile_start()
+        ms = time_steps(step, args.steps, args.warmup)
+        prof = _lib.profile_stop()
+        k_ms = prof["spmm_short_kernel"][1] / prof["spmm_short_kernel"][0]
+        nnz = col.numel()
+        b = spmm_gather_bytes(nnz, N, F, weighted=True, accumulate=True, mean=False)
+        xq = torch.randn(2000, F, generator=g).to(dev)
+        q = torch.empty(2000, F, dtype=torch.uint8, device=dev); pq = torch.empty(2000, 2, device=dev)
+        seg1 = torch.tensor([0, 2000], dtype=torch.int32)
+        ms_q = time_steps(lambda: ops.quantize_tensor_for_all_procs(xq, q, pq, seg1, 1, 8), 50, 10)
+        cpu = None
+        if not args.no_cpu:
+            cpu = cpu_baseline_spmm(rowptr, col, w, x, reps=20)
+            nt = torch.get_num_threads()
+            torch.set_num_threads(1); os.environ["OMP_NUM_THREADS"] = "1"
+            cpu1 = cpu_baseline_spmm(rowptr, col, w, x, reps=5)
+            torch.set_num_threads(nt)
+            extra["cpu_1_thread_GEdges_per_s"] = round(cpu1["value"], 4)
+        extra.update({"kernel_ms": round(k_ms, 5), "kernel_GEdges_per_s": round(nnz / k_ms / 1e6, 2),
+                      "kernel_gather_GBps_cache_resident": round(b / k_ms / 1e6, 1),
+                      "quant_int8_2000x128_us_per_call": round(ms_q * 1e3, 2)})
+        log(f"[bench] small: {ms * 1e3:.1f} us/step wall, kernel {k_ms * 1e3:.1f} us = {nnz / k_ms / 1e6:.1f} GEdges/s; int8 quantize 2000x128 {ms_q * 1e3:.1f} us/call")
+        result = {"metric": "SpMM GEdges/s (10k nodes x 17 edges, F=128, cache-resident)", "value": round(nnz / ms / 1e6, 4),
+                  "unit": "GEdges/s", "config": {"workload": f"small_uniform_{N}n_{nnz}e_F{F}_sum"}, "ms_per_step": ms,
+                  "dtype": "f32", "roofline": None, "cpu_baseline": cpu}
 
     # ---- one partition in pre/post-aggregation mode: remote rows arrive int2-packed -------------
     if args.workload == "prepost":

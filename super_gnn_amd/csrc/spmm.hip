@@ -30,6 +30,7 @@ namespace sgnn {
 
 constexpr int kBlock = 256;
 constexpr int kDefaultLongThreshold = 128;  // rows with more edges go to the class-partitioned piece path
+constexpr int kChunkGroupsWanted = 16384;
 constexpr int kDefaultPieceEdges = 32;      // minimum edges per piece of a long row
 constexpr int kPopularColumns = 16384;      // size of the "popular" column set the plan looks at
 constexpr double kPartitionMinShare = 0.02; // below this share of all edges (popularity ~uniform) leave the long rows as they are
@@ -659,7 +660,14 @@ struct sgnn_spmm_plan {
 // `target` edges each, never containing a long row, starting and ending on a non-empty row.
 static int build_chunks(sgnn_spmm_plan *p, int which, hipStream_t st) {
     const int limit = which == 0 ? 7 : which == 1 ? 15 : 31;
-    const int target = env_int("SGNN_SPMM_CHUNK_EDGES", 128);
+    // About 128 edges per chunk on large matrices (fewer, longer-lived lane groups stream best), but
+    // never so few chunks that the chip idles: a small matrix is cut finer, down to 16 edges, until
+    // there are about kChunkGroupsWanted lane groups to spread over the 256 CUs.
+    int target = env_int("SGNN_SPMM_CHUNK_EDGES", 0);
+    if (target <= 0) {
+        const int64_t short_edges = p->nnz - p->long_edges;
+        target = (int)std::min<int64_t>(128, std::max<int64_t>(16, short_edges / env_int("SGNN_SPMM_CHUNK_GROUPS", kChunkGroupsWanted)));
+    }
     const std::vector<int64_t> &rp = p->h_rowptr;
     std::vector<int2> out;
     const int64_t M = p->M;

@@ -347,3 +347,21 @@ def test_flat_and_row_tiled_dequantizers_agree(bits, F, monkeypatch):
             ops.dequantize_tensor_for_all_procs(q, o, prm, wr_t, P, bits)
             outs.append(o)
         assert torch.equal(outs[0], outs[1])
+
+
+def test_cpu_runnable_configuration_int8_boundary_rows():
+    """2 000 boundary rows x 128 N(0,1) features, int8, one segment: bytes and params bit-exact,
+    dequantized floats within one rounding of code*scale."""
+    from super_gnn_amd import QuantizerForPureBits
+    x = torch.randn(2000, 128, generator=torch.Generator().manual_seed(0))
+    seg = np.array([0, 2000], np.int32)
+    q_ref, p_ref = orc.quant_rows(x.numpy(), seg, 8)
+    q = torch.zeros(2000 * 128, dtype=torch.uint8, device="cuda"); p = torch.zeros(2000, 2, device="cuda")
+    QuantizerForPureBits.quantize_fp32_to_intX(x.cuda(), q, p, 8)
+    assert np.array_equal(q.cpu().numpy().reshape(2000, 128), q_ref) and np.array_equal(p.cpu().numpy(), p_ref)
+    back = torch.zeros(2000, 128, device="cuda")
+    QuantizerForPureBits.dequantize_intX_to_fp32(q, back, p, 8)
+    want = orc.dequant_rows(q_ref, p_ref, seg, 8, 128)
+    tol = dequant_atol(p_ref[:, 0], p_ref[:, 1], 8)[:, None]
+    assert np.all(np.abs(back.cpu().numpy() - want) <= tol)
+    assert np.all(np.abs(back.cpu().numpy() - x.numpy()) <= p_ref[:, 1:2] * 0.5 * (1 + 1e-6) + 4 * tol)

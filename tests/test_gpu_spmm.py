@@ -263,3 +263,35 @@ def test_long_row_modes_agree_and_auto_choice(mode, monkeypatch):
         gu, plan_u = _run_gpu(rowptr_u, col_u, val_u, xu, zu, accumulate=True)
         assert plan_u.info()["partitioned"] == 0 and 0 < plan_u.info()["top_share_ppm"] < 100000
         _assert_close(gu, wu, orc.spmm_f64(rowptr_u, col_u, val_u, xu), _abs_sum64(rowptr_u, col_u, val_u, xu), np.diff(rowptr_u), what="uniform")
+
+
+def _cpu_runnable_case():
+    """The small reference-runnable configuration: 10 000 nodes, 16 random neighbours + a self loop
+    per row (sorted, duplicates kept), unit weights, 10 000 x 128 N(0,1) features, sum into zeros."""
+    N = 10_000
+    g = torch.Generator().manual_seed(0)
+    col = torch.randint(0, N, (N, 16), generator=g)
+    col = torch.sort(torch.cat([col, torch.arange(N).unsqueeze(1)], dim=1), dim=1).values.reshape(-1)
+    rowptr = 17 * torch.arange(N + 1, dtype=torch.int64)
+    x = torch.randn(N, 128, generator=g)
+    return rowptr, col, torch.ones(col.numel()), x, g
+
+
+def test_cpu_runnable_configuration_is_bit_identical():
+    """Every row has 17 edges (short-row path): the GPU performs the reference's fma chain, so the
+    result equals the CPU restatement bit for bit, through the reference's own call signature."""
+    from super_gnn_amd import SparseTensor, SPMM_forward
+    rowptr, col, val, x, _ = _cpu_runnable_case()
+    want = np.zeros((10_000, 128), np.float32)
+    orc.spmm_accumulate(rowptr.numpy(), col.numpy(), val.numpy(), x.numpy(), want)
+    adj = SparseTensor(rowptr=rowptr, col=col, value=val, sparse_sizes=(10_000, 10_000)).cuda()
+    out = torch.zeros(10_000, 128, device="cuda")
+    SPMM_forward(adj, x.cuda(), out)
+    assert np.array_equal(out.cpu().numpy(), want)
+    ref = orc.ref_ops()
+    if ref is not None:   # the reference's own x86 extension, when it was built on this host
+        got = torch.zeros(10_000, 128)
+        T = torch.get_num_threads()     # the reference reads one row range per OpenMP thread (spmm.cpp:408)
+        split = torch.tensor([10_000 * t // T for t in range(T + 1)], dtype=torch.int32)
+        ref.spmm(rowptr, col, val, x, got, 10_000, split, torch.tensor([0, 128], dtype=torch.int32))
+        assert np.array_equal(got.numpy(), want)
