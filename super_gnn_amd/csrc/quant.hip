@@ -89,6 +89,22 @@ __device__ __forceinline__ int find_segment(const int32_t *__restrict__ pseg, in
     return lo;
 }
 
+// First fp32 row held by packed row g, and the end of the segment it belongs to.  With a single
+// segment (single_rows >= 0, the row count) nothing is read from memory, so a wave's first loads are
+// its data loads.
+__device__ __forceinline__ void locate_packed_row(const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg,
+                                                  int P, int64_t single_rows, int g, int epb, int64_t &row0,
+                                                  int64_t &rend) {
+    if (single_rows >= 0) {
+        row0 = (int64_t)g * epb;
+        rend = single_rows;
+    } else {
+        const int p = find_segment(pseg, P, g);
+        row0 = (int64_t)seg[p] + (int64_t)(g - pseg[p]) * epb;
+        rend = seg[p + 1];
+    }
+}
+
 // code = RNE((x - zp) / scale), IEEE subtraction and division (no reciprocal shortcut).
 __device__ __forceinline__ uint32_t quant_code(float x, float zp, float sc) {
     const float q = (x - zp) / sc;
@@ -102,7 +118,8 @@ __device__ __forceinline__ uint32_t quant_code(float x, float zp, float sc) {
 template <int BITS, int VEC, int G, int NV, bool kForceExactDivision>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
     const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
-    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F,
+    int n_units) {
     constexpr int EPB = 8 / BITS;
     constexpr int R = kRowsPerGroup;
     constexpr int NPR = R / EPB;  // packed rows per group
@@ -118,9 +135,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
         const int gp = unit * NPR + pi;
         int64_t row0 = 0, rend = 0;
         if (gp < n_packed) {
-            const int p = P == 1 ? 0 : find_segment(pseg, P, gp);
-            row0 = (int64_t)seg[p] + (int64_t)(gp - pseg[p]) * EPB;
-            rend = seg[p + 1];
+            locate_packed_row(seg, pseg, P, single_rows, gp, EPB, row0, rend);
         }
 #pragma unroll
         for (int k = 0; k < EPB; ++k) {
@@ -285,7 +300,8 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
 template <int BITS, int NV, int RL, bool kForceExactDivision>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
     const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
-    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F,
+    int n_units) {
     constexpr int EPB = 8 / BITS;
     constexpr int VEC = 4;
     const int lane = threadIdx.x & 63, d = lane >> 4, l16 = lane & 15;
@@ -303,9 +319,10 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
         valid[rl] = false;
         row[rl] = 0;
         if (g < n_packed) {
-            const int p = P == 1 ? 0 : find_segment(pseg, P, g);
-            row[rl] = (int64_t)seg[p] + (int64_t)(g - pseg[p]) * EPB + k;
-            valid[rl] = row[rl] < seg[p + 1];
+            int64_t row0, rend;
+            locate_packed_row(seg, pseg, P, single_rows, g, EPB, row0, rend);
+            row[rl] = row0 + k;
+            valid[rl] = row[rl] < rend;
         }
     }
     int off[NV];
@@ -436,7 +453,8 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
 template <int BITS, int VEC, int G, int NV>
 __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_kernel(
     const uint8_t *__restrict__ q, float *__restrict__ x, const ParamBuf pb,
-    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F, int n_units) {
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F,
+    int n_units) {
     constexpr int EPB = 8 / BITS;
     constexpr int R = kRowsPerGroup;
     constexpr int NPR = R / EPB;
@@ -450,9 +468,8 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_kernel(
     for (int pi = 0; pi < NPR; ++pi) {
         const int gp = unit * NPR + pi;
         if (gp >= n_packed) continue;
-        const int p = P == 1 ? 0 : find_segment(pseg, P, gp);
-        const int64_t row0 = (int64_t)seg[p] + (int64_t)(gp - pseg[p]) * EPB;
-        const int64_t rend = seg[p + 1];
+        int64_t row0, rend;
+        locate_packed_row(seg, pseg, P, single_rows, gp, EPB, row0, rend);
         const uint8_t *qr = q + (int64_t)gp * F;
         float zp[EPB], sc[EPB];
 #pragma unroll
@@ -554,14 +571,13 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_kernel(
 template <int BITS>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows_wide_kernel(
     const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
-    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F) {
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F) {
     constexpr int EPB = 8 / BITS;
     const int lane = threadIdx.x & 63;
     const int gp = blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
     if (gp >= n_packed) return;
-    const int p = P == 1 ? 0 : find_segment(pseg, P, gp);
-    const int64_t row0 = (int64_t)seg[p] + (int64_t)(gp - pseg[p]) * EPB;
-    const int64_t rend = seg[p + 1];
+    int64_t row0, rend;
+    locate_packed_row(seg, pseg, P, single_rows, gp, EPB, row0, rend);
     float zp[EPB], sc[EPB];
 #pragma unroll
     for (int k = 0; k < EPB; ++k) {
@@ -604,15 +620,14 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_wide_kernel(
 template <int BITS>
 __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_wide_kernel(
     const uint8_t *__restrict__ q, float *__restrict__ x, const ParamBuf pb,
-    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int n_packed, int F) {
+    const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F) {
     constexpr int EPB = 8 / BITS;
     constexpr uint32_t MASK = (1u << BITS) - 1u;
     const int lane = threadIdx.x & 63;
     const int gp = blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
     if (gp >= n_packed) return;
-    const int p = P == 1 ? 0 : find_segment(pseg, P, gp);
-    const int64_t row0 = (int64_t)seg[p] + (int64_t)(gp - pseg[p]) * EPB;
-    const int64_t rend = seg[p + 1];
+    int64_t row0, rend;
+    locate_packed_row(seg, pseg, P, single_rows, gp, EPB, row0, rend);
     const uint8_t *qr = q + (int64_t)gp * F;
 #pragma unroll
     for (int k = 0; k < EPB; ++k) {
@@ -712,6 +727,7 @@ struct RowsArgs {
     const uint8_t *q_in; float *x_out;                               // dequantize
     ParamBuf params;                                                 // written by quantize, read by dequantize
     const int32_t *seg; const int32_t *pseg; int P; int n_packed; int F; bool quantize;
+    int64_t single_rows;  // the row count when P == 1 (kernels then read no segment table), else -1
     bool layout16;        // diagnostic switch: one fp32 row per 16 lanes (default) vs per lane group
     bool flat;            // dequantize over the flat output (default) vs the row-tiled kernels
     bool exact_division;  // diagnostic: IEEE division for every element (the results are identical either way)
@@ -726,13 +742,13 @@ static void launch_rows(const RowsArgs &a, hipStream_t st) {
     ProfScope prof(a.quantize ? K_QUANT_PACK_ROWS : K_UNPACK_DEQUANT_ROWS, st);
     if (a.quantize && a.exact_division)
         hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
-                           a.q_out, a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                           a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
     else if (a.quantize)
         hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV, false>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
-                           a.q_out, a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                           a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
     else
         hipLaunchKernelGGL((unpack_dequant_rows_kernel<BITS, VEC, G, NV>), dim3(nb), dim3(kQBlock), 0, st, a.q_in,
-                           a.x_out, a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                           a.x_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
 template <int BITS, int NV>
@@ -745,10 +761,10 @@ static void launch_quant16(const RowsArgs &a, hipStream_t st) {
     ProfScope prof(K_QUANT_PACK_ROWS, st);
     if (a.exact_division)
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
-                           a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                           a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
     else
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
-                           a.params, a.seg, a.pseg, a.P, a.n_packed, a.F, n_units);
+                           a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
 template <int BITS, int R>
@@ -789,10 +805,10 @@ static void launch_rows_wide(const RowsArgs &a, hipStream_t st) {
     ProfScope prof(a.quantize ? K_QUANT_PACK_ROWS : K_UNPACK_DEQUANT_ROWS, st);
     if (a.quantize)
         hipLaunchKernelGGL((quant_pack_rows_wide_kernel<BITS>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
-                           a.params, a.seg, a.pseg, a.P, a.n_packed, a.F);
+                           a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F);
     else
         hipLaunchKernelGGL((unpack_dequant_rows_wide_kernel<BITS>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, a.x_out,
-                           a.params, a.seg, a.pseg, a.P, a.n_packed, a.F);
+                           a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F);
 }
 
 template <int BITS, int VEC>
@@ -834,6 +850,9 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
     SGNN_REQUIRE(a.F > 0, "feature width F=%d out of range", a.F);
     SGNN_REQUIRE(n_rows >= 0 && a.n_packed >= 0, "negative row count");
     if (n_rows == 0 || a.n_packed == 0) return SGNN_OK;
+    SGNN_REQUIRE(a.P > 1 || (int64_t)a.n_packed == (n_rows + 8 / bits - 1) / (8 / bits),
+                 "one segment of %lld rows needs %lld packed rows, got %d", (long long)n_rows,
+                 (long long)((n_rows + 8 / bits - 1) / (8 / bits)), a.n_packed);
     SGNN_REQUIRE(fp32_ptr && u8_ptr && a.seg && a.pseg, "null pointer argument");
     SGNN_REQUIRE(a.params.p != nullptr, "params is null");
     SGNN_REQUIRE((int64_t)a.n_packed * (8 / bits) < (int64_t)INT32_MAX, "too many rows for 32-bit row units");
@@ -897,6 +916,7 @@ static int quant_pack_rows_impl(const RowSrc &src, uint8_t *q, void *params, int
     RowsArgs a{};
     a.x_in = src; a.q_out = q; a.params = ParamBuf{params, params_bf16}; a.seg = seg; a.pseg = pseg; a.P = P;
     a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = true;
+    a.single_rows = P == 1 ? n_rows : -1;
     { const char *e = getenv("SGNN_QUANT_EXACT_DIV"); a.exact_division = e && e[0] == '1'; }
     { const char *e = getenv("SGNN_QUANT_LAYOUT16"); a.layout16 = !(e && e[0] == '0'); }
     return run_rows(a, bits, n_rows, src.x, q, (hipStream_t)stream);
@@ -910,6 +930,7 @@ static int unpack_dequant_rows_impl(const uint8_t *q, float *x, const void *para
     RowsArgs a{};
     a.q_in = q; a.x_out = x; a.params = ParamBuf{const_cast<void *>(params), params_bf16}; a.seg = seg; a.pseg = pseg;
     a.P = P; a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = false;
+    a.single_rows = P == 1 ? n_rows : -1;
     { const char *e = getenv("SGNN_QUANT_LAYOUT16"); a.layout16 = !(e && e[0] == '0'); }
     { const char *e = getenv("SGNN_DEQUANT_FLAT"); a.flat = !(e && e[0] == '0'); }
     return run_rows(a, bits, n_rows, x, q, (hipStream_t)stream);
