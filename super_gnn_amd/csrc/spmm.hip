@@ -190,7 +190,7 @@ __host__ __device__ constexpr int chunk_row_limit(int G) { return (G < 32 ? G : 
 template <int VEC, int G, int NV, int BITS>
 __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
     const int64_t *__restrict__ rowptr, const int32_t *__restrict__ col, const float *__restrict__ val,
-    const DenseSrc dense, float *__restrict__ out, const int2 *__restrict__ chunks, int n_chunks, int F,
+    const DenseSrc dense, float *__restrict__ out, const int4 *__restrict__ chunks, int n_chunks, int F,
     int64_t ldo, int accumulate, const float *__restrict__ row_div, uint32_t nblocks) {
     constexpr int GPB = kBlock / G;
     constexpr int TILE = G * VEC * NV;
@@ -199,27 +199,32 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
     const int gid = threadIdx.x / G, lig = threadIdx.x % G;
     const int ci = (int)lb * GPB + gid;
     if (ci >= n_chunks) return;
-    int2 ch = chunks[ci];
+    // A chunk record is (first row, row count, first edge, edge count): the column/weight loads
+    // depend on it alone and are issued before the row pointers come back.
+    int4 ch = chunks[ci];
     if constexpr (G == 64) {
         ch.x = __builtin_amdgcn_readfirstlane(ch.x);
         ch.y = __builtin_amdgcn_readfirstlane(ch.y);
+        ch.z = __builtin_amdgcn_readfirstlane(ch.z);
+        ch.w = __builtin_amdgcn_readfirstlane(ch.w);
     }
     const int rb = ch.x, nr = ch.y;  // rows rb .. rb+nr-1, first and last non-empty, 1 <= nr <= limit
-
-    // Lane i holds rowptr[rb+i] relative to the chunk's first edge (lanes >= nr hold the end).
-    const int64_t rp = rowptr[rb + (lig < nr ? lig : nr)];
-    int64_t B = rp;
-    {
-        const int lo = group_bcast_i<G>((int)(uint32_t)rp, 0), hi = group_bcast_i<G>((int)(uint32_t)((uint64_t)rp >> 32), 0);
-        B = (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint32_t)lo);
-    }
-    const int rel = (int)(rp - B);
-    const int rel_next = __shfl_down(rel, 1, G);
-    const uint32_t mask = group_ballot<G>(lig < nr && rel_next > rel);  // bit i: row rb+i has edges
-    const int E = group_bcast_i<G>(rel, nr);
-    const float mydiv = (row_div && lig < nr) ? row_div[rb + lig] : 1.0f;
+    const int64_t B = ch.z;
+    const int E = ch.w;
     const int32_t *colp = col + B;
     const float *valp = val ? val + B : nullptr;
+    int nc0 = 0;
+    float nw0 = 1.0f;
+    if (lig < E) {
+        nc0 = __builtin_nontemporal_load(colp + lig);
+        if (valp) nw0 = __builtin_nontemporal_load(valp + lig);
+    }
+
+    // Lane i holds rowptr[rb+i] relative to the chunk's first edge (lanes >= nr hold the end).
+    const int rel = (int)(rowptr[rb + (lig < nr ? lig : nr)] - B);
+    const int rel_next = __shfl_down(rel, 1, G);
+    const uint32_t mask = group_ballot<G>(lig < nr && rel_next > rel);  // bit i: row rb+i has edges
+    const float mydiv = (row_div && lig < nr) ? row_div[rb + lig] : 1.0f;
 
     for (int f0 = 0; f0 < F; f0 += TILE) {
         int off[NV];
@@ -247,9 +252,9 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
             }
         }
 
-        int nc = 0;
-        float nw = 1.0f;
-        if (lig < E) {
+        int nc = nc0;
+        float nw = nw0;
+        if (f0 > 0 && lig < E) {  // a later feature tile walks the chunk's edges again
             nc = __builtin_nontemporal_load(colp + lig);
             if (valp) nw = __builtin_nontemporal_load(valp + lig);
         }
@@ -358,17 +363,18 @@ __global__ __launch_bounds__(kBlock) void spmm_empty_rows_kernel(const int32_t *
 template <int VEC, int G, int NV, int BITS, bool PERM>
 __global__ __launch_bounds__(kBlock) void spmm_piece_kernel(
     const int32_t *__restrict__ col_long, const int32_t *__restrict__ eperm, const float *__restrict__ val,
-    const DenseSrc dense, float *__restrict__ partial, const int32_t *__restrict__ item_begin,
-    const int32_t *__restrict__ item_len, const int32_t *__restrict__ cls_list, const int32_t *__restrict__ cls_off,
-    int F) {
+    const DenseSrc dense, float *__restrict__ partial, const int4 *__restrict__ cls_work, int cls_stride, int F) {
     constexpr int GPB = kBlock / G;
     constexpr int TILE = G * VEC * NV;
     const int gid = threadIdx.x / G, lig = threadIdx.x % G;
     const int cls = blockIdx.x % kNumXCD;
-    const int idx = cls_off[cls] + (int)(blockIdx.x / kNumXCD) * GPB + gid;
-    if (idx >= cls_off[cls + 1]) return;
-    int item = cls_list[idx];
-    int b = item_begin[item], len = item_len[item];
+    const int slot = (int)(blockIdx.x / kNumXCD) * GPB + gid;
+    if (slot >= cls_stride) return;
+    // One record per piece, (piece id, first edge, edge count): the only load between the start of
+    // the wave and its column loads.  Every class's list is padded to cls_stride records.
+    const int4 w = cls_work[(int64_t)cls * cls_stride + slot];
+    int item = w.x, b = w.y, len = w.z;
+    if (len == 0) return;
     if constexpr (G == 64) {
         item = __builtin_amdgcn_readfirstlane(item);
         b = __builtin_amdgcn_readfirstlane(b);
@@ -539,12 +545,12 @@ __global__ __launch_bounds__(kBlock) void column_popularity_kernel(const int32_t
 // ------------------------------------------------------------------------------------------------
 struct ShortArgs {
     const int64_t *rowptr; const int32_t *col; const float *val; DenseSrc dense; float *out;
-    const int2 *chunks; int n_chunks; const int32_t *empty_rows; int n_empty;
+    const int4 *chunks; int n_chunks; const int32_t *empty_rows; int n_empty;
     int F; int64_t ldo; int accumulate; const float *row_div;
 };
 struct PieceArgs {
     const int32_t *col_long; const int32_t *eperm; const float *val; float *partial;
-    const int32_t *item_begin; const int32_t *item_len; const int32_t *cls_list; const int32_t *cls_off;
+    const int4 *cls_work;
     int max_cls_items; int F;
 };
 struct FinalArgs {
@@ -574,10 +580,10 @@ static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &
             ProfScope prof(BITS == 0 ? K_SPMM_PIECE : K_FUSED_PIECE, st);
             if (s.eperm)
                 hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS, true>), dim3(nb), dim3(kBlock), 0, st, s.col_long,
-                                   s.eperm, s.val, a.dense, s.partial, s.item_begin, s.item_len, s.cls_list, s.cls_off, s.F);
+                                   s.eperm, s.val, a.dense, s.partial, s.cls_work, s.max_cls_items, s.F);
             else
                 hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS, false>), dim3(nb), dim3(kBlock), 0, st, s.col_long,
-                                   s.eperm, s.val, a.dense, s.partial, s.item_begin, s.item_len, s.cls_list, s.cls_off, s.F);
+                                   s.eperm, s.val, a.dense, s.partial, s.cls_work, s.max_cls_items, s.F);
         }
         const uint32_t nb = (uint32_t)((f.n_long + GPB - 1) / GPB);
         ProfScope prof(K_SPMM_LONG_FINAL, st);
@@ -641,10 +647,7 @@ struct sgnn_spmm_plan {
     int32_t *long_pbeg = nullptr;   // [n_long + 1] first piece of each long row
     int32_t *col_long = nullptr;    // [long_edges] columns regrouped by class inside each long row
     int32_t *eperm = nullptr;       // [long_edges] original edge index of each regrouped edge
-    int32_t *item_begin = nullptr;  // [n_items] offset into col_long / eperm
-    int32_t *item_len = nullptr;    // [n_items]
-    int32_t *cls_list = nullptr;    // [n_items] piece ids grouped by class
-    int32_t *cls_off = nullptr;     // [9]
+    int4 *cls_work = nullptr;       // [8 * max_cls_items] (piece id, first edge in col_long / eperm, edges, 0) per class, zero-padded
     float *partial = nullptr;       // [n_items * F], grown on demand
     size_t partial_floats = 0;
     // rows without edges
@@ -652,7 +655,7 @@ struct sgnn_spmm_plan {
     int64_t n_empty = 0;
     // Short-row chunks, one list per chunk row limit (7, 15, 31), built on first use.
     std::vector<int64_t> h_rowptr;
-    int2 *chunks[3] = {nullptr, nullptr, nullptr};
+    int4 *chunks[3] = {nullptr, nullptr, nullptr};
     int64_t n_chunks[3] = {-1, -1, -1};
 };
 
@@ -669,7 +672,7 @@ static int build_chunks(sgnn_spmm_plan *p, int which, hipStream_t st) {
         target = (int)std::min<int64_t>(128, std::max<int64_t>(16, short_edges / env_int("SGNN_SPMM_CHUNK_GROUPS", kChunkGroupsWanted)));
     }
     const std::vector<int64_t> &rp = p->h_rowptr;
-    std::vector<int2> out;
+    std::vector<int4> out;
     const int64_t M = p->M;
     int64_t m = 0;
     while (m < M) {
@@ -684,12 +687,12 @@ static int build_chunks(sgnn_spmm_plan *p, int which, hipStream_t st) {
             edges += d;
             ++m;
         }
-        out.push_back(make_int2((int)start, (int)(last - start + 1)));
+        out.push_back(make_int4((int)start, (int)(last - start + 1), (int)rp[start], (int)(rp[last + 1] - rp[start])));
     }
     p->n_chunks[which] = (int64_t)out.size();
     if (!out.empty()) {
-        SGNN_HIP_CHECK(hipMalloc(&p->chunks[which], sizeof(int2) * out.size()));
-        SGNN_HIP_CHECK(hipMemcpyAsync(p->chunks[which], out.data(), sizeof(int2) * out.size(), hipMemcpyHostToDevice, st));
+        SGNN_HIP_CHECK(hipMalloc(&p->chunks[which], sizeof(int4) * out.size()));
+        SGNN_HIP_CHECK(hipMemcpyAsync(p->chunks[which], out.data(), sizeof(int4) * out.size(), hipMemcpyHostToDevice, st));
         SGNN_HIP_CHECK(hipStreamSynchronize(st));
     }
     return SGNN_OK;
@@ -703,10 +706,7 @@ extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     (void)hipFree(p->long_pbeg);
     if (p->col_long != p->col) (void)hipFree(p->col_long);
     (void)hipFree(p->eperm);
-    (void)hipFree(p->item_begin);
-    (void)hipFree(p->item_len);
-    (void)hipFree(p->cls_list);
-    (void)hipFree(p->cls_off);
+    (void)hipFree(p->cls_work);
     (void)hipFree(p->partial);
     (void)hipFree(p->empty_rows);
     for (int i = 0; i < 3; ++i) (void)hipFree(p->chunks[i]);
@@ -831,7 +831,7 @@ static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void
             p->eperm = nullptr;
         }
 
-        std::vector<int32_t> item_begin, item_len, long_pbeg, cls_off(kNumXCD + 1, 0);
+        std::vector<int32_t> item_begin, item_len, long_pbeg;
         std::vector<std::vector<int32_t>> cls_items(kNumXCD);
         std::vector<uint32_t> item_key;  // partitioned pieces: position of the piece inside its (row, class) run, 16.16
         long_pbeg.push_back(0);
@@ -877,19 +877,15 @@ static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void
                 std::stable_sort(cls_items[c].begin(), cls_items[c].end(),
                                  [&](int32_t a, int32_t b) { return item_key[a] < item_key[b]; });
         }
-        std::vector<int32_t> cls_list;
-        cls_list.reserve(item_begin.size());
-        for (int c = 0; c < kNumXCD; ++c) {
-            cls_off[c] = (int32_t)cls_list.size();
-            cls_list.insert(cls_list.end(), cls_items[c].begin(), cls_items[c].end());
-            p->max_cls_items = std::max<int>(p->max_cls_items, (int)cls_items[c].size());
-        }
-        cls_off[kNumXCD] = (int32_t)cls_list.size();
+        for (int c = 0; c < kNumXCD; ++c) p->max_cls_items = std::max<int>(p->max_cls_items, (int)cls_items[c].size());
+        std::vector<int4> cls_work((size_t)kNumXCD * (size_t)p->max_cls_items, make_int4(0, 0, 0, 0));
+        for (int c = 0; c < kNumXCD; ++c)
+            for (size_t i = 0; i < cls_items[c].size(); ++i) {
+                const int32_t it = cls_items[c][i];
+                cls_work[(size_t)c * p->max_cls_items + i] = make_int4(it, item_begin[it], item_len[it], 0);
+            }
         if ((rc = upload(&p->long_pbeg, long_pbeg, st)) != SGNN_OK) return rc;
-        if ((rc = upload(&p->item_begin, item_begin, st)) != SGNN_OK) return rc;
-        if ((rc = upload(&p->item_len, item_len, st)) != SGNN_OK) return rc;
-        if ((rc = upload(&p->cls_list, cls_list, st)) != SGNN_OK) return rc;
-        if ((rc = upload(&p->cls_off, cls_off, st)) != SGNN_OK) return rc;
+        if ((rc = upload(&p->cls_work, cls_work, st)) != SGNN_OK) return rc;
     }
     SGNN_HIP_CHECK(hipStreamSynchronize(st));  // the host vectors die at return
     return SGNN_OK;
@@ -973,8 +969,7 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     }
     ShortArgs a{p->rowptr, p->col, val, dense, out, p->chunks[which], (int)p->n_chunks[which], p->empty_rows,
                 (int)p->n_empty, (int)F, ldo, accumulate, row_div};
-    PieceArgs s{p->col_long, p->eperm, val, p->partial, p->item_begin, p->item_len, p->cls_list, p->cls_off,
-                p->max_cls_items, (int)F};
+    PieceArgs s{p->col_long, p->eperm, val, p->partial, p->cls_work, p->max_cls_items, (int)F};
     FinalArgs f{p->long_rows, p->long_pbeg, p->partial, out, (int)p->n_long, (int)F, ldo, accumulate, row_div};
     if (bits != 0 && dense.params.bf16) {
         if (bits == 8) dispatch_shape_dq<8 + kBf16Params>(nvec, a, s, f, st);
