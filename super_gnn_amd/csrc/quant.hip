@@ -850,6 +850,8 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
     SGNN_REQUIRE(a.F > 0, "feature width F=%d out of range", a.F);
     SGNN_REQUIRE(n_rows >= 0 && a.n_packed >= 0, "negative row count");
     if (n_rows == 0 || a.n_packed == 0) return SGNN_OK;
+    SGNN_REQUIRE(n_rows * (int64_t)a.F < ((int64_t)1 << 40), "n_rows * F = %lld elements is beyond the supported grid",
+                 (long long)(n_rows * (int64_t)a.F));
     SGNN_REQUIRE(a.P > 1 || (int64_t)a.n_packed == (n_rows + 8 / bits - 1) / (8 / bits),
                  "one segment of %lld rows needs %lld packed rows, got %d", (long long)n_rows,
                  (long long)((n_rows + 8 / bits - 1) / (8 / bits)), a.n_packed);
