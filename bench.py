@@ -39,13 +39,16 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def spmm_gather_bytes(nnz, rows, F, weighted, accumulate, mean):
+def spmm_gather_bytes(nnz, rows, F, weighted, accumulate, mean, empty_rows=0):
     """Algorithmic bytes of one SpMM under the gather model (no cache credit), int32 columns:
-    per edge 4F (dense row) + 4 (col) + 4 (val, if weighted); per row 4F (write) + 8 (rowptr)
-    + 4F when accumulating onto a previous out + 4 for the mean divisor."""
+    per edge 4F (dense row) + 4 (col) + 4 (val, if weighted); per row 8 (rowptr); per row that is
+    written 4F, + 4F when accumulating onto a previous out, + 4 for the mean divisor.  In plain
+    accumulate mode a row without edges is not touched (the reference skips it, spmm.cpp:486), so
+    ``empty_rows`` of the ``rows`` do not count there."""
     per_edge = 4 * F + 4 + (4 if weighted else 0)
-    per_row = 4 * F + 8 + (4 * F if accumulate else 0) + (4 if mean else 0)
-    return nnz * per_edge + rows * per_row
+    touched = rows - (empty_rows if (accumulate and not mean) else 0)
+    per_touched = 4 * F + (4 * F if accumulate else 0) + (4 if mean else 0)
+    return nnz * per_edge + rows * 8 + touched * per_touched
 
 
 def quant_bytes(rows, F, bits):
@@ -306,8 +309,10 @@ def main():
         # dominant kernel: the short-row kernel; its share of the algorithmic bytes
         short_edges = nnz - info["long_edges"]
         short_rows = M - info["long_rows"]
-        b_short = spmm_gather_bytes(short_edges, short_rows, F, weighted=True, accumulate=True, mean=False)
-        b_total = spmm_gather_bytes(nnz, M, F, weighted=True, accumulate=True, mean=False)
+        n_empty = int(((rowptr[1:] - rowptr[:-1]) == 0).sum())
+        b_short = spmm_gather_bytes(short_edges, short_rows, F, weighted=True, accumulate=True, mean=False, empty_rows=n_empty)
+        b_total = spmm_gather_bytes(nnz, M, F, weighted=True, accumulate=True, mean=False, empty_rows=n_empty)
+        extra["empty_rows"] = n_empty
         dom = max(prof, key=lambda k: prof[k][1])
         dom_ms = prof[dom][1] / prof[dom][0]
         if dom == "spmm_short_kernel":
@@ -471,7 +476,8 @@ def main():
         dom_ms = prof[dom][1] / prof[dom][0]
         dom_edges = info["long_edges"] if "piece" in dom else nnz - info["long_edges"]
         dom_bytes = dom_edges * (4 * F + 4)
-        b_total = spmm_gather_bytes(nnz, n, F, weighted=False, accumulate=True, mean=False)
+        b_total = spmm_gather_bytes(nnz, n, F, weighted=False, accumulate=True, mean=False,
+                                    empty_rows=int(((rowptr[1:] - rowptr[:-1]) == 0).sum()))
         extra.update({"kernel_avg_ms": per_kernel, "plan": {k: info[k] for k in ("long_rows", "pieces", "long_edges")},
                       "spmm_total_gather_GBps": round(b_total / ms / 1e6, 1)})
         log(f"[bench] sbm sum: {ms:.3f} ms/step, {nnz / ms / 1e6:.2f} GEdges/s, {b_total / ms / 1e6:.0f} GB/s gather model, {per_kernel}")
