@@ -663,13 +663,13 @@ struct sgnn_spmm_plan {
 // `target` edges each, never containing a long row, starting and ending on a non-empty row.
 static int build_chunks(sgnn_spmm_plan *p, int which, hipStream_t st) {
     const int limit = which == 0 ? 7 : which == 1 ? 15 : 31;
-    // About 128 edges per chunk on large matrices (fewer, longer-lived lane groups stream best), but
-    // never so few chunks that the chip idles: a small matrix is cut finer, down to 16 edges, until
-    // there are about kChunkGroupsWanted lane groups to spread over the 256 CUs.
+    // About 64 edges per chunk on large matrices (measured plateau 32-96 on the power-law graph; 128
+    // is 4 % slower, 256 15 %), and never so few chunks that the chip idles: a small matrix is cut
+    // finer, down to 16 edges, until there are about kChunkGroupsWanted lane groups for the 256 CUs.
     int target = env_int("SGNN_SPMM_CHUNK_EDGES", 0);
     if (target <= 0) {
         const int64_t short_edges = p->nnz - p->long_edges;
-        target = (int)std::min<int64_t>(128, std::max<int64_t>(16, short_edges / env_int("SGNN_SPMM_CHUNK_GROUPS", kChunkGroupsWanted)));
+        target = (int)std::min<int64_t>(64, std::max<int64_t>(16, short_edges / env_int("SGNN_SPMM_CHUNK_GROUPS", kChunkGroupsWanted)));
     }
     const std::vector<int64_t> &rp = p->h_rowptr;
     std::vector<int4> out;
