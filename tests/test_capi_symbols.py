@@ -97,3 +97,29 @@ def test_row_split_matches_the_reference_greedy_rule():
         assert got == literal(rowptr, value, T), (M, T)
     assert disribute_work_for_col(torch.zeros(3, 128), 1).tolist() == [0, 128]
     assert disribute_work_for_col(torch.zeros(3, 10), 4).tolist() == [0, 2, 4, 6, 10]
+
+
+def test_package_fails_loudly_without_the_library(tmp_path):
+    """No CPU fallback: a copy of the package without libsgnn_hip.so must refuse to import."""
+    import shutil
+    import subprocess
+    import sys
+    pkg = os.path.join(ROOT, "super_gnn_amd")
+    shutil.copytree(pkg, tmp_path / "super_gnn_amd",
+                    ignore=shutil.ignore_patterns("*.so", "csrc", "__pycache__", "obj"))
+    r = subprocess.run([sys.executable, "-c", "import super_gnn_amd"], cwd=tmp_path, capture_output=True, text=True,
+                       env={**os.environ, "PYTHONPATH": str(tmp_path)})
+    assert r.returncode != 0
+    assert "libsgnn_hip" in r.stderr
+
+
+def test_product_never_imports_the_oracle():
+    """The oracle is test infrastructure: nothing under super_gnn_amd/ may import or load it."""
+    import re
+    pkg = os.path.join(ROOT, "super_gnn_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp")):
+                text = open(os.path.join(base, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", text, re.M), f
+                assert "liborc" not in text and "oracle/" not in text, f
