@@ -76,6 +76,15 @@ int sgnn_spmm_plan_destroy(sgnn_spmm_plan *plan);
  * it was not measured). */
 int sgnn_spmm_plan_info(const sgnn_spmm_plan *plan, int64_t info[10]);
 
+/* Optional: declare an edge-value array constant until the next bind.  The plan keeps a copy of the
+ * long rows' values in its own (regrouped) edge order, and later sgnn_spmm_csr_f32 /
+ * sgnn_spmm_csr_dq*_f32 calls that pass the SAME pointer read that copy contiguously instead of
+ * going through the edge permutation (-8 % on the long-row kernel of the power-law graph).  The
+ * caller must bind again after changing the array's contents; val == NULL unbinds.  The reference
+ * passes `value` on every call (super_gnn/ops/spmm_kernel.py:60-65) but never changes it after the
+ * graph is built (DataProcessor.py:112,119), which is what this exploits. */
+int sgnn_spmm_plan_bind_values(sgnn_spmm_plan *plan, const float *val, sgnn_stream_t stream);
+
 /* out[M,F] (+)= A[M,K] * x[K,F], fp32, row-major, leading dimensions ldx / ldo (in floats).
  *
  * Replaces supergnn_ops.spmm (super_gnn/ops/csrc/spmm.cpp:594-608):

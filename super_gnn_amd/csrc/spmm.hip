@@ -540,6 +540,12 @@ __global__ __launch_bounds__(kBlock) void column_popularity_kernel(const int32_t
     for (; i < n; i += stride) atomicAdd(popularity + col[i], 1);
 }
 
+__global__ __launch_bounds__(kBlock) void permute_values_kernel(const float *__restrict__ val, const int32_t *__restrict__ eperm,
+                                                                float *__restrict__ dst, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) dst[i] = val[__builtin_nontemporal_load(eperm + i)];
+}
+
 // ------------------------------------------------------------------------------------------------
 // Launch tables.
 // ------------------------------------------------------------------------------------------------
@@ -647,6 +653,8 @@ struct sgnn_spmm_plan {
     int32_t *long_pbeg = nullptr;   // [n_long + 1] first piece of each long row
     int32_t *col_long = nullptr;    // [long_edges] columns regrouped by class inside each long row
     int32_t *eperm = nullptr;       // [long_edges] original edge index of each regrouped edge
+    float *val_long = nullptr;      // [long_edges] bound edge values in regrouped order (sgnn_spmm_plan_bind_values)
+    const float *bound_val = nullptr;  // the caller's array val_long was taken from
     int4 *cls_work = nullptr;       // [8 * max_cls_items] (piece id, first edge in col_long / eperm, edges, 0) per class, zero-padded
     float *partial = nullptr;       // [n_items * F], grown on demand
     size_t partial_floats = 0;
@@ -707,6 +715,7 @@ extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     if (p->col_long != p->col) (void)hipFree(p->col_long);
     (void)hipFree(p->eperm);
     (void)hipFree(p->cls_work);
+    (void)hipFree(p->val_long);
     (void)hipFree(p->partial);
     (void)hipFree(p->empty_rows);
     for (int i = 0; i < 3; ++i) (void)hipFree(p->chunks[i]);
@@ -970,6 +979,10 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     ShortArgs a{p->rowptr, p->col, val, dense, out, p->chunks[which], (int)p->n_chunks[which], p->empty_rows,
                 (int)p->n_empty, (int)F, ldo, accumulate, row_div};
     PieceArgs s{p->col_long, p->eperm, val, p->partial, p->cls_work, p->max_cls_items, (int)F};
+    if (val != nullptr && val == p->bound_val && p->val_long != nullptr) {
+        s.eperm = nullptr;   // values already sit in regrouped order: contiguous reads, no indirection
+        s.val = p->val_long;
+    }
     FinalArgs f{p->long_rows, p->long_pbeg, p->partial, out, (int)p->n_long, (int)F, ldo, accumulate, row_div};
     if (bits != 0 && dense.params.bf16) {
         if (bits == 8) dispatch_shape_dq<8 + kBf16Params>(nvec, a, s, f, st);
@@ -982,6 +995,19 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     else if (vec == 2) dispatch_shape<2>(nvec, a, s, f, st);
     else dispatch_shape<1>(nvec, a, s, f, st);
     SGNN_HIP_CHECK(hipGetLastError());
+    return SGNN_OK;
+}
+
+extern "C" int sgnn_spmm_plan_bind_values(sgnn_spmm_plan *p, const float *val, sgnn_stream_t stream) {
+    SGNN_REQUIRE(p != nullptr, "plan is null");
+    p->bound_val = nullptr;
+    if (val == nullptr || !p->partitioned || p->long_edges == 0) return SGNN_OK;  // nothing to regroup
+    if (p->val_long == nullptr) SGNN_HIP_CHECK(hipMalloc(&p->val_long, sizeof(float) * (size_t)p->long_edges));
+    const int64_t nb = (p->long_edges + kBlock - 1) / kBlock;
+    hipLaunchKernelGGL(permute_values_kernel, dim3((uint32_t)nb), dim3(kBlock), 0, (hipStream_t)stream, val, p->eperm,
+                       p->val_long, p->long_edges);
+    SGNN_HIP_CHECK(hipGetLastError());
+    p->bound_val = val;
     return SGNN_OK;
 }
 

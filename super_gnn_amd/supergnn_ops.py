@@ -106,6 +106,8 @@ class SpmmPlan:
         check(lib.sgnn_spmm_plan_create(_ptr(rp), _ptr(cl), int(cl.dtype == torch.int64), self.M, self.K, self.nnz,
                                         int(long_row_threshold), int(piece_edges), _stream(), ctypes.byref(h)))
         self._h = h
+        self._bound = None   # (value tensor, version) whose long-row values the plan holds in its own order
+        self._seen = None    # (value tensor, version) of the previous call
         self.device = dev
 
     def info(self):
@@ -139,9 +141,29 @@ class SpmmPlan:
         s_out = _Staged(out, dev, writeback=True)
         s_div = _Staged(row_div, dev) if row_div is not None else None
         F = mat.shape[1]
+        if value is not None and value.is_cuda and value.is_contiguous():
+            self._maybe_bind(value)
         check(lib.sgnn_spmm_csr_f32(self._h, _ptr(s_val.dev) if s_val else None, _ptr(s_mat.dev), _ptr(s_out.dev),
                                     F, F, F, int(bool(accumulate)), _ptr(s_div.dev) if s_div else None, _stream()))
         s_out.commit()
+
+    def _maybe_bind(self, value):
+        """Edge values that come back unchanged are bound to the plan on their second use: the plan
+        then keeps the long rows' values in its own edge order (sgnn_spmm_plan_bind_values).
+
+        "Unchanged" = same address and same version counter as a tensor this plan still holds a
+        reference to (so the address cannot have been recycled; a view of it shares its counter).
+        Anything else at the bound address is rebound at once, so the library never reads a stale
+        copy."""
+        def same(ref):
+            return ref is not None and value.data_ptr() == ref[0].data_ptr() and value._version == ref[1]
+        if same(self._bound):
+            return
+        stale = self._bound is not None and value.data_ptr() == self._bound[0].data_ptr()
+        if stale or same(self._seen):
+            check(lib.sgnn_spmm_plan_bind_values(self._h, _ptr(value), _stream()))
+            self._bound = (value, value._version)
+        self._seen = (value, value._version)
 
     def run_quantized(self, value, data_int8, params, segs, bits, out, accumulate=True, row_div=None):
         """out (+)= A @ dequantize(data_int8): the dense operand stays packed (row-group layout,
@@ -170,6 +192,8 @@ class SpmmPlan:
         if row_div is not None:
             _want(row_div, torch.float32, "row_div")
         slots = segs.row_slots(bits)
+        if value is not None and value.is_contiguous():
+            self._maybe_bind(value)
         if bf16:
             check(lib.sgnn_spmm_csr_dq_wire_f32(self._h, _ptr(value), _ptr(data_int8), _ptr(params), 1, _ptr(slots), bits,
                                                 _ptr(out), F, F, int(bool(accumulate)), _ptr(row_div), _stream()))

@@ -295,3 +295,33 @@ def test_cpu_runnable_configuration_is_bit_identical():
         split = torch.tensor([10_000 * t // T for t in range(T + 1)], dtype=torch.int32)
         ref.spmm(rowptr, col, val, x, got, 10_000, split, torch.tensor([0, 128], dtype=torch.int32))
         assert np.array_equal(got.numpy(), want)
+
+
+def test_bound_values_follow_in_place_changes():
+    """Values bound to the plan (second use of the same tensor) give the same bits as unbound ones,
+    and an in-place change of the tensor is picked up by the very next call."""
+    ops = _gpu()
+    rowptr, col, val = random_csr(600, 500, 8, seed=77, empty_frac=0.1, hubs=6, hub_deg=900)
+    x = np.random.default_rng(1).standard_normal((500, 64)).astype(np.float32)
+    dev = torch.device("cuda:0")
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), 500, long_row_threshold=32)
+    assert plan.info()["long_rows"] > 0
+    v, xd = torch.from_numpy(val).to(dev), torch.from_numpy(x).to(dev)
+    outs = []
+    for _ in range(3):               # call 1 unbound, call 2 binds, call 3 uses the bound copy
+        o = torch.zeros(600, 64, device=dev)
+        plan.run(v, xd, o, accumulate=True)
+        outs.append(o)
+    assert plan._bound is not None and plan._bound[0] is v
+    o = torch.zeros(600, 64, device=dev)
+    plan.run(v[:], xd, o, accumulate=True)      # a view of the bound tensor: still bound, same bits
+    assert plan._bound[0] is v and torch.equal(o, outs[0])
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    v.mul_(-2.0)                     # in place: same tensor, new version
+    o = torch.zeros(600, 64, device=dev)
+    plan.run(v, xd, o, accumulate=True)
+    assert torch.equal(o, -2.0 * outs[0])
+    v2 = v.clone()                   # another tensor: unbound path, same result
+    o2 = torch.zeros(600, 64, device=dev)
+    plan.run(v2, xd, o2, accumulate=True)
+    assert torch.equal(o2, o)
