@@ -339,6 +339,8 @@ def main():
             extra["spmm_cache_flushed"] = time_reps_events(step, 20, 2, flush=lambda: scratch.fill_(1.0))
             log(f"[bench] weighted sum per repetition: warm {extra['spmm_warm']}, caches flushed before each {extra['spmm_cache_flushed']}")
             del scratch
+        # one-time preparation, like the plan itself: the unchanged weight tensor was bound during warm-up
+        extra["edge_values_bound_to_plan"] = plan._bound is not None
         extra["spmm_total_gather_GBps"] = round(b_total / ms / 1e6, 1)
         extra["spmm_total_frac_of_hbm_peak"] = round(b_total / ms / 1e6 / HBM_PEAK_GBPS, 4)
         extra["spmm_GFLOPs"] = round(2.0 * nnz * F / ms / 1e6, 1)
