@@ -42,11 +42,12 @@ def log(*a):
 def spmm_gather_bytes(nnz, rows, F, weighted, accumulate, mean, empty_rows=0):
     """Algorithmic bytes of one SpMM under the gather model (no cache credit), int32 columns:
     per edge 4F (dense row) + 4 (col) + 4 (val, if weighted); per row 8 (rowptr); per row that is
-    written 4F, + 4F when accumulating onto a previous out, + 4 for the mean divisor.  In plain
-    accumulate mode a row without edges is not touched (the reference skips it, spmm.cpp:486), so
-    ``empty_rows`` of the ``rows`` do not count there."""
+    written 4F, + 4F when accumulating onto a previous out, + 4 for the mean divisor.  In
+    accumulate mode a row without edges is not touched (the reference skips it, spmm.cpp:486; with
+    the mean divisor its degree is clamped to 1 and x / 1 == x), so ``empty_rows`` of the ``rows``
+    do not count there."""
     per_edge = 4 * F + 4 + (4 if weighted else 0)
-    touched = rows - (empty_rows if (accumulate and not mean) else 0)
+    touched = rows - (empty_rows if accumulate else 0)
     per_touched = 4 * F + (4 * F if accumulate else 0) + (4 if mean else 0)
     return nnz * per_edge + rows * 8 + touched * per_touched
 
@@ -331,7 +332,7 @@ def main():
             out2 = torch.zeros(M, F, device=dev)
             ms_mean = time_steps(lambda: plan.run(None, x, out2, accumulate=True, row_div=deg), 10, 3)
             extra["spmm_mean_GEdges_per_s"] = round(nnz / ms_mean / 1e6, 3)
-            extra["spmm_mean_gather_GBps"] = round(spmm_gather_bytes(nnz, M, F, False, True, True) / ms_mean / 1e6, 1)
+            extra["spmm_mean_gather_GBps"] = round(spmm_gather_bytes(nnz, M, F, False, True, True, empty_rows=n_empty) / ms_mean / 1e6, 1)
             del out2
         if not args.no_extras:
             scratch = torch.empty(192 * 1024 * 1024, device=dev)   # 768 MB > 8 x 4 MB L2 + 256 MB Infinity Cache

@@ -334,6 +334,9 @@ __global__ __launch_bounds__(kBlock) void spmm_empty_rows_kernel(const int32_t *
     if (i >= n_empty) return;
     const int64_t row = empty_rows[i];
     const float div = row_div ? row_div[row] : 1.0f;
+    // x / 1 == x for every float, so an accumulating call leaves such a row exactly as it is: nothing
+    // to read or write (the mean epilogue divides rows without edges by a degree clamped to 1).
+    if (accumulate && div == 1.0f) return;
     for (int f0 = 0; f0 < F; f0 += TILE) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
