@@ -561,6 +561,7 @@ struct PieceArgs {
     const int32_t *col_long; const int32_t *eperm; const float *val; float *partial;
     const int4 *cls_work;
     int max_cls_items; int F;
+    hipStream_t side; hipEvent_t ev_fork, ev_join;  // side != null: long rows run beside the short rows
 };
 struct FinalArgs {
     const int32_t *long_rows; const int32_t *long_pbeg; const float *partial; float *out; int n_long;
@@ -570,6 +571,31 @@ struct FinalArgs {
 template <int VEC, int G, int NV, int BITS>
 static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &f, hipStream_t st) {
     constexpr int GPB = kBlock / G;
+    // The long rows (pieces + final sum) and the short rows write disjoint output rows.  With a side
+    // stream they are issued side by side: fork after the caller's earlier work, join before returning.
+    hipStream_t ls = st;
+    if (s.side != nullptr && f.n_long > 0 && a.n_chunks > 0) {
+        (void)hipEventRecord(s.ev_fork, st);
+        (void)hipStreamWaitEvent(s.side, s.ev_fork, 0);
+        ls = s.side;
+    }
+    if (f.n_long > 0) {
+        {
+            // workgroup i serves class i % 8: grid = 8 * (workgroups of the fullest class)
+            const uint32_t nb = (uint32_t)kNumXCD * (uint32_t)((s.max_cls_items + GPB - 1) / GPB);
+            ProfScope prof(BITS == 0 ? K_SPMM_PIECE : K_FUSED_PIECE, ls);
+            if (s.eperm)
+                hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS, true>), dim3(nb), dim3(kBlock), 0, ls, s.col_long,
+                                   s.eperm, s.val, a.dense, s.partial, s.cls_work, s.max_cls_items, s.F);
+            else
+                hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS, false>), dim3(nb), dim3(kBlock), 0, ls, s.col_long,
+                                   s.eperm, s.val, a.dense, s.partial, s.cls_work, s.max_cls_items, s.F);
+        }
+        const uint32_t nb = (uint32_t)((f.n_long + GPB - 1) / GPB);
+        ProfScope prof(K_SPMM_LONG_FINAL, ls);
+        hipLaunchKernelGGL((spmm_long_final_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, ls, f.long_rows,
+                           f.long_pbeg, f.partial, f.out, f.n_long, f.F, f.ldo, f.accumulate, f.row_div);
+    }
     if (a.n_chunks > 0) {
         const uint32_t nb = (uint32_t)((a.n_chunks + GPB - 1) / GPB);
         ProfScope prof(BITS == 0 ? K_SPMM_SHORT : K_FUSED_SHORT, st);
@@ -582,22 +608,9 @@ static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &
         hipLaunchKernelGGL((spmm_empty_rows_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, a.empty_rows, a.n_empty,
                            a.out, a.F, a.ldo, a.accumulate, a.row_div);
     }
-    if (f.n_long > 0) {
-        {
-            // workgroup i serves class i % 8: grid = 8 * (workgroups of the fullest class)
-            const uint32_t nb = (uint32_t)kNumXCD * (uint32_t)((s.max_cls_items + GPB - 1) / GPB);
-            ProfScope prof(BITS == 0 ? K_SPMM_PIECE : K_FUSED_PIECE, st);
-            if (s.eperm)
-                hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS, true>), dim3(nb), dim3(kBlock), 0, st, s.col_long,
-                                   s.eperm, s.val, a.dense, s.partial, s.cls_work, s.max_cls_items, s.F);
-            else
-                hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS, false>), dim3(nb), dim3(kBlock), 0, st, s.col_long,
-                                   s.eperm, s.val, a.dense, s.partial, s.cls_work, s.max_cls_items, s.F);
-        }
-        const uint32_t nb = (uint32_t)((f.n_long + GPB - 1) / GPB);
-        ProfScope prof(K_SPMM_LONG_FINAL, st);
-        hipLaunchKernelGGL((spmm_long_final_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, f.long_rows,
-                           f.long_pbeg, f.partial, f.out, f.n_long, f.F, f.ldo, f.accumulate, f.row_div);
+    if (ls != st) {
+        (void)hipEventRecord(s.ev_join, ls);
+        (void)hipStreamWaitEvent(st, s.ev_join, 0);
     }
 }
 
@@ -656,6 +669,8 @@ struct sgnn_spmm_plan {
     int32_t *long_pbeg = nullptr;   // [n_long + 1] first piece of each long row
     int32_t *col_long = nullptr;    // [long_edges] columns regrouped by class inside each long row
     int32_t *eperm = nullptr;       // [long_edges] original edge index of each regrouped edge
+    hipStream_t side = nullptr;     // long rows run here, beside the short rows on the caller's stream
+    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
     float *val_long = nullptr;      // [long_edges] bound edge values in regrouped order (sgnn_spmm_plan_bind_values)
     const float *bound_val = nullptr;  // the caller's array val_long was taken from
     int4 *cls_work = nullptr;       // [8 * max_cls_items] (piece id, first edge in col_long / eperm, edges, 0) per class, zero-padded
@@ -719,6 +734,9 @@ extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     (void)hipFree(p->eperm);
     (void)hipFree(p->cls_work);
     (void)hipFree(p->val_long);
+    if (p->ev_fork) (void)hipEventDestroy(p->ev_fork);
+    if (p->ev_join) (void)hipEventDestroy(p->ev_join);
+    if (p->side) (void)hipStreamDestroy(p->side);
     (void)hipFree(p->partial);
     (void)hipFree(p->empty_rows);
     for (int i = 0; i < 3; ++i) (void)hipFree(p->chunks[i]);
@@ -981,7 +999,13 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     }
     ShortArgs a{p->rowptr, p->col, val, dense, out, p->chunks[which], (int)p->n_chunks[which], p->empty_rows,
                 (int)p->n_empty, (int)F, ldo, accumulate, row_div};
-    PieceArgs s{p->col_long, p->eperm, val, p->partial, p->cls_work, p->max_cls_items, (int)F};
+    if (p->side == nullptr && p->n_long > 0 && env_int("SGNN_SPMM_OVERLAP", 0) != 0) {
+        SGNN_HIP_CHECK(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));  // default priority
+        SGNN_HIP_CHECK(hipEventCreateWithFlags(&p->ev_fork, hipEventDisableTiming));
+        SGNN_HIP_CHECK(hipEventCreateWithFlags(&p->ev_join, hipEventDisableTiming));
+    }
+    PieceArgs s{p->col_long, p->eperm, val, p->partial, p->cls_work, p->max_cls_items, (int)F,
+                p->side, p->ev_fork, p->ev_join};
     if (val != nullptr && val == p->bound_val && p->val_long != nullptr) {
         s.eperm = nullptr;   // values already sit in regrouped order: contiguous reads, no indirection
         s.val = p->val_long;
