@@ -1,0 +1,92 @@
+"""Seeded random sweeps over shapes the fixed cases do not list: every configuration is derived from
+its index, so a failure names a reproducible case.  Same bars as the fixed tests: SpMM within
+rel 1e-5 / abs 1e-6 of the oracle (long rows adjudicated against fp64), quantized bytes and params
+bit-exact, dequantized floats within one rounding of code*scale."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from _util import random_csr, abs_sum64, assert_spmm_close, dequant_atol
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("case", range(40))
+def test_spmm_random_shapes(case):
+    from super_gnn_amd import supergnn_ops as ops
+    rng = np.random.default_rng(1000 + case)
+    M, K = int(rng.integers(1, 3000)), int(rng.integers(1, 3000))
+    F = int(rng.choice([1, 3, 4, 8, 30, 32, 64, 100, 128, 130, 256, 300, 602, 1028]))
+    deg = float(rng.choice([0.3, 1, 4, 17, 60]))
+    hubs = int(rng.integers(0, 4)) if M > 8 else 0
+    rowptr, col, val = random_csr(M, K, deg, seed=case, empty_frac=float(rng.choice([0, 0.3, 0.9])), hubs=hubs,
+                                  hub_deg=int(rng.integers(100, 4000)), dup=bool(rng.integers(0, 2)))
+    x = rng.standard_normal((K, F)).astype(np.float32)
+    init = rng.standard_normal((M, F)).astype(np.float32)
+    accumulate = bool(rng.integers(0, 2))
+    weighted = bool(rng.integers(0, 3))           # 1 in 3: unit weights passed as None
+    mean = bool(rng.integers(0, 2))
+    thresh = int(rng.choice([0, 8, 40, 128]))
+    piece = int(rng.choice([0, 8, 32]))
+    dev = torch.device("cuda:0")
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev).to(torch.int32 if case % 2 else torch.int64),
+                        K, long_row_threshold=thresh, piece_edges=piece)
+    div = np.maximum(np.diff(rowptr), 1).astype(np.float32) if mean else None
+    v = val if weighted else None
+    out = torch.from_numpy(init.copy()).to(dev)
+    for _ in range(2 if case % 3 == 0 else 1):    # the second call runs with the values bound to the plan
+        out.copy_(torch.from_numpy(init))
+        plan.run(torch.from_numpy(v).to(dev) if v is not None else None, torch.from_numpy(x).to(dev), out,
+                 accumulate=accumulate, row_div=torch.from_numpy(div).to(dev) if mean else None)
+    got = out.cpu().numpy()
+    want = init.copy() if accumulate else np.zeros_like(init)
+    ones = np.ones(col.shape[0], np.float32)
+    (orc.spmm_accumulate if accumulate else orc.spmm_overwrite)(rowptr, col, v if v is not None else ones, x, want)
+    base = init if accumulate else None
+    f64 = orc.spmm_f64(rowptr, col, v if v is not None else ones, x, base)
+    asum = abs_sum64(rowptr, col, v if v is not None else ones, x, base)
+    if mean:
+        orc.row_divide(want, div)
+        f64 = f64 / div[:, None].astype(np.float64)
+        asum = asum / div[:, None].astype(np.float64)
+    assert_spmm_close(got, want, f64, asum, np.diff(rowptr), what=f"case {case}: M={M} K={K} F={F} deg={deg} acc={accumulate} mean={mean}")
+
+
+@pytest.mark.parametrize("case", range(40))
+def test_quant_random_shapes(case):
+    from super_gnn_amd import supergnn_ops as ops
+    rng = np.random.default_rng(2000 + case)
+    bits = int(rng.choice([8, 4, 2]))
+    F = int(rng.choice([1, 2, 4, 7, 16, 64, 100, 128, 255, 256, 600, 1024, 1030, 2050]))
+    P = int(rng.choice([1, 1, 2, 5, 16]))
+    sizes = rng.integers(0, 200, size=P)
+    seg = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    n = int(seg[-1])
+    if n == 0:
+        seg[-1] = n = 3
+    x = (rng.standard_normal((n, F)) * np.exp(rng.uniform(-10, 10, size=(n, 1)))).astype(np.float32)
+    x[rng.random(n) < 0.05] = 0.0
+    x[rng.random(n) < 0.05] = 1.5              # constant rows: scale 0 -> 1
+    q_ref, p_ref = orc.quant_rows(x, seg, bits)
+    seg_t = torch.from_numpy(seg)
+    bf16 = bool(rng.integers(0, 2))
+    q = torch.zeros(q_ref.shape, dtype=torch.uint8, device="cuda")
+    prm = torch.zeros((n, 2), device="cuda", dtype=torch.bfloat16 if bf16 else torch.float32)
+    xd = torch.from_numpy(x).cuda()
+    if case % 4 == 0:                           # through a row index over a larger, strided source
+        src = torch.zeros((n + 50, F + 4), device="cuda")
+        perm = torch.randperm(n + 50, generator=torch.Generator().manual_seed(case))[:n].cuda()
+        src[perm, 2:2 + F] = xd
+        ops.quantize_tensor_for_all_procs(src[:, 2:2 + F], q, prm, seg_t, P, bits, row_index=perm)
+    else:
+        ops.quantize_tensor_for_all_procs(xd, q, prm, seg_t, P, bits)
+    assert np.array_equal(q.cpu().numpy(), q_ref), f"case {case}: bits={bits} F={F} P={P} n={n}"
+    want_p = torch.from_numpy(p_ref).to(torch.bfloat16) if bf16 else torch.from_numpy(p_ref)
+    assert torch.equal(prm.cpu(), want_p)
+    back = torch.zeros((n, F), device="cuda")
+    ops.dequantize_tensor_for_all_procs(q, back, prm, seg_t, P, bits)
+    p_used = prm.to(torch.float32).cpu().numpy()
+    want = orc.dequant_rows(q_ref, p_used, seg, bits, F)
+    tol = dequant_atol(p_used[:, 0], p_used[:, 1], bits)[:, None]
+    assert np.all(np.abs(back.cpu().numpy() - want) <= tol), f"case {case}"
