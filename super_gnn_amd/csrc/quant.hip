@@ -91,13 +91,22 @@ __device__ __forceinline__ int find_segment(const int32_t *__restrict__ pseg, in
 
 // First fp32 row held by packed row g, and the end of the segment it belongs to.  With a single
 // segment (single_rows >= 0, the row count) nothing is read from memory, so a wave's first loads are
-// its data loads.
+// its data loads.  With several segments the table is searched once per wavefront, for g_wave (a
+// wave-uniform packed row <= g, so the search runs on scalar loads), and only a lane whose packed
+// row lies beyond that segment searches again on its own.
 __device__ __forceinline__ void locate_packed_row(const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg,
-                                                  int P, int64_t single_rows, int g, int epb, int64_t &row0,
-                                                  int64_t &rend) {
+                                                  int P, int64_t single_rows, int g, int g_wave, int epb,
+                                                  int64_t &row0, int64_t &rend) {
     if (single_rows >= 0) {
         row0 = (int64_t)g * epb;
         rend = single_rows;
+        return;
+    }
+    const int pw = find_segment(pseg, P, g_wave);
+    const int ps0 = pseg[pw], ps1 = pseg[pw + 1], s0 = seg[pw], s1 = seg[pw + 1];
+    if (g < ps1) {
+        row0 = (int64_t)s0 + (int64_t)(g - ps0) * epb;
+        rend = s1;
     } else {
         const int p = find_segment(pseg, P, g);
         row0 = (int64_t)seg[p] + (int64_t)(g - pseg[p]) * epb;
@@ -135,7 +144,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
         const int gp = unit * NPR + pi;
         int64_t row0 = 0, rend = 0;
         if (gp < n_packed) {
-            locate_packed_row(seg, pseg, P, single_rows, gp, EPB, row0, rend);
+            locate_packed_row(seg, pseg, P, single_rows, gp, __builtin_amdgcn_readfirstlane(gp), EPB, row0, rend);
         }
 #pragma unroll
         for (int k = 0; k < EPB; ++k) {
@@ -320,7 +329,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
         row[rl] = 0;
         if (g < n_packed) {
             int64_t row0, rend;
-            locate_packed_row(seg, pseg, P, single_rows, g, EPB, row0, rend);
+            locate_packed_row(seg, pseg, P, single_rows, g, __builtin_amdgcn_readfirstlane(g), EPB, row0, rend);
             row[rl] = row0 + k;
             valid[rl] = row[rl] < rend;
         }
@@ -469,7 +478,7 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_kernel(
         const int gp = unit * NPR + pi;
         if (gp >= n_packed) continue;
         int64_t row0, rend;
-        locate_packed_row(seg, pseg, P, single_rows, gp, EPB, row0, rend);
+        locate_packed_row(seg, pseg, P, single_rows, gp, __builtin_amdgcn_readfirstlane(gp), EPB, row0, rend);
         const uint8_t *qr = q + (int64_t)gp * F;
         float zp[EPB], sc[EPB];
 #pragma unroll
@@ -526,6 +535,22 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_kernel(
     uint32_t word[R];
     float2 ps[R];
     int shift[R];
+    // The segment that holds the wave's first row, searched once per wave on wave-uniform values
+    // (scalar loads); lanes further on fall back to their own search.
+    int w_p = 0, w_s0 = 0, w_s1 = 0, w_ps0 = 0;
+    if constexpr (SEGMENTED) {
+        const int64_t i0 = ((int64_t)blockIdx.x * (kQBlock / 64) + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))) * (R * 64);
+        const int row_w = (int)(POW2 ? (i0 >> g_shift) : (i0 / G));
+        int lo = 0, hi = P - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (seg[mid + 1] > row_w) hi = mid; else lo = mid + 1;
+        }
+        w_p = lo;
+        w_s0 = seg[lo];
+        w_s1 = seg[lo + 1];
+        w_ps0 = pseg[lo];
+    }
 #pragma unroll
     for (int u = 0; u < R; ++u) {
         const int64_t i = base + u * 64;
@@ -543,12 +568,16 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_kernel(
         }
         int slot = row;
         if constexpr (SEGMENTED) {  // sub-byte codes and more than one segment: segments start on packed-row boundaries
-            int lo = 0, hi = P - 1;
-            while (lo < hi) {
-                const int mid = (lo + hi) >> 1;
-                if (seg[mid + 1] > row) hi = mid; else lo = mid + 1;
+            if (row < w_s1) {
+                slot = w_ps0 * EPB + (row - w_s0);
+            } else {             // this lane's row lies beyond the segment the wave starts in
+                int lo = w_p, hi = P - 1;
+                while (lo < hi) {
+                    const int mid = (lo + hi) >> 1;
+                    if (seg[mid + 1] > row) hi = mid; else lo = mid + 1;
+                }
+                slot = pseg[lo] * EPB + (row - seg[lo]);
             }
-            slot = pseg[lo] * EPB + (row - seg[lo]);
         }
         ps[u] = load_params(pb, row);
         shift[u] = (EPB - 1 - (slot % EPB)) * BITS;
@@ -577,7 +606,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_wide_kernel(
     const int gp = blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
     if (gp >= n_packed) return;
     int64_t row0, rend;
-    locate_packed_row(seg, pseg, P, single_rows, gp, EPB, row0, rend);
+    locate_packed_row(seg, pseg, P, single_rows, gp, __builtin_amdgcn_readfirstlane(gp), EPB, row0, rend);
     float zp[EPB], sc[EPB];
 #pragma unroll
     for (int k = 0; k < EPB; ++k) {
@@ -627,7 +656,7 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_rows_wide_kernel(
     const int gp = blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
     if (gp >= n_packed) return;
     int64_t row0, rend;
-    locate_packed_row(seg, pseg, P, single_rows, gp, EPB, row0, rend);
+    locate_packed_row(seg, pseg, P, single_rows, gp, __builtin_amdgcn_readfirstlane(gp), EPB, row0, rend);
     const uint8_t *qr = q + (int64_t)gp * F;
 #pragma unroll
     for (int k = 0; k < EPB; ++k) {
