@@ -177,6 +177,15 @@ int sgnn_spmm_csr_dq_f32(sgnn_spmm_plan *plan, const float *val, const uint8_t *
                          const int32_t *row_slot, int bits, float *out, int64_t F, int64_t ldo,
                          int accumulate, const float *row_div, sgnn_stream_t stream);
 
+/* The fused calls below never look row_slot up per gathered row: the plan keeps
+ * row_slot[col[e]] for each of its edges, streamed next to the column indices (a table lookup in
+ * front of every packed-row fetch cost +23 % on the remote step).  That per-edge stream is built by
+ * this call -- or by the first fused call that sees a new row_slot POINTER -- and reused while
+ * the same pointer comes back: a table is taken to be constant (a partition's segment table is fixed
+ * when its graph is built, super_gnn/data_manager/CommBuffer.py:37-44).  Call this again after
+ * changing a table in place; row_slot == NULL drops the stream. */
+int sgnn_spmm_plan_bind_row_slots(sgnn_spmm_plan *plan, const int32_t *row_slot, sgnn_stream_t stream);
+
 /* sgnn_spmm_csr_dq_f32 with params in either form (params_bf16: see
  * sgnn_quant_pack_rows_wire_f32).  With a 0/1 selection matrix as A this is also the scatter of the
  * plain mode's backward pass, local_grad.index_add_(0, idx, dequantize(q))

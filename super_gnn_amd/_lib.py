@@ -27,6 +27,7 @@ SIGNATURES = {
     "sgnn_unpack_dequant_rows_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
     "sgnn_quant_row_slots": (_int, [_vp, _vp, _int, _int, _i64, _vp, _vp]),
     "sgnn_spmm_plan_bind_values": (_int, [_vp, _vp, _vp]),
+    "sgnn_spmm_plan_bind_row_slots": (_int, [_vp, _vp, _vp]),
     "sgnn_spmm_csr_dq_f32": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _i64, _i64, _int, _vp, _vp]),
     "sgnn_quant_pack_rows_wire_f32": (_int, [_vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),
     "sgnn_unpack_dequant_rows_wire_f32": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp]),

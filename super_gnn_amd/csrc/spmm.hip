@@ -61,12 +61,15 @@ __device__ __forceinline__ int64_t uniform64(int64_t v) {
 // template parameter BITS is a format code: the low four bits are the code width (8, 4 or 2) and
 // kBf16Params is added when (zero_point, scale) are bf16 pairs instead of fp32 pairs.
 constexpr int kBf16Params = 16;
+constexpr int kEdgeSlots = 32;  // added when every edge carries its slot (plan-bound row slots)
 struct DenseSrc {
     const float *x;        // fp32: [K, ldx]
     int64_t ldx;
     const uint8_t *q;      // quantized: packed rows of qF bytes
     ParamBuf params;       // quantized: (zero_point, scale) per dense row, fp32 or bf16 pairs
-    const int32_t *slot;   // quantized: dense row -> index in the padded row space (null = identity)
+    const int32_t *eslot_csr;   // quantized, ragged segments: position of each edge's dense row in the padded row
+                                // space, row_slot[col[e]], in CSR order (bound to the plan) ...
+    const int32_t *eslot_long;  // ... and in the regrouped order of the long rows; null = no padding (slot == row)
     int qF;
 };
 
@@ -82,8 +85,8 @@ struct Fetched {
 };
 
 template <int VEC, int NV, int BITS>
-__device__ __forceinline__ void fetch_row(Fetched<VEC, NV, BITS> &r, const DenseSrc &d, int c, const int (&off)[NV],
-                                          const bool (&act)[NV]) {
+__device__ __forceinline__ void fetch_row(Fetched<VEC, NV, BITS> &r, const DenseSrc &d, int c, int edge_slot,
+                                          const int (&off)[NV], const bool (&act)[NV]) {
     if constexpr (BITS == 0) {
         const float *xr = d.x + (int64_t)c * d.ldx;
 #pragma unroll
@@ -92,7 +95,7 @@ __device__ __forceinline__ void fetch_row(Fetched<VEC, NV, BITS> &r, const Dense
     } else {
         constexpr int NB = BITS & 15;
         constexpr int EPB = 8 / NB;
-        const int sl = d.slot ? d.slot[c] : c;
+        const int sl = (BITS & kEdgeSlots) != 0 ? edge_slot : c;  // without a slot stream the row space has no padding
         const float2 ps = load_params_as<(BITS & kBf16Params) != 0>(d.params.p, c);
         r.zp = ps.x;
         r.sc = ps.y;
@@ -134,23 +137,25 @@ __device__ __forceinline__ void fma_row(float (&acc)[NV][VEC], float w, const Fe
 template <int VEC, int G, int NV, int BITS, bool PERM>
 __device__ __forceinline__ void gather_piece(float (&acc)[NV][VEC], const int32_t *__restrict__ colp,
                                              const int32_t *__restrict__ eperm, const float *__restrict__ val,
-                                             int deg, const DenseSrc &dense, const int (&off)[NV],
-                                             const bool (&act)[NV], int lig) {
+                                             const int32_t *__restrict__ slotp, int deg, const DenseSrc &dense,
+                                             const int (&off)[NV], const bool (&act)[NV], int lig) {
     constexpr int U = unroll_of(NV);
     // (col,val) pairs are fetched G at a time, one chunk ahead of the gathers that consume them.
-    int nc = 0;
+    int nc = 0, ns = -1;
     float nw = 1.0f;
     if (lig < deg) {
         nc = __builtin_nontemporal_load(colp + lig);
         if (val) nw = PERM ? val[__builtin_nontemporal_load(eperm + lig)] : __builtin_nontemporal_load(val + lig);
+        if constexpr ((BITS & kEdgeSlots) != 0) ns = __builtin_nontemporal_load(slotp + lig);
     }
     for (int base = 0; base < deg; base += G) {
-        const int myc = nc;
+        const int myc = nc, mys = ns;
         const float myw = nw;
         const int nidx = base + G + lig;
         if (nidx < deg) {
             nc = __builtin_nontemporal_load(colp + nidx);
             if (val) nw = PERM ? val[__builtin_nontemporal_load(eperm + nidx)] : __builtin_nontemporal_load(val + nidx);
+            if constexpr ((BITS & kEdgeSlots) != 0) ns = __builtin_nontemporal_load(slotp + nidx);
         }
         const int cnt = deg - base < G ? deg - base : G;
         for (int j = 0; j < cnt; j += U) {
@@ -160,7 +165,9 @@ __device__ __forceinline__ void gather_piece(float (&acc)[NV][VEC], const int32_
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int src = j + u < cnt ? j + u : cnt - 1;
-                fetch_row<VEC, NV, BITS>(xv[u], dense, group_bcast_i<G>(myc, src), off, act);
+                int es = -1;
+                if constexpr ((BITS & kEdgeSlots) != 0) es = group_bcast_i<G>(mys, src);
+                fetch_row<VEC, NV, BITS>(xv[u], dense, group_bcast_i<G>(myc, src), es, off, act);
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -213,11 +220,14 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
     const int E = ch.w;
     const int32_t *colp = col + B;
     const float *valp = val ? val + B : nullptr;
-    int nc0 = 0;
+    const int32_t *slotp = nullptr;
+    if constexpr ((BITS & kEdgeSlots) != 0) slotp = dense.eslot_csr + B;
+    int nc0 = 0, ns0 = -1;
     float nw0 = 1.0f;
     if (lig < E) {
         nc0 = __builtin_nontemporal_load(colp + lig);
         if (valp) nw0 = __builtin_nontemporal_load(valp + lig);
+        if constexpr ((BITS & kEdgeSlots) != 0) ns0 = __builtin_nontemporal_load(slotp + lig);
     }
 
     // Lane i holds rowptr[rb+i] relative to the chunk's first edge (lanes >= nr hold the end).
@@ -252,19 +262,21 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
             }
         }
 
-        int nc = nc0;
+        int nc = nc0, ns = ns0;
         float nw = nw0;
         if (f0 > 0 && lig < E) {  // a later feature tile walks the chunk's edges again
             nc = __builtin_nontemporal_load(colp + lig);
             if (valp) nw = __builtin_nontemporal_load(valp + lig);
+            if constexpr ((BITS & kEdgeSlots) != 0) ns = __builtin_nontemporal_load(slotp + lig);
         }
         for (int base = 0; base < E; base += G) {
-            const int myc = nc;
+            const int myc = nc, mys = ns;
             const float myw = nw;
             const int nidx = base + G + lig;  // next chunk, fetched one chunk ahead of its gathers
             if (nidx < E) {
                 nc = __builtin_nontemporal_load(colp + nidx);
                 if (valp) nw = __builtin_nontemporal_load(valp + nidx);
+                if constexpr ((BITS & kEdgeSlots) != 0) ns = __builtin_nontemporal_load(slotp + nidx);
             }
             const int cnt = E - base < G ? E - base : G;
             for (int j = 0; j < cnt; j += U) {
@@ -274,7 +286,9 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const int src = j + u < cnt ? j + u : cnt - 1;
-                    fetch_row<VEC, NV, BITS>(xv[u], dense, group_bcast_i<G>(myc, src), off, act);
+                    int es = -1;
+                    if constexpr ((BITS & kEdgeSlots) != 0) es = group_bcast_i<G>(mys, src);
+                    fetch_row<VEC, NV, BITS>(xv[u], dense, group_bcast_i<G>(myc, src), es, off, act);
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -395,7 +409,8 @@ __global__ __launch_bounds__(kBlock) void spmm_piece_kernel(
             for (int k = 0; k < VEC; ++k) acc[v][k] = 0.0f;
         }
         gather_piece<VEC, G, NV, BITS, PERM>(acc, col_long + b, PERM ? eperm + b : nullptr, (PERM || !val) ? val : val + b,
-                                             len, dense, off, act, lig);
+                                             (BITS & kEdgeSlots) != 0 ? dense.eslot_long + b : nullptr, len, dense,
+                                             off, act, lig);
 #pragma unroll
         for (int v = 0; v < NV; ++v)
             if (act[v]) vec_store<VEC>(partial + (int64_t)item * F + off[v], acc[v]);
@@ -543,6 +558,13 @@ __global__ __launch_bounds__(kBlock) void column_popularity_kernel(const int32_t
     for (; i < n; i += stride) atomicAdd(popularity + col[i], 1);
 }
 
+// dst[i] = table[idx[i]]: the per-edge slot stream of a plan (idx = the plan's column array).
+__global__ __launch_bounds__(kBlock) void translate_columns_kernel(const int32_t *__restrict__ idx, const int32_t *__restrict__ table,
+                                                                   int32_t *__restrict__ dst, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) dst[i] = table[__builtin_nontemporal_load(idx + i)];
+}
+
 __global__ __launch_bounds__(kBlock) void permute_values_kernel(const float *__restrict__ val, const int32_t *__restrict__ eperm,
                                                                 float *__restrict__ dst, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -673,6 +695,9 @@ struct sgnn_spmm_plan {
     hipEvent_t ev_fork = nullptr, ev_join = nullptr;
     float *val_long = nullptr;      // [long_edges] bound edge values in regrouped order (sgnn_spmm_plan_bind_values)
     const float *bound_val = nullptr;  // the caller's array val_long was taken from
+    int32_t *eslot_csr = nullptr;      // [nnz] row_slot[col[e]] in CSR order (sgnn_spmm_plan_bind_row_slots)
+    int32_t *eslot_long = nullptr;     // [long_edges] the same in regrouped order (partitioned plans)
+    const int32_t *bound_slots = nullptr;  // the caller's table they were taken from
     int4 *cls_work = nullptr;       // [8 * max_cls_items] (piece id, first edge in col_long / eperm, edges, 0) per class, zero-padded
     float *partial = nullptr;       // [n_items * F], grown on demand
     size_t partial_floats = 0;
@@ -734,6 +759,8 @@ extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     (void)hipFree(p->eperm);
     (void)hipFree(p->cls_work);
     (void)hipFree(p->val_long);
+    (void)hipFree(p->eslot_csr);
+    (void)hipFree(p->eslot_long);
     if (p->ev_fork) (void)hipEventDestroy(p->ev_fork);
     if (p->ev_join) (void)hipEventDestroy(p->ev_join);
     if (p->side) (void)hipStreamDestroy(p->side);
@@ -1011,13 +1038,18 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
         s.val = p->val_long;
     }
     FinalArgs f{p->long_rows, p->long_pbeg, p->partial, out, (int)p->n_long, (int)F, ldo, accumulate, row_div};
-    if (bits != 0 && dense.params.bf16) {
-        if (bits == 8) dispatch_shape_dq<8 + kBf16Params>(nvec, a, s, f, st);
-        else if (bits == 4) dispatch_shape_dq<4 + kBf16Params>(nvec, a, s, f, st);
-        else dispatch_shape_dq<2 + kBf16Params>(nvec, a, s, f, st);
-    } else if (bits == 8) dispatch_shape_dq<8>(nvec, a, s, f, st);
-    else if (bits == 4) dispatch_shape_dq<4>(nvec, a, s, f, st);
-    else if (bits == 2) dispatch_shape_dq<2>(nvec, a, s, f, st);
+    if (bits != 0) {
+        const int fmt = bits + (dense.params.bf16 ? kBf16Params : 0) + (dense.eslot_csr ? kEdgeSlots : 0);
+        switch (fmt) {
+#define SGNN_DQ(FMT) case FMT: dispatch_shape_dq<FMT>(nvec, a, s, f, st); break
+            SGNN_DQ(8); SGNN_DQ(4); SGNN_DQ(2);
+            SGNN_DQ(8 + kBf16Params); SGNN_DQ(4 + kBf16Params); SGNN_DQ(2 + kBf16Params);
+            SGNN_DQ(8 + kEdgeSlots); SGNN_DQ(4 + kEdgeSlots); SGNN_DQ(2 + kEdgeSlots);
+            SGNN_DQ(8 + kBf16Params + kEdgeSlots); SGNN_DQ(4 + kBf16Params + kEdgeSlots); SGNN_DQ(2 + kBf16Params + kEdgeSlots);
+#undef SGNN_DQ
+            default: return fail(SGNN_ERR_ARG, "unsupported quantized format %d", fmt);
+        }
+    }
     else if (vec == 4) dispatch_shape<4>(nvec, a, s, f, st);
     else if (vec == 2) dispatch_shape<2>(nvec, a, s, f, st);
     else dispatch_shape<1>(nvec, a, s, f, st);
@@ -1038,13 +1070,31 @@ extern "C" int sgnn_spmm_plan_bind_values(sgnn_spmm_plan *p, const float *val, s
     return SGNN_OK;
 }
 
+extern "C" int sgnn_spmm_plan_bind_row_slots(sgnn_spmm_plan *p, const int32_t *row_slot, sgnn_stream_t stream) {
+    SGNN_REQUIRE(p != nullptr, "plan is null");
+    p->bound_slots = nullptr;
+    if (row_slot == nullptr || p->nnz == 0) return SGNN_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (p->eslot_csr == nullptr) SGNN_HIP_CHECK(hipMalloc(&p->eslot_csr, sizeof(int32_t) * (size_t)p->nnz));
+    hipLaunchKernelGGL(translate_columns_kernel, dim3((uint32_t)((p->nnz + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, p->col,
+                       row_slot, p->eslot_csr, p->nnz);
+    if (p->partitioned && p->long_edges > 0) {
+        if (p->eslot_long == nullptr) SGNN_HIP_CHECK(hipMalloc(&p->eslot_long, sizeof(int32_t) * (size_t)p->long_edges));
+        hipLaunchKernelGGL(translate_columns_kernel, dim3((uint32_t)((p->long_edges + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           st, p->col_long, row_slot, p->eslot_long, p->long_edges);
+    }
+    SGNN_HIP_CHECK(hipGetLastError());
+    p->bound_slots = row_slot;
+    return SGNN_OK;
+}
+
 extern "C" int sgnn_spmm_csr_f32(sgnn_spmm_plan *p, const float *val, const float *x, float *out, int64_t F,
                                  int64_t ldx, int64_t ldo, int accumulate, const float *row_div,
                                  sgnn_stream_t stream) {
     SGNN_REQUIRE(p != nullptr, "plan is null");
     SGNN_REQUIRE(ldx >= F, "leading dimension smaller than F (ldx=%lld F=%lld)", (long long)ldx, (long long)F);
     SGNN_REQUIRE(x != nullptr || p->nnz == 0 || p->M == 0, "x is null");
-    DenseSrc d{x, ldx, nullptr, ParamBuf{nullptr, 0}, nullptr, 0};
+    DenseSrc d{x, ldx, nullptr, ParamBuf{nullptr, 0}, nullptr, nullptr, 0};
     return spmm_run(p, val, d, 0, out, F, ldo, accumulate, row_div, (hipStream_t)stream);
 }
 
@@ -1058,7 +1108,18 @@ static int spmm_dq_impl(sgnn_spmm_plan *p, const float *val, const uint8_t *q, c
     SGNN_REQUIRE((q != nullptr && params != nullptr) || p->nnz == 0 || p->M == 0, "q / params is null");
     SGNN_REQUIRE(aligned(q, 4) && aligned(params, params_bf16 ? 4 : 8), "q must be 4-byte and params %d-byte aligned",
                  params_bf16 ? 4 : 8);
-    DenseSrc d{nullptr, 0, q, ParamBuf{const_cast<void *>(params), params_bf16}, row_slot, (int)F};
+    DenseSrc d{nullptr, 0, q, ParamBuf{const_cast<void *>(params), params_bf16}, nullptr, nullptr, (int)F};
+    if (row_slot != nullptr && p->nnz > 0) {
+        // Every edge carries its slot next to its column, so a gather never looks the table up.  The
+        // per-edge stream is built the first time a table is seen and kept while the same pointer
+        // comes back (the table is taken to be constant; sgnn_spmm_plan_bind_row_slots refreshes it).
+        if (row_slot != p->bound_slots) {
+            const int rc = sgnn_spmm_plan_bind_row_slots(p, row_slot, stream);
+            if (rc != SGNN_OK) return rc;
+        }
+        d.eslot_csr = p->eslot_csr;
+        d.eslot_long = p->eslot_long ? p->eslot_long : p->eslot_csr;  // unregrouped long rows index the CSR arrays
+    }
     return spmm_run(p, val, d, bits, out, F, ldo, accumulate, row_div, (hipStream_t)stream);
 }
 

@@ -108,6 +108,7 @@ class SpmmPlan:
         self._h = h
         self._bound = None   # (value tensor, version) whose long-row values the plan holds in its own order
         self._seen = None    # (value tensor, version) of the previous call
+        self._bound_slots = None  # row-slot table (a tensor owned by a _Segments object) bound to the plan
         self.device = dev
 
     def info(self):
@@ -192,6 +193,10 @@ class SpmmPlan:
         if row_div is not None:
             _want(row_div, torch.float32, "row_div")
         slots = segs.row_slots(bits)
+        if slots is not None and self._bound_slots is not slots:
+            # the segment table of a partition never changes: carry each edge's slot with its column
+            check(lib.sgnn_spmm_plan_bind_row_slots(self._h, _ptr(slots), _stream()))
+            self._bound_slots = slots
         if value is not None and value.is_contiguous():
             self._maybe_bind(value)
         if bf16:
