@@ -201,7 +201,8 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
     int64_t ldo, int accumulate, const float *__restrict__ row_div, uint32_t nblocks) {
     constexpr int GPB = kBlock / G;
     constexpr int TILE = G * VEC * NV;
-    constexpr int U = unroll_of(NV);
+    // gathers in flight per lane group: 6 keeps the kernel at 75 VGPRs (6 waves per SIMD); 8 costs 83 (5 waves)
+    constexpr int U = NV == 1 ? 6 : unroll_of(NV);
     const uint32_t lb = xcd_contiguous_block(blockIdx.x, nblocks);
     const int gid = threadIdx.x / G, lig = threadIdx.x % G;
     const int ci = (int)lb * GPB + gid;
