@@ -306,7 +306,8 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
 // at int2 (two DPP rows at int4), so packing is a shift in each lane followed by an OR across DPP
 // rows.
 // ------------------------------------------------------------------------------------------------
-template <int BITS, int NV, int RL, bool kForceExactDivision>
+// FULL: F == 64 * NV, every lane's every vector lies inside the row (no per-load lane predicates).
+template <int BITS, int NV, int RL, bool kForceExactDivision, bool FULL = false>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
     const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F,
@@ -339,7 +340,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         off[v] = (v * 16 + l16) * VEC;
-        act[v] = off[v] < F;
+        act[v] = FULL ? true : off[v] < F;
     }
     float xv[RL][NV][VEC];
 #pragma unroll
@@ -790,6 +791,9 @@ static void launch_quant16(const RowsArgs &a, hipStream_t st) {
     ProfScope prof(K_QUANT_PACK_ROWS, st);
     if (a.exact_division)
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
+                           a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
+    else if (a.F == 64 * NV)
+        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
                            a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
     else
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
