@@ -28,8 +28,8 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 # this file (see profiles/), scaled by what the same counters read for sgnn_stream_copy_f32 of a
 # known size.  Keyed by workload name; None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    # spmm_piece_kernel (values bound to the plan): FETCH_SIZE 4036481 x 2.000 + WRITE_SIZE 860068 x 1.000 (KiB per launch)
-    "rmat_2450000n_62000000e_F128_gcn_weighted_sum": 9_147_000_000,
+    # spmm_piece_kernel (values bound to the plan): FETCH_SIZE 4041502 x 2.000 + WRITE_SIZE 860068 x 1.000 (KiB per launch)
+    "rmat_2450000n_62000000e_F128_gcn_weighted_sum": 9_157_000_000,
     # quant_pack_rows16_kernel<2,...>: FETCH_SIZE 500052 x 2.000 + WRITE_SIZE 76196 x 1.000
     "quant_pack_int2_1000000x256": 1_102_000_000,
 }
