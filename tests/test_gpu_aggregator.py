@@ -260,3 +260,29 @@ def test_sage_model_is_partition_invariant_and_trains():
         opt.step()
         losses.append(loss.item())
     assert losses[-1] < losses[0] - 0.05, losses
+
+
+def test_world_from_reference_partition_files(tmp_path):
+    """Graph -> the reference's per-rank files -> loader -> loop-back world: one int8 aggregation
+    equals the global product at the quantization error scale, and the fp32 one within the SpMM bar."""
+    from super_gnn_amd.aggregator import LoopbackWorld
+    from super_gnn_amd.data_manager import load_loopback_partitions, save_partition_files
+    rowptr, col, _ = _graph(n=5000, und_edges=30000, seed=21)
+    n, F = rowptr.numel() - 1, 64
+    gen = torch.Generator().manual_seed(2)
+    feat = torch.randn(n, F, generator=gen)
+    label = torch.randint(0, 5, (n,), generator=gen)
+    idx = torch.arange(n)
+    bounds = torch.tensor([0, 1100, 2600, 3900, n])
+    save_partition_files(str(tmp_path), "g", rowptr, col, bounds, feat, label, idx[::3], idx[1::3], idx[2::3])
+    rp, c = rowptr.numpy(), col.numpy().astype(np.int64)
+    want = np.zeros((n, F), np.float32)
+    orc.spmm_accumulate(rp, c, np.ones(c.size, np.float32), feat.numpy(), want)
+    for bits, pre in ((32, True), (8, False), (8, True)):
+        graphs, data = load_loopback_partitions(str(tmp_path), "g", 4, F, num_bits=bits, is_pre_delay=pre)
+        feats = [d["nodes_features"].cuda() for d in data]
+        got = torch.cat(LoopbackWorld(graphs, bits, pre).aggregate(feats)).cpu().numpy()
+        if bits == 32:
+            assert np.all(np.abs(got - want) <= 1e-4 + 1e-5 * np.abs(want))
+        else:
+            assert np.linalg.norm(got - want) / np.linalg.norm(want) < 0.01

@@ -325,3 +325,41 @@ def test_bound_values_follow_in_place_changes():
     o2 = torch.zeros(600, 64, device=dev)
     plan.run(v2, xd, o2, accumulate=True)
     assert torch.equal(o2, o)
+
+
+def test_steady_state_calls_replay_from_a_captured_graph():
+    """After warm-up a call only launches kernels (no allocation, no synchronisation), so an
+    SpMM + quantize + fused-SpMM sequence can be captured once and replayed; every replay, with eager
+    work in between, must reproduce the eager result bit for bit."""
+    ops = _gpu()
+    dev = torch.device("cuda:0")
+    rowptr, col, val = random_csr(4000, 3000, 9, seed=5, empty_frac=0.2, hubs=8, hub_deg=1200)
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(3000, 128, generator=gen).to(dev)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), 3000)
+    v = torch.from_numpy(val).to(dev)
+    seg = torch.tensor([0, 1001, 2003, 3000], dtype=torch.int32)
+    segs = ops.quant_segments(seg, 4)
+    q = torch.zeros(segs.n_packed, 128, dtype=torch.uint8, device=dev)
+    prm = torch.zeros(3000, 2, device=dev)
+    out, out_q = torch.zeros(4000, 128, device=dev), torch.zeros(4000, 128, device=dev)
+
+    def step():
+        out.zero_(); out_q.zero_()
+        plan.run(v, x, out, accumulate=True)
+        ops.quantize_tensor_for_all_procs(x, q, prm, seg, 3, 4)
+        plan.run_quantized(v, q, prm, segs, 4, out_q, accumulate=True)
+
+    for _ in range(3):          # warm-up: lazy work lists, partial buffer, value and slot binding
+        step()
+    torch.cuda.synchronize()
+    want, want_q = out.clone(), out_q.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for i in range(4):
+        out.fill_(float(i)); out_q.fill_(-1.0); q.zero_()          # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want) and torch.equal(out_q, want_q), f"replay {i}"
