@@ -733,6 +733,167 @@ __global__ __launch_bounds__(kQBlock) void dequant_v1_kernel(const uint8_t *__re
     }
 }
 
+// The same two operations with float4 lanes (F % 4 == 0, F <= 256 * NV, 16-byte aligned fp32 rows): a
+// wavefront takes R consecutive rows, each row read once into registers, 64-lane DPP reductions, and the
+// four codes of a lane packed into one 32/16/8-bit store (int8/int4/int2).  A row's layout depends on
+// two loaded values (its bit width and its byte offset range[i]); all R rows' values are requested
+// before the first is used, so the wave pays that latency once per R KB instead of once per row.
+// A row's bytes need not start 4- or 2-byte aligned; such a row falls back to byte stores / loads.
+template <int NV, int R>
+__global__ __launch_bounds__(kQBlock) void quant_v1_vec_kernel(const float *__restrict__ x, uint8_t *__restrict__ q,
+                                                               const int64_t *__restrict__ range,
+                                                               float *__restrict__ params, int64_t n, int F) {
+    const int lane = threadIdx.x & 63;
+    const int64_t i0 = ((int64_t)blockIdx.x * (kQBlock / 64) + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))) * R;
+    if (i0 >= n) return;
+    float bits_f[R];
+    int64_t r0[R];
+    float xv[R][NV][4];
+    int off[NV];
+    bool act[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        off[v] = (v * 64 + lane) * 4;
+        act[v] = off[v] < F;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t i = i0 + r < n ? i0 + r : n - 1;  // a short last wave repeats the last row's loads
+        bits_f[r] = params[i * 3];
+        r0[r] = range[i];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) vec_load_nt<4>(xv[r][v], x + i * F + (act[v] ? off[v] : 0));  // unconditional
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t i = i0 + r;
+        if (i >= n) break;
+        const int b = (int)bits_f[r];
+        if (b != 8 && b != 4 && b != 2) continue;  // the reference prints an error and leaves the row (quantization_x86.cpp:244-245)
+        float mn = INFINITY, mx = -INFINITY;
+        int key = INT_MAX;
+#pragma unroll
+        for (int v = NV - 1; v >= 0; --v) {
+            if (!act[v]) continue;
+#pragma unroll
+            for (int k = 3; k >= 0; --k) {
+                mn = fminf(mn, xv[r][v][k]);
+                mx = fmaxf(mx, xv[r][v][k]);
+                if (xv[r][v][k] == 0.0f) key = ((off[v] + k) << 1) | (int)(__float_as_uint(xv[r][v][k]) >> 31);
+            }
+        }
+        mn = group_allreduce_f<64, OpMinF>(mn);
+        mx = group_allreduce_f<64, OpMaxF>(mx);
+        key = group_allmin_i<64>(key);
+        const float z = (key & 1) ? -0.0f : 0.0f;
+        if (mn == 0.0f) mn = z;
+        if (mx == 0.0f) mx = z;
+        const float first = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(xv[r][0][0])));
+        if (first != first) { mn = first; mx = first; }
+        float s = (mx - mn) / (float)((1 << b) - 1);
+        if (s == 0.0f) s = 1.0f;
+        if (lane == 0) { params[i * 3 + 1] = mn; params[i * 3 + 2] = s; }
+        uint8_t *qo = q + r0[r];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            if (!act[v]) continue;
+            uint32_t c[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) c[k] = quant_code(xv[r][v][k], mn, s);
+            if (b == 8) {
+                uint8_t *dst = qo + off[v];
+                if ((r0[r] & 3) == 0) {
+                    __builtin_nontemporal_store(c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24), reinterpret_cast<uint32_t *>(dst));
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) dst[k] = (uint8_t)c[k];
+                }
+            } else if (b == 4) {
+                uint8_t *dst = qo + off[v] / 2;
+                const uint32_t b0 = (c[0] << 4) | c[1], b1 = (c[2] << 4) | c[3];
+                if ((r0[r] & 1) == 0) {
+                    __builtin_nontemporal_store((uint16_t)(b0 | (b1 << 8)), reinterpret_cast<uint16_t *>(dst));
+                } else {
+                    dst[0] = (uint8_t)b0;
+                    dst[1] = (uint8_t)b1;
+                }
+            } else {
+                qo[off[v] / 4] = (uint8_t)((c[0] << 6) | (c[1] << 4) | (c[2] << 2) | c[3]);
+            }
+        }
+    }
+}
+
+template <int NV, int R>
+__global__ __launch_bounds__(kQBlock) void dequant_v1_vec_kernel(const uint8_t *__restrict__ q, float *__restrict__ x,
+                                                                 const int64_t *__restrict__ range,
+                                                                 const float *__restrict__ params, int64_t n, int F) {
+    const int lane = threadIdx.x & 63;
+    const int64_t i0 = ((int64_t)blockIdx.x * (kQBlock / 64) + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))) * R;
+    if (i0 >= n) return;
+    float bits_f[R], zp[R], sc[R];
+    int64_t r0[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t i = i0 + r < n ? i0 + r : n - 1;
+        bits_f[r] = params[i * 3];
+        zp[r] = params[i * 3 + 1];
+        sc[r] = params[i * 3 + 2];
+        r0[r] = range[i];
+    }
+    uint32_t w[R][NV];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int b = (int)bits_f[r];
+        const uint8_t *qi = q + r0[r];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int off = (v * 64 + lane) * 4;
+            w[r][v] = 0;
+            if (off >= F || i0 + r >= n) continue;
+            if (b == 8) {
+                const uint8_t *src = qi + off;
+                if ((r0[r] & 3) == 0) w[r][v] = *reinterpret_cast<const uint32_t *>(src);
+                else w[r][v] = src[0] | (src[1] << 8) | (src[2] << 16) | ((uint32_t)src[3] << 24);
+            } else if (b == 4) {
+                const uint8_t *src = qi + off / 2;
+                if ((r0[r] & 1) == 0) w[r][v] = *reinterpret_cast<const uint16_t *>(src);
+                else w[r][v] = src[0] | (src[1] << 8);
+            } else if (b == 2) {
+                w[r][v] = qi[off / 4];
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t i = i0 + r;
+        if (i >= n) break;
+        const int b = (int)bits_f[r];
+        if (b != 8 && b != 4 && b != 2) continue;
+        float *xo = x + i * F;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int off = (v * 64 + lane) * 4;
+            if (off >= F) continue;
+            const uint32_t ww = w[r][v];
+            uint32_t c[4];
+            if (b == 8) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) c[k] = (ww >> (8 * k)) & 255u;
+            } else if (b == 4) {
+                c[0] = (ww >> 4) & 15u; c[1] = ww & 15u; c[2] = (ww >> 12) & 15u; c[3] = (ww >> 8) & 15u;
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) c[k] = (ww >> (6 - 2 * k)) & 3u;
+            }
+            float o[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) o[k] = fmaf((float)c[k], sc[r], zp[r]);
+            vec_store_nt<4>(xo + off, o);
+        }
+    }
+}
+
 // Position of every row in the padded row space (EPB rows per packed row, every segment starting
 // on a packed-row boundary): slot[r] = pseg[p] * EPB + (r - seg[p]) for the segment p holding r.
 // Packed row = slot / EPB, position inside the byte = slot % EPB.
@@ -1005,7 +1166,17 @@ extern "C" int sgnn_quant_v1_f32(const float *x, uint8_t *q, const int64_t *rang
     SGNN_REQUIRE(x && q && range && params, "null pointer argument");
     const int64_t nb = (n + kQBlock / 64 - 1) / (kQBlock / 64);
     SGNN_REQUIRE(nb < INT32_MAX, "too many rows");
-    hipLaunchKernelGGL(quant_v1_kernel, dim3((uint32_t)nb), dim3(kQBlock), 0, (hipStream_t)stream, x, q, range, params, n, (int)F);
+    ProfScope prof(K_QUANT_V1, (hipStream_t)stream);
+    const dim3 grid((uint32_t)nb), block(kQBlock);
+    const auto grid_r = [&](int rows) { return dim3((uint32_t)((nb + rows - 1) / rows)); };
+    hipStream_t st = (hipStream_t)stream;
+    if (F % 4 == 0 && F <= 1024 && aligned(x, 16)) {
+        if (F <= 256) hipLaunchKernelGGL((quant_v1_vec_kernel<1, 4>), grid_r(4), block, 0, st, x, q, range, params, n, (int)F);
+        else if (F <= 512) hipLaunchKernelGGL((quant_v1_vec_kernel<2, 2>), grid_r(2), block, 0, st, x, q, range, params, n, (int)F);
+        else hipLaunchKernelGGL((quant_v1_vec_kernel<4, 1>), grid, block, 0, st, x, q, range, params, n, (int)F);
+    } else {
+        hipLaunchKernelGGL(quant_v1_kernel, grid, block, 0, st, x, q, range, params, n, (int)F);
+    }
     SGNN_HIP_CHECK(hipGetLastError());
     return SGNN_OK;
 }
@@ -1017,7 +1188,17 @@ extern "C" int sgnn_dequant_v1_f32(const uint8_t *q, float *x, const int64_t *ra
     SGNN_REQUIRE(x && q && range && params, "null pointer argument");
     const int64_t nb = (n + kQBlock / 64 - 1) / (kQBlock / 64);
     SGNN_REQUIRE(nb < INT32_MAX, "too many rows");
-    hipLaunchKernelGGL(dequant_v1_kernel, dim3((uint32_t)nb), dim3(kQBlock), 0, (hipStream_t)stream, q, x, range, params, n, (int)F);
+    ProfScope prof(K_DEQUANT_V1, (hipStream_t)stream);
+    const dim3 grid((uint32_t)nb), block(kQBlock);
+    const auto grid_r = [&](int rows) { return dim3((uint32_t)((nb + rows - 1) / rows)); };
+    hipStream_t st = (hipStream_t)stream;
+    if (F % 4 == 0 && F <= 1024 && aligned(x, 16)) {
+        if (F <= 256) hipLaunchKernelGGL((dequant_v1_vec_kernel<1, 4>), grid_r(4), block, 0, st, q, x, range, params, n, (int)F);
+        else if (F <= 512) hipLaunchKernelGGL((dequant_v1_vec_kernel<2, 2>), grid_r(2), block, 0, st, q, x, range, params, n, (int)F);
+        else hipLaunchKernelGGL((dequant_v1_vec_kernel<4, 1>), grid, block, 0, st, q, x, range, params, n, (int)F);
+    } else {
+        hipLaunchKernelGGL(dequant_v1_kernel, grid, block, 0, st, q, x, range, params, n, (int)F);
+    }
     SGNN_HIP_CHECK(hipGetLastError());
     return SGNN_OK;
 }

@@ -365,3 +365,30 @@ def test_cpu_runnable_configuration_int8_boundary_rows():
     tol = dequant_atol(p_ref[:, 0], p_ref[:, 1], 8)[:, None]
     assert np.all(np.abs(back.cpu().numpy() - want) <= tol)
     assert np.all(np.abs(back.cpu().numpy() - x.numpy()) <= p_ref[:, 1:2] * 0.5 * (1 + 1e-6) + 4 * tol)
+
+
+@pytest.mark.parametrize("F", [4, 12, 100, 128, 256, 600, 1024, 1028, 37])
+def test_v1_mixed_bits_all_widths(F):
+    """Feature-packed mixed-bit rows (2/4/8 bits chosen per row, so row byte offsets fall on every
+    alignment): bytes and params bit-exact vs the oracle, floats within one rounding; widths on both
+    the float4 kernels (F % 4 == 0, F <= 1024) and the general ones."""
+    from super_gnn_amd import supergnn_ops as ops
+    rng_ = np.random.default_rng(F)
+    n = 777
+    x = (rng_.standard_normal((n, F)) * np.exp(rng_.uniform(-5, 5, size=(n, 1)))).astype(np.float32)
+    x[5] = 0.0; x[6] = -0.0; x[7] = 2.5
+    if F > 1:
+        x[8, 0] = 0.0; x[8, 1] = -0.0
+    bits = rng_.choice([2, 4, 8], size=n)
+    q_ref, r_ref, p_ref = orc.quant_v1(x, bits)
+    q = torch.zeros(q_ref.shape[0], dtype=torch.uint8, device="cuda")
+    prm = torch.zeros(n, 3, device="cuda"); prm[:, 0] = torch.from_numpy(bits.astype(np.float32)).cuda()
+    r = torch.from_numpy(r_ref).cuda()
+    ops.quantize_tensor_v1(torch.from_numpy(x).cuda(), q, r, prm)
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    assert np.array_equal(prm.cpu().numpy(), p_ref)
+    back = torch.full((n, F), 9.0, device="cuda")
+    ops.dequantize_tensor_v1(q, back, r, prm)
+    want = orc.dequant_v1(q_ref, r_ref, p_ref, F)
+    tol = dequant_atol(p_ref[:, 1], p_ref[:, 2], bits)[:, None]
+    assert np.all(np.abs(back.cpu().numpy() - want) <= tol)
