@@ -793,13 +793,26 @@ __global__ __launch_bounds__(kQBlock) void quant_v1_vec_kernel(const float *__re
         float s = (mx - mn) / (float)((1 << b) - 1);
         if (s == 0.0f) s = 1.0f;
         if (lane == 0) { params[i * 3 + 1] = mn; params[i * 3 + 2] = s; }
+        const float rinv = __builtin_amdgcn_rcpf(s);
         uint8_t *qo = q + r0[r];
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             if (!act[v]) continue;
+            // product with the hardware reciprocal first, IEEE division only for a lane that sees an
+            // element within 2^-13 of a rounding tie (same argument as in quant_pack_rows16_kernel)
             uint32_t c[4];
+            bool redo = !(s >= 0x1p-100f && s <= 0x1p100f);
 #pragma unroll
-            for (int k = 0; k < 4; ++k) c[k] = quant_code(xv[r][v][k], mn, s);
+            for (int k = 0; k < 4; ++k) {
+                const float qf = (xv[r][v][k] - mn) * rinv;
+                const float ri = rintf(qf);
+                if (!(fabsf(qf - ri) < 0.5f - 0x1p-13f)) redo = true;
+                c[k] = (uint32_t)ri;
+            }
+            if (redo) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) c[k] = quant_code(xv[r][v][k], mn, s);
+            }
             if (b == 8) {
                 uint8_t *dst = qo + off[v];
                 if ((r0[r] & 3) == 0) {

@@ -380,6 +380,15 @@ def test_v1_mixed_bits_all_widths(F):
     if F > 1:
         x[8, 0] = 0.0; x[8, 1] = -0.0
     bits = rng_.choice([2, 4, 8], size=n)
+    # rows of rounding ties and their one-ulp neighbours: min 0, max 2^b - 1 (scale exactly 1), and a
+    # scale that is not a power of two
+    for row, b in ((9, 8), (10, 4), (11, 2), (12, 8), (13, 2)):
+        bits[row] = b
+        qmax = float((1 << b) - 1)
+        ties = (rng_.integers(0, int(qmax), size=F) + 0.5).astype(np.float32)
+        ties = np.nextafter(ties, ties + rng_.choice([-1.0, 0.0, 1.0], size=F).astype(np.float32)).astype(np.float32)
+        ties[0], ties[-1] = 0.0, qmax
+        x[row] = ties * (np.float32(1.0) if row < 12 else np.float32(0.3))
     q_ref, r_ref, p_ref = orc.quant_v1(x, bits)
     q = torch.zeros(q_ref.shape[0], dtype=torch.uint8, device="cuda")
     prm = torch.zeros(n, 3, device="cuda"); prm[:, 0] = torch.from_numpy(bits.astype(np.float32)).cuda()
