@@ -9,7 +9,6 @@
 // quantize+pack kernel keeps the rows it packs in registers between the min/max reduction and the
 // quantization, so the fp32 input is read from memory exactly once.
 #include <algorithm>
-#include <cfloat>
 #include <climits>
 #include <cstdlib>
 
@@ -177,9 +176,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
         zp[r] = 0.0f;
         sc[r] = 1.0f;
         if (!valid[r]) continue;
-        float mn = FLT_MAX, mx = -FLT_MAX;
-        mn = INFINITY;
-        mx = -INFINITY;
+        float mn = INFINITY, mx = -INFINITY;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             if (!act[v]) continue;

@@ -5,20 +5,22 @@
 //
 // The work is a random gather of dense rows, bound by memory bandwidth and latency; there is no
 // MFMA here.  Scheduling is by row class:
-//   * short rows (degree <= threshold): consecutive rows are cut into chunks of ~128 edges; one
-//     group of G lanes owns one chunk.  G*VEC*NV floats cover the feature axis (F=128: 32 lanes x
-//     float4, two chunks per wavefront).  Because the edges of consecutive CSR rows are contiguous,
-//     the group streams the chunk's (col,val) pairs G at a time with one coalesced load, broadcasts
-//     them lane by lane and keeps U whole-row gathers in flight regardless of where rows begin
-//     and end; a row boundary only switches the accumulator (store the finished row, continue with
-//     the next one, whose old value was prefetched).  Edges are summed in CSR order with one fma
-//     per edge, starting from the old out value: the same operation sequence as the reference's
-//     kernel_1xN (spmm.cpp:87-162), so these rows are bit-identical to the reference.
-//   * long rows (power-law hubs): at plan time the row's edges are regrouped by column class
-//     (a hash of the column index, 8 classes) and each class run is cut into pieces; one lane group sums one piece into a partial
-//     buffer, and a last small kernel adds a row's partials in piece order (deterministic, no
-//     float atomics).  Workgroup i only takes pieces of class i % 8, i.e. each XCD gathers only
-//     its own class of dense rows, so the eight L2 caches hold disjoint sets of popular rows.
+//   * short rows (degree <= threshold): consecutive rows are cut into chunks of about 64 edges (fewer
+//     on small matrices, so that the chip stays full); one group of G lanes owns one chunk.
+//     G*VEC*NV floats cover the feature axis (F=128: 32 lanes x float4, two chunks per wavefront).
+//     Because the edges of consecutive CSR rows are contiguous, the group streams the chunk's
+//     (col,val) pairs G at a time with one coalesced load, broadcasts them lane by lane and keeps
+//     several whole-row gathers in flight regardless of where rows begin and end; a row boundary
+//     only switches the accumulator (store the finished row, continue with the next one, whose old
+//     value was prefetched).  Edges are summed in CSR order with one fma per edge, starting from
+//     the old out value: the same operation sequence as the reference's kernel_1xN
+//     (spmm.cpp:87-162), so these rows are bit-identical to the reference.
+//   * long rows (power-law hubs): at plan time the row's edges are regrouped by column class (a
+//     hash of the column index, 8 classes) and each class run is cut into pieces; one lane group
+//     sums one piece into a partial buffer, and a last small kernel adds a row's partials in piece
+//     order (deterministic, no float atomics).  Workgroup i only takes pieces of class i % 8, i.e.
+//     each XCD gathers only its own class of dense rows, so the eight L2 caches hold disjoint sets
+//     of popular rows.
 #include <algorithm>
 #include <cstdlib>
 #include <functional>
@@ -371,9 +373,9 @@ __global__ __launch_bounds__(kBlock) void spmm_empty_rows_kernel(const int32_t *
 }
 
 // ------------------------------------------------------------------------------------------------
-// Long rows, step 1: pieces.  At plan time a long row's edges are regrouped by column class
-// (a hash of the column index, 8 classes) and each class run is cut into pieces; a piece is summed by one lane group into
-// partial[piece, :].  All pieces a workgroup handles belong to ONE class, and workgroup i takes
+// Long rows, step 1: pieces.  At plan time a long row's edges are regrouped by column class (a hash
+// of the column index, 8 classes) and each class run is cut into pieces; a piece is summed by one
+// lane group into partial[piece, :].  All pieces a workgroup handles belong to ONE class, and workgroup i takes
 // class i % 8: workgroups are dealt round-robin to the 8 XCDs, so every XCD gathers only the dense
 // rows of its own class and the eight 4 MB L2s hold eight DISJOINT sets of popular rows instead of
 // eight copies of the same set.
@@ -778,6 +780,13 @@ extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     return SGNN_OK;
 }
 
+// A plan-time device temporary, freed on every way out of the scope.
+template <typename T>
+struct DevTmp {
+    T *p = nullptr;
+    ~DevTmp() { (void)hipFree(p); }
+};
+
 template <typename T>
 static int upload(T **dst, const std::vector<T> &src, hipStream_t st) {
     if (src.empty()) return SGNN_OK;
@@ -821,22 +830,18 @@ static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void
     int rc = upload(&p->empty_rows, empty_rows, st);
     if (rc != SGNN_OK) return rc;
     if (nnz > 0) {
-        int *bad = nullptr;
-        SGNN_HIP_CHECK(hipMalloc(&bad, sizeof(int)));
-        SGNN_HIP_CHECK(hipMemsetAsync(bad, 0, sizeof(int), st));
+        DevTmp<int> bad;
+        SGNN_HIP_CHECK(hipMalloc(&bad.p, sizeof(int)));
+        SGNN_HIP_CHECK(hipMemsetAsync(bad.p, 0, sizeof(int), st));
         const int nb = (int)std::min<int64_t>((nnz + kBlock - 1) / kBlock, 65536);
         if (col_is_i64)
-            hipLaunchKernelGGL((narrow_cols_kernel<int64_t>), dim3(nb), dim3(kBlock), 0, st, (const int64_t *)col, p->col, nnz, K, bad);
+            hipLaunchKernelGGL((narrow_cols_kernel<int64_t>), dim3(nb), dim3(kBlock), 0, st, (const int64_t *)col, p->col, nnz, K, bad.p);
         else
-            hipLaunchKernelGGL((narrow_cols_kernel<int32_t>), dim3(nb), dim3(kBlock), 0, st, (const int32_t *)col, p->col, nnz, K, bad);
+            hipLaunchKernelGGL((narrow_cols_kernel<int32_t>), dim3(nb), dim3(kBlock), 0, st, (const int32_t *)col, p->col, nnz, K, bad.p);
         int h_bad = 0;
-        hipError_t e1 = hipGetLastError();
-        hipError_t e2 = hipMemcpyAsync(&h_bad, bad, sizeof(int), hipMemcpyDeviceToHost, st);
-        hipError_t e3 = hipStreamSynchronize(st);
-        (void)hipFree(bad);
-        SGNN_HIP_CHECK(e1);
-        SGNN_HIP_CHECK(e2);
-        SGNN_HIP_CHECK(e3);
+        SGNN_HIP_CHECK(hipGetLastError());
+        SGNN_HIP_CHECK(hipMemcpyAsync(&h_bad, bad.p, sizeof(int), hipMemcpyDeviceToHost, st));
+        SGNN_HIP_CHECK(hipStreamSynchronize(st));
         if (h_bad) return fail(SGNN_ERR_RANGE, "a column index lies outside [0, %lld)", (long long)K);
     }
 
@@ -852,19 +857,15 @@ static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void
         } else if (K <= kPopularColumns) {
             p->partitioned = true;  // every dense row is "popular": eight disjoint slices beat eight full copies
         } else {
-            int *pop = nullptr;
-            SGNN_HIP_CHECK(hipMalloc(&pop, sizeof(int) * (size_t)K));
-            SGNN_HIP_CHECK(hipMemsetAsync(pop, 0, sizeof(int) * (size_t)K, st));
+            DevTmp<int> pop;
+            SGNN_HIP_CHECK(hipMalloc(&pop.p, sizeof(int) * (size_t)K));
+            SGNN_HIP_CHECK(hipMemsetAsync(pop.p, 0, sizeof(int) * (size_t)K, st));
             const int nb = (int)std::min<int64_t>((nnz + kBlock - 1) / kBlock, 65536);
-            hipLaunchKernelGGL(column_popularity_kernel, dim3(nb), dim3(kBlock), 0, st, p->col, nnz, pop);
+            hipLaunchKernelGGL(column_popularity_kernel, dim3(nb), dim3(kBlock), 0, st, p->col, nnz, pop.p);
             std::vector<int> h_pop((size_t)K);
-            hipError_t e1 = hipGetLastError();
-            hipError_t e2 = hipMemcpyAsync(h_pop.data(), pop, sizeof(int) * h_pop.size(), hipMemcpyDeviceToHost, st);
-            hipError_t e3 = hipStreamSynchronize(st);
-            (void)hipFree(pop);
-            SGNN_HIP_CHECK(e1);
-            SGNN_HIP_CHECK(e2);
-            SGNN_HIP_CHECK(e3);
+            SGNN_HIP_CHECK(hipGetLastError());
+            SGNN_HIP_CHECK(hipMemcpyAsync(h_pop.data(), pop.p, sizeof(int) * h_pop.size(), hipMemcpyDeviceToHost, st));
+            SGNN_HIP_CHECK(hipStreamSynchronize(st));
             std::nth_element(h_pop.begin(), h_pop.begin() + kPopularColumns, h_pop.end(), std::greater<int>());
             int64_t top = 0;
             for (int i = 0; i < kPopularColumns; ++i) top += h_pop[i];
@@ -874,22 +875,17 @@ static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void
         }
         std::vector<int32_t> cls_count;
         if (p->partitioned) {
-            int32_t *d_long_off = nullptr, *d_cls_count = nullptr;
-            if ((rc = upload(&d_long_off, long_off, st)) != SGNN_OK) return rc;
-            SGNN_HIP_CHECK(hipMalloc(&d_cls_count, sizeof(int32_t) * (size_t)p->n_long * kNumXCD));
+            DevTmp<int32_t> d_long_off, d_cls_count;
+            if ((rc = upload(&d_long_off.p, long_off, st)) != SGNN_OK) return rc;
+            SGNN_HIP_CHECK(hipMalloc(&d_cls_count.p, sizeof(int32_t) * (size_t)p->n_long * kNumXCD));
             SGNN_HIP_CHECK(hipMalloc(&p->col_long, sizeof(int32_t) * (size_t)p->long_edges));
             SGNN_HIP_CHECK(hipMalloc(&p->eperm, sizeof(int32_t) * (size_t)p->long_edges));
             hipLaunchKernelGGL(partition_long_rows_kernel, dim3((uint32_t)p->n_long), dim3(kBlock), 0, st, p->rowptr, p->col,
-                               p->long_rows, d_long_off, p->col_long, p->eperm, d_cls_count);
+                               p->long_rows, d_long_off.p, p->col_long, p->eperm, d_cls_count.p);
             cls_count.resize((size_t)p->n_long * kNumXCD);
-            hipError_t e1 = hipGetLastError();
-            hipError_t e2 = hipMemcpyAsync(cls_count.data(), d_cls_count, sizeof(int32_t) * cls_count.size(), hipMemcpyDeviceToHost, st);
-            hipError_t e3 = hipStreamSynchronize(st);
-            (void)hipFree(d_long_off);
-            (void)hipFree(d_cls_count);
-            SGNN_HIP_CHECK(e1);
-            SGNN_HIP_CHECK(e2);
-            SGNN_HIP_CHECK(e3);
+            SGNN_HIP_CHECK(hipGetLastError());
+            SGNN_HIP_CHECK(hipMemcpyAsync(cls_count.data(), d_cls_count.p, sizeof(int32_t) * cls_count.size(), hipMemcpyDeviceToHost, st));
+            SGNN_HIP_CHECK(hipStreamSynchronize(st));
         } else {
             p->col_long = p->col;  // pieces index the CSR arrays directly; no permutation
             p->eperm = nullptr;
