@@ -363,3 +363,67 @@ def test_steady_state_calls_replay_from_a_captured_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, want) and torch.equal(out_q, want_q), f"replay {i}"
+
+
+def test_full_size_graph_exact_on_small_integers():
+    # The headline shape (2.45 M nodes, ~62 M edges, F = 128).  With small integer features and weights every
+    # partial sum is an integer below 2^24, so fp32 addition is exact in any order and the product has ONE
+    # right answer: the kernels (short rows, class-regrouped long rows, final sums, mean epilogue, transpose)
+    # must reproduce it bit for bit.  The expected values are accumulated in fp64 with index_add_.
+    from super_gnn_amd import synth
+    ops = _gpu()
+    dev = torch.device("cuda:0")
+    n, F = 2_450_000, 128
+    rowptr, col = synth.rmat_graph(n, 31_000_000, seed=1, device=dev)
+    nnz = int(col.numel())
+    g = torch.Generator(device=dev); g.manual_seed(11)
+    w = torch.randint(1, 3, (nnz,), generator=g, device=dev).float()
+    x = torch.randint(-4, 5, (n, F), generator=g, device=dev).float()
+    deg = rowptr[1:] - rowptr[:-1]
+    assert int(deg.max()) * 8 < 2 ** 24
+    rows = torch.repeat_interleave(torch.arange(n, device=dev), deg)
+
+    def expected(init):
+        want = init.double()
+        step = 1 << 22
+        for e0 in range(0, nnz, step):
+            e1 = min(nnz, e0 + step)
+            want.index_add_(0, rows[e0:e1], x[col[e0:e1]].double() * w[e0:e1, None].double())
+        return want
+
+    plan = ops.SpmmPlan(rowptr, col.to(torch.int32), n)
+    info = plan.info()
+    assert info["long_rows"] > 1000 and info["partitioned"] == 1
+    init = torch.randint(-3, 4, (n, F), generator=g, device=dev).float()
+    want = expected(init)
+    out = init.clone()
+    plan.run(w, x, out, accumulate=True)
+    assert torch.equal(out.double(), want)
+    # a second call takes the bound-weights path for the long rows: same answer
+    out2 = init.clone()
+    plan.run(w, x, out2, accumulate=True)
+    assert torch.equal(out2, out)
+    # overwrite mode + mean epilogue: (A x) / max(deg, 1), one correctly rounded division per element
+    div = deg.clamp(min=1).float()
+    out3 = torch.full((n, F), 7.0, device=dev)
+    plan.run(w, x, out3, accumulate=False, row_div=div)
+    want3 = (want - init.double()).float() / div[:, None]
+    assert torch.equal(out3, want3)
+    del want, want3, out2, out3
+    # the fused int8 path on the same graph: rows quantized with scale 1 decode to the integers again
+    seg = torch.tensor([0, n], dtype=torch.int32)
+    q = torch.empty(n, F, dtype=torch.uint8, device=dev)
+    p = torch.empty(n, 2, device=dev)
+    x8 = x.clone(); x8[:, 0] = -100.0; x8[:, 1] = 155.0   # every row spans exactly 255 steps of 1.0
+    ops.quantize_tensor_for_all_procs(x8, q, p, seg, 1, 8)
+    assert bool((p[:, 1] == 1.0).all()) and bool((p[:, 0] == -100.0).all())
+    d8 = torch.empty_like(x8)
+    ops.dequantize_tensor_for_all_procs(q, d8, p, seg, 1, 8)
+    assert torch.equal(d8, x8)
+    w1 = torch.ones_like(w)   # keep the sums of the two wide columns below 2^24
+    assert int(deg.max()) * 155 < 2 ** 24
+    ref = torch.zeros(n, F, device=dev)
+    plan.run(w1, x8, ref, accumulate=True)
+    fused = torch.zeros(n, F, device=dev)
+    plan.run_quantized(w1, q, p, ops.quant_segments(seg, 8), 8, fused, accumulate=True)
+    assert torch.equal(fused, ref)
