@@ -153,3 +153,68 @@ def test_fused_with_bf16_params_equals_widened_params(bits, hubs):
     assert torch.equal(a, b)
     with pytest.raises(TypeError):
         plan.run_quantized(v, q, params.to(torch.float16), segs, bits, a, accumulate=True)
+
+
+@pytest.fixture(scope="module")
+def full_size_partition():
+    # One partition at the largest configured size: 8 M local rows with ~320 M local edges, plus ~80 M edges
+    # to 2 M remote boundary rows.  Built once on the GPU, together with the exact local product in fp64.
+    import super_gnn_amd  # noqa: F401
+    from super_gnn_amd import supergnn_ops as ops, synth
+    dev = torch.device("cuda:0")
+    Ml, Kr, F = 8_000_000, 2_000_000, 128
+    rp_l, col_l = synth.rmat_graph(Ml, 160_000_000, seed=6, device=dev)
+    g = torch.Generator(device=dev); g.manual_seed(7)
+    deg_l = rp_l[1:] - rp_l[:-1]
+    rows_r = torch.multinomial(deg_l.float() + 0.05, 80_000_000, replacement=True, generator=g)
+    cols_r = torch.randint(0, Kr, (80_000_000,), generator=g, device=dev)
+    rp_r, col_r = synth.csr_from_pairs(rows_r, cols_r, Ml, Kr, dedupe=True)
+    del rows_r, cols_r
+    x_l = torch.randint(-4, 5, (Ml, F), generator=g, device=dev).float()
+    plan_l = ops.SpmmPlan(rp_l, col_l.to(torch.int32), Ml)
+    plan_r = ops.SpmmPlan(rp_r, col_r.to(torch.int32), Kr)
+    local = torch.zeros(Ml, F, dtype=torch.float64, device=dev)
+    _index_add_product(local, rp_l, col_l, x_l)
+    yield dict(ops=ops, dev=dev, Ml=Ml, Kr=Kr, F=F, g=g, x_l=x_l, plan_l=plan_l, plan_r=plan_r, rp_r=rp_r, col_r=col_r,
+               local=local, max_deg_l=int(deg_l.max()), max_deg_r=int((rp_r[1:] - rp_r[:-1]).max()))
+
+
+def _index_add_product(acc, rp, col, x, step=1 << 22):
+    rows = torch.repeat_interleave(torch.arange(rp.numel() - 1, device=col.device), rp[1:] - rp[:-1])
+    for e0 in range(0, int(col.numel()), step):
+        e1 = min(int(col.numel()), e0 + step)
+        acc.index_add_(0, rows[e0:e1], x[col[e0:e1]].double())
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_full_size_partition_exact_on_small_integers(bits, full_size_partition):
+    # The remote rows arrive packed from 8 senders (ragged segments).  Integer features that the quantizer
+    # represents exactly (every row spans exactly 2^bits - 1 steps of 1.0) and unit weights make every sum
+    # exact in fp32, so local SpMM + fused remote SpMM has one right answer, checked against fp64.
+    w = full_size_partition
+    ops, dev, Ml, Kr, F, g = w["ops"], w["dev"], w["Ml"], w["Kr"], w["F"], w["g"]
+    P, top = 8, 2 ** bits - 1
+    assert w["max_deg_l"] * 4 + w["max_deg_r"] * (top + 5) < 2 ** 24
+    zp = torch.randint(-5, 6, (Kr, 1), generator=g, device=dev).float()
+    x_r = torch.randint(0, top + 1, (Kr, F), generator=g, device=dev).float() + zp
+    x_r[:, 0:1] = zp
+    x_r[:, 1:2] = zp + top
+    bounds = [0] + sorted(int(v) for v in torch.randint(1, Kr, (P - 1,), generator=g, device=dev).tolist()) + [Kr]
+    wr = torch.tensor(bounds, dtype=torch.int32)   # ragged: segments do not end on packed-row boundaries
+    epb = 8 // bits
+    npk = sum((bounds[i + 1] - bounds[i] + epb - 1) // epb for i in range(P))
+    q = torch.empty(npk, F, dtype=torch.uint8, device=dev)
+    prm = torch.empty(Kr, 2, device=dev)
+    ops.quantize_tensor_for_all_procs(x_r, q, prm, wr, P, bits)
+    assert torch.equal(prm[:, 0:1], zp) and bool((prm[:, 1] == 1.0).all())
+    back = torch.empty_like(x_r)
+    ops.dequantize_tensor_for_all_procs(q, back, prm, wr, P, bits)
+    assert torch.equal(back, x_r)
+    del back
+
+    out = torch.full((Ml, F), 3.0, device=dev)
+    w["plan_l"].run(None, w["x_l"], out, accumulate=False)
+    w["plan_r"].run_quantized(None, q, prm, ops.quant_segments(wr, bits), bits, out, accumulate=True)
+    want = w["local"].clone()
+    _index_add_product(want, w["rp_r"], w["col_r"], x_r)
+    assert torch.equal(out.double(), want)
