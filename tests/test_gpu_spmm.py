@@ -427,3 +427,35 @@ def test_full_size_graph_exact_on_small_integers():
     fused = torch.zeros(n, F, device=dev)
     plan.run_quantized(w1, q, p, ops.quant_segments(seg, 8), 8, fused, accumulate=True)
     assert torch.equal(fused, ref)
+
+
+def test_full_size_community_graph_exact_on_small_integers():
+    # The wide-feature configuration (233 k nodes, ~114 M edges, average degree ~490, F = 602: float2 lanes,
+    # every row on the long-row path), mean aggregation, forward and transpose.  Exact for the same reason
+    # as the test above.
+    from super_gnn_amd import synth
+    ops = _gpu()
+    dev = torch.device("cuda:0")
+    n, F = 233_000, 602
+    rowptr, col = synth.sbm_graph(n, 50, 0.03048, 0.001524, seed=3, device=dev)
+    nnz = int(col.numel())
+    g = torch.Generator(device=dev); g.manual_seed(12)
+    x = torch.randint(-4, 5, (n, F), generator=g, device=dev).float()
+    deg = rowptr[1:] - rowptr[:-1]
+    assert int(deg.max()) * 4 < 2 ** 24
+    rows = torch.repeat_interleave(torch.arange(n, device=dev), deg)
+    want = torch.zeros(n, F, dtype=torch.float64, device=dev)
+    step = 1 << 20
+    for e0 in range(0, nnz, step):
+        e1 = min(nnz, e0 + step)
+        want.index_add_(0, rows[e0:e1], x[col[e0:e1]].double())
+    div = deg.clamp(min=1).float()
+    plan = ops.SpmmPlan(rowptr, col.to(torch.int32), n)
+    assert plan.info()["long_rows"] > n // 2
+    out = torch.full((n, F), -1.0, device=dev)
+    plan.run(None, x, out, accumulate=False, row_div=div)
+    assert torch.equal(out, want.float() / div[:, None])
+    # the graph is symmetric: the transpose product (backward) is the same matrix
+    out_t = torch.zeros(n, F, device=dev)
+    ops.SpmmPlan(rowptr, col, n).run(torch.ones(nnz, device=dev), x, out_t, accumulate=True)
+    assert torch.equal(out_t.double(), want)
