@@ -546,7 +546,9 @@ def main():
             model.train()
             opt.zero_grad()
             out = torch.cat(model(world, feats))
-            loss = torch.nn.functional.nll_loss(out, labels)
+            # nll_loss(out, labels) written as a gather: torch's nll_loss kernels reduce 2.45 M rows in a
+            # single workgroup (5 ms forward, 4 ms backward)
+            loss = -out.gather(1, labels.view(-1, 1)).mean()
             loss.backward()
             opt.step()
 

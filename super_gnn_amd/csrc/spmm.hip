@@ -339,35 +339,49 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
 }
 
 // Rows without edges, only needed when they must be written: overwrite mode (zeros) or the mean
-// epilogue (old value / divisor).  One lane group per empty row.
+// epilogue (old value / divisor).  One lane group per kEmptyRowsPerGroup empty rows: the row ids (and
+// divisors) of all of them are requested before the first store, so a wave pays the latency of the
+// dependent id -> address chain once, not once per row.
+constexpr int kEmptyRowsPerGroup = 4;
 template <int VEC, int G, int NV>
 __global__ __launch_bounds__(kBlock) void spmm_empty_rows_kernel(const int32_t *__restrict__ empty_rows, int n_empty,
                                                                  float *__restrict__ out, int F, int64_t ldo,
                                                                  int accumulate, const float *__restrict__ row_div) {
     constexpr int GPB = kBlock / G;
     constexpr int TILE = G * VEC * NV;
+    constexpr int R = kEmptyRowsPerGroup;
     const int gid = threadIdx.x / G, lig = threadIdx.x % G;
-    const int i = blockIdx.x * GPB + gid;
-    if (i >= n_empty) return;
-    const int64_t row = empty_rows[i];
-    const float div = row_div ? row_div[row] : 1.0f;
-    // x / 1 == x for every float, so an accumulating call leaves such a row exactly as it is: nothing
-    // to read or write (the mean epilogue divides rows without edges by a degree clamped to 1).
-    if (accumulate && div == 1.0f) return;
-    for (int f0 = 0; f0 < F; f0 += TILE) {
+    const int i0 = (blockIdx.x * GPB + gid) * R;
+    if (i0 >= n_empty) return;
+    int64_t rows[R];
+    float divs[R];
 #pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int off = f0 + (v * G + lig) * VEC;
-            if (off >= F) continue;
-            float a[VEC];
+    for (int r = 0; r < R; ++r) rows[r] = empty_rows[i0 + r < n_empty ? i0 + r : n_empty - 1];
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) a[k] = 0.0f;
-            if (accumulate) vec_load_nt<VEC>(a, out + row * ldo + off);
-            if (row_div) {
+    for (int r = 0; r < R; ++r) divs[r] = row_div ? row_div[rows[r]] : 1.0f;
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) a[k] = a[k] / div;
+    for (int r = 0; r < R; ++r) {
+        if (i0 + r >= n_empty) break;
+        const int64_t row = rows[r];
+        const float div = divs[r];
+        // x / 1 == x for every float, so an accumulating call leaves such a row exactly as it is: nothing
+        // to read or write (the mean epilogue divides rows without edges by a degree clamped to 1).
+        if (accumulate && div == 1.0f) continue;
+        for (int f0 = 0; f0 < F; f0 += TILE) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                const int off = f0 + (v * G + lig) * VEC;
+                if (off >= F) continue;
+                float a[VEC];
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) a[k] = 0.0f;
+                if (accumulate) vec_load_nt<VEC>(a, out + row * ldo + off);
+                if (row_div) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) a[k] = a[k] / div;
+                }
+                vec_store_nt<VEC>(out + row * ldo + off, a);
             }
-            vec_store_nt<VEC>(out + row * ldo + off, a);
         }
     }
 }
@@ -634,7 +648,7 @@ static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &
                            a.dense, a.out, a.chunks, a.n_chunks, a.F, a.ldo, a.accumulate, a.row_div, nb);
     }
     if (a.n_empty > 0 && (!a.accumulate || a.row_div)) {
-        const uint32_t nb = (uint32_t)((a.n_empty + GPB - 1) / GPB);
+        const uint32_t nb = (uint32_t)((a.n_empty + GPB * kEmptyRowsPerGroup - 1) / (GPB * kEmptyRowsPerGroup));
         ProfScope prof(K_SPMM_EMPTY_ROWS, st);
         hipLaunchKernelGGL((spmm_empty_rows_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, a.empty_rows, a.n_empty,
                            a.out, a.F, a.ldo, a.accumulate, a.row_div);

@@ -136,3 +136,27 @@ def test_reference_partition_files_round_trip(tmp_path):
             assert torch.equal(rec["nodes_labels"], label[b:e])
             assert torch.equal(rec["nodes_train_masks"] + b, train[(train >= b) & (train < e)])
             assert rec["graph"] is graphs[rank]
+
+
+def test_sage_combine_matches_the_plain_formula_and_its_gradients():
+    # lin_neigh(agg / deg) + lin_self(x) + bias (sageconv.py:83-89), fused into two accumulating products
+    from super_gnn_amd.layers import _SageCombine
+    g = torch.Generator().manual_seed(3)
+    n, fin, fout = 37, 5, 7
+    mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64, requires_grad=True)
+    agg, x, wn, ws, b = mk(n, fin), mk(n, fin), mk(fout, fin), mk(fout, fin), mk(fout)
+    deg = torch.randint(1, 9, (n, 1), generator=g).double()
+    want = (agg / deg) @ wn.t() + x @ ws.t() + b
+    got = _SageCombine.apply(agg, x, deg, wn, ws, b)
+    assert torch.allclose(got, want, rtol=1e-12, atol=1e-12)
+    assert torch.autograd.gradcheck(_SageCombine.apply, (agg, x, deg, wn, ws, b))
+    assert torch.autograd.gradcheck(lambda a, c, d: _SageCombine.apply(a, x.detach(), None, c, d, None), (agg, wn, ws))
+
+
+def test_split_weight_gradient_equals_the_plain_product():
+    from super_gnn_amd import layers
+    g = torch.Generator().manual_seed(5)
+    n = layers._SPLIT_K * 1024 + 37
+    a, b = torch.randn(n, 6, generator=g, dtype=torch.float64), torch.randn(n, 5, generator=g, dtype=torch.float64)
+    assert torch.allclose(layers._weight_grad(a, b), a.t() @ b, rtol=1e-11, atol=1e-9)
+    assert torch.equal(layers._weight_grad(a[:100], b[:100]), a[:100].t() @ b[:100])
