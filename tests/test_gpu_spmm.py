@@ -459,3 +459,31 @@ def test_full_size_community_graph_exact_on_small_integers():
     out_t = torch.zeros(n, F, device=dev)
     ops.SpmmPlan(rowptr, col, n).run(torch.ones(nnz, device=dev), x, out_t, accumulate=True)
     assert torch.equal(out_t.double(), want)
+
+
+@pytest.mark.parametrize("F,pad_x,pad_o,off_x,off_o", [(128, 64, 32, 16, 8), (128, 3, 5, 1, 2), (602, 2, 6, 2, 4), (64, 0, 64, 0, 64)])
+def test_leading_dimensions_through_the_c_abi(F, pad_x, pad_o, off_x, off_o):
+    # X and out as column windows of wider matrices (ldx, ldo > F; aligned and unaligned starts): same bits as
+    # the contiguous call, and nothing outside the window is written
+    ops = _gpu()
+    from super_gnn_amd._lib import lib, check
+    dev = torch.device("cuda:0")
+    M, K = 3000, 2500
+    rowptr, col, val = random_csr(M, K, 9, seed=21, empty_frac=0.1, hubs=3, hub_deg=900)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    g = torch.Generator().manual_seed(22)
+    xw = torch.randn(K, F + pad_x, generator=g).to(dev)
+    ow = torch.randn(M, F + pad_o, generator=g).to(dev)
+    w = torch.from_numpy(val).to(dev)
+    div = torch.from_numpy(np.maximum(np.diff(rowptr), 1).astype(np.float32)).to(dev)
+    for accumulate, row_div in ((1, None), (0, None), (1, div)):
+        want = ow[:, off_o:off_o + F].contiguous()
+        plan.run(w, xw[:, off_x:off_x + F].contiguous(), want, accumulate=bool(accumulate), row_div=row_div)
+        got = ow.clone()
+        check(lib.sgnn_spmm_csr_f32(plan._h, w.data_ptr(), xw.data_ptr() + 4 * off_x, got.data_ptr() + 4 * off_o, F,
+                                    F + pad_x, F + pad_o, accumulate, row_div.data_ptr() if row_div is not None else None,
+                                    torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert torch.equal(got[:, off_o:off_o + F], want)
+        keep = torch.ones(F + pad_o, dtype=torch.bool, device=dev); keep[off_o:off_o + F] = False
+        assert torch.equal(got[:, keep], ow[:, keep])
