@@ -155,6 +155,32 @@ def test_fused_with_bf16_params_equals_widened_params(bits, hubs):
         plan.run_quantized(v, q, params.to(torch.float16), segs, bits, a, accumulate=True)
 
 
+def test_fused_output_window_through_the_c_abi():
+    # out as a 16-byte-aligned column window of a wider matrix (ldo > F): same bits, nothing else written;
+    # a window that is not 16-byte aligned is refused
+    from super_gnn_amd._lib import lib, check
+    bits, F = 4, 128
+    ops, plan, rowptr, col, val, x, seg_t, P, q, params = _setup(1500, 2000, F, 7, bits, [0, 700, 1303, 2000], seed=31, hubs=2)
+    w = torch.from_numpy(val).cuda()
+    segs = ops.quant_segments(seg_t, bits)
+    ow = torch.randn(1500, F + 32, generator=torch.Generator().manual_seed(32)).cuda()
+    want = ow[:, 16:16 + F].contiguous()
+    plan.run_quantized(w, q, params, segs, bits, want, accumulate=True)
+    got = ow.clone()
+    slots = segs.row_slots(bits)
+    stream = torch.cuda.current_stream().cuda_stream
+    check(lib.sgnn_spmm_csr_dq_f32(plan._h, w.data_ptr(), q.data_ptr(), params.data_ptr(),
+                                   slots.data_ptr() if slots is not None else None, bits, got.data_ptr() + 64, F, F + 32, 1,
+                                   None, stream))
+    torch.cuda.synchronize()
+    assert torch.equal(got[:, 16:16 + F], want)
+    assert torch.equal(got[:, :16], ow[:, :16]) and torch.equal(got[:, 16 + F:], ow[:, 16 + F:])
+    rc = lib.sgnn_spmm_csr_dq_f32(plan._h, w.data_ptr(), q.data_ptr(), params.data_ptr(),
+                                  slots.data_ptr() if slots is not None else None, bits, got.data_ptr() + 8, F, F + 32, 1,
+                                  None, stream)
+    assert rc != 0 and b"aligned" in lib.sgnn_last_error()
+
+
 @pytest.fixture(scope="module")
 def full_size_partition():
     # One partition at the largest configured size: 8 M local rows with ~320 M local edges, plus ~80 M edges
