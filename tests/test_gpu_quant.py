@@ -401,3 +401,39 @@ def test_v1_mixed_bits_all_widths(F):
     want = orc.dequant_v1(q_ref, r_ref, p_ref, F)
     tol = dequant_atol(p_ref[:, 1], p_ref[:, 2], bits)[:, None]
     assert np.all(np.abs(back.cpu().numpy() - want) <= tol)
+
+
+def test_offsets_beyond_four_gigabytes():
+    # 9 M x 128 fp32 = 4.6 GB: byte offsets of the last rows do not fit 32 bits.  Params against torch's
+    # min/max, the round-trip bound everywhere, and the last rows of every segment bit-exact against the oracle.
+    ops = _ops()
+    n, F, bits, P = 9_000_000, 128, 2, 3
+    epb = 8 // bits
+    g = torch.Generator(device="cuda"); g.manual_seed(41)
+    x = torch.randn(n, F, generator=g, device="cuda")
+    bounds = [0, 2_999_999, 6_000_002, n]
+    seg = torch.tensor(bounds, dtype=torch.int32)
+    pk = [(bounds[i + 1] - bounds[i] + epb - 1) // epb for i in range(P)]
+    q = torch.empty(sum(pk), F, dtype=torch.uint8, device="cuda")
+    p = torch.empty(n, 2, device="cuda")
+    ops.quantize_tensor_for_all_procs(x, q, p, seg, P, bits)
+    mn, mx = x.min(dim=1).values, x.max(dim=1).values
+    assert torch.equal(p[:, 0], mn)
+    assert torch.equal(p[:, 1], (mx - mn) / torch.full_like(mx, float(2 ** bits - 1)))
+    d = torch.empty_like(x)
+    ops.dequantize_tensor_for_all_procs(q, d, p, seg, P, bits)
+    slack = (p[:, 0:1].abs() + float(2 ** bits - 1) * p[:, 1:2]) * 2.0 ** -22 + 1e-30
+    assert bool(((d - x).abs() <= p[:, 1:2] * 0.5 + slack).all())
+    pstart = 0
+    for i in range(P):
+        rows = bounds[i + 1] - bounds[i]
+        tail = (rows - 1) // epb * epb - 4096          # a packed-row-aligned window ending at the segment's last row
+        xs = x[bounds[i] + tail:bounds[i + 1]].cpu().numpy()
+        q_ref, p_ref = orc.quant_rows(xs, [0, xs.shape[0]], bits)
+        q_got = q[pstart + tail // epb:pstart + pk[i]].cpu().numpy()
+        assert np.array_equal(q_got, q_ref)
+        assert np.array_equal(p[bounds[i] + tail:bounds[i + 1]].cpu().numpy().view(np.uint32), p_ref.view(np.uint32))
+        d_ref = orc.dequant_rows(q_ref, p_ref, [0, xs.shape[0]], bits, F)
+        d_got = d[bounds[i] + tail:bounds[i + 1]].cpu().numpy()
+        assert np.all(np.abs(d_got - d_ref) <= dequant_atol(p_ref[:, 0], p_ref[:, 1], bits)[:, None])
+        pstart += pk[i]
