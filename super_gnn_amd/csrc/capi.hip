@@ -1,4 +1,4 @@
-// Error reporting and version of the C ABI.
+// Error reporting, the HIP-event profiler behind bench.py, the streaming-copy yardstick and the ABI version.
 #include <algorithm>
 #include <atomic>
 #include <mutex>

@@ -11,7 +11,6 @@
 
 namespace sgnn {
 
-constexpr int kWave = 64;
 constexpr int kNumXCD = 8;  // MI355X: 8 accelerator dies, each with its own L2
 
 std::string &last_error();
@@ -66,21 +65,6 @@ __device__ __forceinline__ uint32_t xcd_contiguous_block(uint32_t bid, uint32_t 
     const uint32_t xcd = bid % kNumXCD, idx = bid / kNumXCD;
     return xcd * per + (xcd < rem ? xcd : rem) + idx;
 }
-
-template <int VEC>
-struct VecT;
-template <>
-struct VecT<1> {
-    using type = float;
-};
-template <>
-struct VecT<2> {
-    using type = float2;
-};
-template <>
-struct VecT<4> {
-    using type = float4;
-};
 
 template <int VEC>
 __device__ __forceinline__ void vec_load(float (&r)[VEC], const float *p) {
