@@ -90,3 +90,42 @@ def test_quant_random_shapes(case):
     want = orc.dequant_rows(q_ref, p_used, seg, bits, F)
     tol = dequant_atol(p_used[:, 0], p_used[:, 1], bits)[:, None]
     assert np.all(np.abs(back.cpu().numpy() - want) <= tol), f"case {case}"
+
+
+@pytest.mark.parametrize("case", range(30))
+def test_fused_random_shapes(case):
+    # random widths (every lane-group shape), ragged segments, hub rows, fp32 / bf16 params, all epilogues:
+    # the fused product must equal dequantize-then-SpMM on the same plan bit for bit
+    from super_gnn_amd import supergnn_ops as ops
+    rng = np.random.default_rng(3000 + case)
+    bits = int(rng.choice([8, 4, 2]))
+    F = int(rng.choice([4, 8, 12, 36, 64, 100, 128, 256, 260, 512, 1028]))
+    M, K = int(rng.integers(1, 1500)), int(rng.integers(8, 1500))
+    deg = int(rng.choice([1, 3, 9, 40]))
+    hubs = int(rng.choice([0, 0, 3]))
+    rowptr, col, val = random_csr(M, K, deg, seed=3000 + case, empty_frac=0.2, hubs=hubs, hub_deg=min(2 * K, 700))
+    P = int(rng.choice([1, 2, 7]))
+    cuts = np.sort(rng.integers(0, K + 1, size=P - 1))
+    seg = np.concatenate([[0], cuts, [K]]).astype(np.int32)
+    seg_t = torch.from_numpy(seg)
+    x = torch.from_numpy((rng.standard_normal((K, F)) * np.exp(rng.uniform(-3, 3, size=(K, 1)))).astype(np.float32)).cuda()
+    bf16 = bool(rng.integers(0, 2))
+    npk = int(orc.packed_rows(seg, bits).sum())
+    q = torch.zeros(npk, F, dtype=torch.uint8, device="cuda")
+    prm = torch.zeros(K, 2, device="cuda", dtype=torch.bfloat16 if bf16 else torch.float32)
+    ops.quantize_tensor_for_all_procs(x, q, prm, seg_t, P, bits)
+    recv = torch.empty(K, F, device="cuda")
+    ops.dequantize_tensor_for_all_procs(q, recv, prm, seg_t, P, bits)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).cuda(), torch.from_numpy(col).cuda(), K,
+                        long_row_threshold=int(rng.choice([0, 16, 64])))
+    segs = ops.quant_segments(seg_t, bits)
+    w = torch.from_numpy(val).cuda() if rng.integers(0, 2) else None
+    accumulate = bool(rng.integers(0, 2))
+    div = torch.from_numpy(np.maximum(np.diff(rowptr), 1).astype(np.float32)).cuda() if rng.integers(0, 2) else None
+    init = torch.from_numpy(rng.standard_normal((M, F)).astype(np.float32)).cuda()
+    want, got = init.clone(), init.clone()
+    for _ in range(2):   # the second call runs with the weights and row slots bound to the plan
+        plan.run(w, recv, want, accumulate=accumulate, row_div=div)
+        plan.run_quantized(w, q, prm, segs, bits, got, accumulate=accumulate, row_div=div)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want), f"case {case}: bits={bits} F={F} M={M} K={K} deg={deg} hubs={hubs} P={P} bf16={bf16}"
