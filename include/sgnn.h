@@ -101,6 +101,22 @@ int sgnn_spmm_csr_f32(sgnn_spmm_plan *plan, const float *val, const float *x, fl
                       int64_t F, int64_t ldx, int64_t ldo, int accumulate, const float *row_div,
                       sgnn_stream_t stream);
 
+/* sgnn_spmm_csr_f32 for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same
+ * arguments, same kernels and same results, bit for bit, as sgnn_spmm_csr_f32, but the call
+ * performs no hipMalloc / hipFree and creates no stream or event: the partial sums of the long rows
+ * go to a 64 MiB scratch array that lives inside the library's code object (one copy per GPU, held
+ * until the process ends) instead of the plan's growable buffer.
+ *   - limit: (#long-row pieces of the plan) * F * 4 bytes <= 64 MiB (sgnn_spmm_plan_info, info[4]);
+ *     a larger product is refused with SGNN_ERR_ARG and nothing is launched.  Matrices without long
+ *     rows never touch the scratch and have no limit;
+ *   - every call on one GPU shares that GPU's scratch: two calls whose kernels may overlap in time
+ *     (different streams, different host threads) race on it.  Calls queued on one stream are safe.
+ *     Nothing in the scratch has to start at zero: each call writes every partial it later reads. */
+int sgnn_spmm_csr_f32_noalloc(sgnn_spmm_plan *plan, const float *val, const float *x, float *out,
+                              int64_t F, int64_t ldx, int64_t ldo, int accumulate,
+                              const float *row_div, sgnn_stream_t stream);
+
 /* 1 if the reference's spmm() would take its overwrite branch for this shape
  * (float(nnz)/M/K <= 1e-4 && F > 256, super_gnn/ops/csrc/spmm.cpp:601-602), else 0. */
 int sgnn_spmm_reference_overwrites(int64_t nnz, int64_t M, int64_t K, int64_t F);

@@ -116,4 +116,4 @@ extern "C" int sgnn_stream_copy_f32(const float *src, float *dst, int64_t n, sgn
 
 extern "C" const char *sgnn_last_error(void) { return sgnn::last_error().c_str(); }
 
-extern "C" int sgnn_version(void) { return 1; }
+extern "C" int sgnn_version(void) { return 2; }

@@ -24,6 +24,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <functional>
+#include <mutex>
 #include <vector>
 
 #include "common.hpp"
@@ -699,6 +700,34 @@ static int env_int(const char *name, int dflt) {
     return e ? atoi(e) : dflt;
 }
 
+// ------------------------------------------------------------------------------------------------
+// Scratch of sgnn_spmm_csr_f32_noalloc: the piece partials of the long rows, in a device array the
+// code object itself carries (every GPU the library is loaded on holds its own 64 MiB copy until
+// the process ends).  In host code the array's NAME is only a handle for hipGetSymbolAddress; the
+// address kernels and copies must use is looked up once per device and kept in g_scratch_ptr.
+// ------------------------------------------------------------------------------------------------
+constexpr size_t kScratchFloats = (size_t)16 << 20;  // 64 MiB
+static __device__ __align__(256) float g_spmm_scratch[kScratchFloats];
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static float *g_scratch_ptr[kMaxDevices] = {};
+
+// Address of the CURRENT device's copy of the scratch array (looked up on first use per device).
+static int scratch_for_current_device(float **out) {
+    int dev = 0;
+    SGNN_HIP_CHECK(hipGetDevice(&dev));
+    SGNN_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d beyond the %d this library keeps scratch addresses for", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        float *ptr = nullptr;
+        SGNN_HIP_CHECK(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(g_spmm_scratch)));
+        SGNN_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned a null scratch address on device %d", dev);
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return SGNN_OK;
+}
+
 struct sgnn_spmm_plan {
     int device = 0;
     int64_t M = 0, K = 0, nnz = 0;
@@ -962,6 +991,10 @@ static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void
         if ((rc = upload(&p->cls_work, cls_work, st)) != SGNN_OK) return rc;
     }
     SGNN_HIP_CHECK(hipStreamSynchronize(st));  // the host vectors die at return
+    // The short-row chunk lists of all three lane-group shapes (a few MB in total): no later call has
+    // to build, and therefore allocate, one.
+    for (int which = 0; which < 3; ++which)
+        if ((rc = build_chunks(p, which, st)) != SGNN_OK) return rc;
     return SGNN_OK;
 }
 
@@ -1002,8 +1035,11 @@ extern "C" int sgnn_spmm_reference_overwrites(int64_t nnz, int64_t M, int64_t K,
     return (sparsity <= 0.0001f && F > 256) ? 1 : 0;
 }
 
+// scratch != null: the call must not allocate.  The piece partials then go to `scratch` (scratch_floats
+// floats) instead of the plan's own, growable buffer, and nothing is created on the way.
 static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, int bits, float *out, int64_t F,
-                    int64_t ldo, int accumulate, const float *row_div, hipStream_t st) {
+                    int64_t ldo, int accumulate, const float *row_div, hipStream_t st, float *scratch = nullptr,
+                    size_t scratch_floats = 0) {
     SGNN_REQUIRE(p != nullptr, "plan is null");
     SGNN_REQUIRE(F > 0 && F < (1 << 24), "feature width F=%lld out of range", (long long)F);
     SGNN_REQUIRE(ldo >= F, "leading dimension smaller than F (ldo=%lld F=%lld)", (long long)ldo, (long long)F);
@@ -1013,7 +1049,15 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     SGNN_HIP_CHECK(hipGetDevice(&dev));
     SGNN_REQUIRE(dev == p->device, "plan was created on device %d, current device is %d", p->device, dev);
 
-    if (p->n_items > 0) {
+    float *partial = p->partial;
+    if (scratch != nullptr) {
+        const size_t need = (size_t)p->n_items * (size_t)F;
+        SGNN_REQUIRE(need <= scratch_floats,
+                     "the long rows of this matrix need %zu bytes of partial sums at F=%lld; the scratch of the "
+                     "non-allocating entry point holds %zu bytes (use sgnn_spmm_csr_f32)",
+                     need * sizeof(float), (long long)F, scratch_floats * sizeof(float));
+        partial = scratch;
+    } else if (p->n_items > 0) {
         const size_t need = (size_t)p->n_items * (size_t)F;
         if (need > p->partial_floats) {
             // The old buffer may still be read by work queued on another stream: drain first.
@@ -1024,6 +1068,7 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
             SGNN_HIP_CHECK(hipMalloc(&p->partial, need * sizeof(float)));
             p->partial_floats = need;
         }
+        partial = p->partial;
     }
     int vec = 1;
     if (bits != 0) {
@@ -1037,24 +1082,21 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     const int nvec = (int)(F / vec);
     const int gw = group_width(nvec);
     const int which = gw == 8 ? 0 : gw == 16 ? 1 : 2;
-    if (p->n_chunks[which] < 0) {
-        const int rc = build_chunks(p, which, st);
-        if (rc != SGNN_OK) return rc;
-    }
+    SGNN_REQUIRE(p->n_chunks[which] >= 0, "plan has no chunk list for this feature width (plan creation failed?)");
     ShortArgs a{p->rowptr, p->col, val, dense, out, p->chunks[which], (int)p->n_chunks[which], p->empty_rows,
                 (int)p->n_empty, (int)F, ldo, accumulate, row_div};
-    if (p->side == nullptr && p->n_long > 0 && env_int("SGNN_SPMM_OVERLAP", 0) != 0) {
+    if (scratch == nullptr && p->side == nullptr && p->n_long > 0 && env_int("SGNN_SPMM_OVERLAP", 0) != 0) {
         SGNN_HIP_CHECK(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));  // default priority
         SGNN_HIP_CHECK(hipEventCreateWithFlags(&p->ev_fork, hipEventDisableTiming));
         SGNN_HIP_CHECK(hipEventCreateWithFlags(&p->ev_join, hipEventDisableTiming));
     }
-    PieceArgs s{p->col_long, p->eperm, val, p->partial, p->cls_work, p->max_cls_items, (int)F,
-                p->side, p->ev_fork, p->ev_join};
+    PieceArgs s{p->col_long, p->eperm, val, partial, p->cls_work, p->max_cls_items, (int)F,
+                scratch == nullptr ? p->side : nullptr, p->ev_fork, p->ev_join};
     if (val != nullptr && val == p->bound_val && p->val_long != nullptr) {
         s.eperm = nullptr;   // values already sit in regrouped order: contiguous reads, no indirection
         s.val = p->val_long;
     }
-    FinalArgs f{p->long_rows, p->long_pbeg, p->partial, out, (int)p->n_long, (int)F, ldo, accumulate, row_div};
+    FinalArgs f{p->long_rows, p->long_pbeg, partial, out, (int)p->n_long, (int)F, ldo, accumulate, row_div};
     if (bits != 0) {
         const int fmt = bits + (dense.params.bf16 ? kBf16Params : 0) + (dense.eslot_csr ? kEdgeSlots : 0);
         switch (fmt) {
@@ -1113,6 +1155,19 @@ extern "C" int sgnn_spmm_csr_f32(sgnn_spmm_plan *p, const float *val, const floa
     SGNN_REQUIRE(x != nullptr || p->nnz == 0 || p->M == 0, "x is null");
     DenseSrc d{x, ldx, nullptr, ParamBuf{nullptr, 0}, nullptr, nullptr, 0};
     return spmm_run(p, val, d, 0, out, F, ldo, accumulate, row_div, (hipStream_t)stream);
+}
+
+extern "C" int sgnn_spmm_csr_f32_noalloc(sgnn_spmm_plan *p, const float *val, const float *x, float *out, int64_t F,
+                                         int64_t ldx, int64_t ldo, int accumulate, const float *row_div,
+                                         sgnn_stream_t stream) {
+    SGNN_REQUIRE(p != nullptr, "plan is null");
+    SGNN_REQUIRE(ldx >= F, "leading dimension smaller than F (ldx=%lld F=%lld)", (long long)ldx, (long long)F);
+    SGNN_REQUIRE(x != nullptr || p->nnz == 0 || p->M == 0, "x is null");
+    float *scratch = nullptr;
+    const int rc = scratch_for_current_device(&scratch);
+    if (rc != SGNN_OK) return rc;
+    DenseSrc d{x, ldx, nullptr, ParamBuf{nullptr, 0}, nullptr, nullptr, 0};
+    return spmm_run(p, val, d, 0, out, F, ldo, accumulate, row_div, (hipStream_t)stream, scratch, kScratchFloats);
 }
 
 static int spmm_dq_impl(sgnn_spmm_plan *p, const float *val, const uint8_t *q, const void *params, int params_bf16,
