@@ -42,7 +42,10 @@ def main():
 
     run_spmm("spmm_acc", 96, 64, 70, 6, 1, 0.25)       # accumulate branch, F with a masked tail tile
     run_spmm("spmm_acc128", 40, 40, 128, 17, 2, 0.0)   # F = 128 (two full 64-wide tiles)
-    run_spmm("spmm_ovw", 160, 160, 257, 0.0125, 3, 0.0, integer_init=True)  # sparsity <= 1e-4, F > 256: overwrite branch
+    # sparsity <= 1e-4 and F > 256: the overwrite branch, with a few dozen edges
+    run_spmm("spmm_ovw", 640, 640, 257, 0.06, 3, 0.0, integer_init=True)
+    nnz_ovw = out["spmm_ovw_col"].shape[0]
+    assert nnz_ovw >= 20 and orc.takes_overwrite_branch(nnz_ovw, 640, 640, 257), nnz_ovw
 
     for bits in (8, 4, 2):
         n, F = 23, 37  # 23 rows: a short last group for int4 (1 of 2) and int2 (3 of 4)

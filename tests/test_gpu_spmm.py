@@ -365,6 +365,27 @@ def test_steady_state_calls_replay_from_a_captured_graph():
         assert torch.equal(out, want) and torch.equal(out_q, want_q), f"replay {i}"
 
 
+@pytest.mark.parametrize("tag", ["spmm_acc", "spmm_acc128", "spmm_ovw"])
+def test_committed_reference_extension_vectors(tag):
+    # inputs and the outputs the reference's own x86 extension produced for them (tests/golden/make_ref_vectors.py);
+    # needs neither the reference checkout nor AVX-512 on the test host
+    import os
+    RV = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_vectors.npz"))
+    ops = _gpu()
+    rowptr, col, val, x, init, want = (RV[f"{tag}_{k}"] for k in ("rowptr", "col", "val", "x", "init", "out"))
+    M, F = init.shape
+    out = torch.from_numpy(init.copy())
+    # CPU tensors in, the reference's own dispatch rule decides accumulate / overwrite
+    ops.spmm(torch.from_numpy(rowptr), torch.from_numpy(col), torch.from_numpy(val), torch.from_numpy(x), out, M)
+    got = out.numpy()
+    if tag == "spmm_ovw":
+        assert ops.reference_overwrites(col.shape[0], M, x.shape[0], F)
+        np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-7)  # mul+add vs fma is build dependent in that branch
+        assert np.all(got[np.diff(rowptr) == 0] == 0)
+    else:
+        assert np.array_equal(got, want), "short rows: the reference's fma sequence, bit for bit"
+
+
 def test_full_size_graph_exact_on_small_integers():
     # The headline shape (2.45 M nodes, ~62 M edges, F = 128).  With small integer features and weights every
     # partial sum is an integer below 2^24, so fp32 addition is exact in any order and the product has ONE

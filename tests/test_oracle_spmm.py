@@ -132,3 +132,36 @@ def test_row_divide_is_true_division():
     orc.row_divide(out, np.array([3.0, 7.0], dtype=np.float32))
     assert np.array_equal(out, np.array([[np.float32(1) / np.float32(3), np.float32(2) / np.float32(3)],
                                          [np.float32(3) / np.float32(7), np.float32(5) / np.float32(7)]], dtype=np.float32))
+
+
+# ---- committed outputs of the reference's x86 extension (tests/golden/make_ref_vectors.py) ----------
+import os  # noqa: E402
+
+RV = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_vectors.npz"))
+
+
+@pytest.mark.parametrize("tag", ["spmm_acc", "spmm_acc128"])
+def test_accumulate_bit_exact_vs_committed_reference_vectors(tag):
+    # runs on any host: no AVX-512 and no reference checkout needed
+    rowptr, col, val, x = (RV[f"{tag}_{k}"] for k in ("rowptr", "col", "val", "x"))
+    out = RV[f"{tag}_init"].copy()
+    orc.spmm_accumulate(rowptr, col, val, x, out)
+    assert np.array_equal(out, RV[f"{tag}_out"])
+    assert not np.array_equal(out, RV[f"{tag}_init"])
+    deg = np.diff(rowptr)
+    assert np.array_equal(out[deg == 0], RV[f"{tag}_init"][deg == 0])
+
+
+def test_overwrite_branch_vs_committed_reference_vectors():
+    rowptr, col, val, x = (RV[f"spmm_ovw_{k}"] for k in ("rowptr", "col", "val", "x"))
+    M, K, F = rowptr.shape[0] - 1, x.shape[0], x.shape[1]
+    assert col.shape[0] >= 20 and orc.takes_overwrite_branch(col.shape[0], M, K, F)
+    want = RV["spmm_ovw_out"]
+    a = RV["spmm_ovw_init"].copy()
+    orc.spmm_dispatch(rowptr, col, val, x, a)          # the dispatch rule must pick the overwrite kernel
+    b = RV["spmm_ovw_init"].copy()
+    orc.spmm_overwrite(rowptr, col, val, x, b)
+    np.testing.assert_allclose(a, want, rtol=1e-6, atol=1e-7)
+    assert np.array_equal(a, b)
+    deg = np.diff(rowptr)
+    assert np.all(want[deg == 0] == 0) and np.any(want[deg > 0] != 0)   # old contents discarded, empty rows zeroed
