@@ -76,6 +76,19 @@ int sgnn_spmm_plan_destroy(sgnn_spmm_plan *plan);
  * it was not measured). */
 int sgnn_spmm_plan_info(const sgnn_spmm_plan *plan, int64_t info[10]);
 
+/* Which schedule sgnn_spmm_csr_f32 takes for a dense operand of F contiguous, 16-byte aligned fp32 columns:
+ * info[0] = 1 for the band schedule, 0 for the row-class schedule above.  The band schedule is for
+ * dense-degree matrices whose dense operand does not fit the L2 caches (e.g. 233 k nodes with ~490 edges
+ * per row at F = 602): the column space is cut into bands of info[1] columns (info[2] bands), the product
+ * is one launch per band accumulating onto out, and inside a launch the eight XCDs split the feature axis
+ * into info[3] slices so that each L2 holds one band of one slice and every repeated gather hits it.  It
+ * needs column-sorted rows (checked on first use; unsorted matrices keep the row-class schedule) and is
+ * built on the first call that wants it.  A row's edges are summed in CSR order with one fma per edge
+ * starting from the old out value, so its results are bit-identical to the reference's for every row
+ * length.  Replaces the per-64-column re-walk of the edge list in the reference's kernel
+ * (super_gnn/ops/csrc/spmm.cpp:502-510). */
+int sgnn_spmm_plan_schedule(const sgnn_spmm_plan *plan, int64_t F, int64_t info[4]);
+
 /* Optional: declare an edge-value array constant until the next bind.  The plan keeps a copy of the
  * long rows' values in its own (regrouped) edge order, and later sgnn_spmm_csr_f32 /
  * sgnn_spmm_csr_dq*_f32 calls that pass the SAME pointer read that copy contiguously instead of

@@ -20,6 +20,7 @@ SIGNATURES = {
     "sgnn_spmm_plan_create": (_int, [_vp, _vp, _int, _i64, _i64, _i64, _int, _int, _vp, ctypes.POINTER(_vp)]),
     "sgnn_spmm_plan_destroy": (_int, [_vp]),
     "sgnn_spmm_plan_info": (_int, [_vp, ctypes.POINTER(_i64)]),
+    "sgnn_spmm_plan_schedule": (_int, [_vp, _i64, ctypes.POINTER(_i64)]),
     "sgnn_spmm_csr_f32": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp, _vp]),
     "sgnn_spmm_csr_f32_noalloc": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _int, _vp, _vp]),
     "sgnn_spmm_reference_overwrites": (_int, [_i64, _i64, _i64, _i64]),

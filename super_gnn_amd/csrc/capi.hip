@@ -50,7 +50,7 @@ ProfScope::~ProfScope() {
 static const char *kKernelNames[K_COUNT] = {
     "spmm_short_kernel",  "spmm_piece_kernel", "spmm_long_final_kernel", "quant_pack_rows_kernel",
     "unpack_dequant_rows_kernel", "quant_v1_kernel", "dequant_v1_kernel", "stream_copy_kernel",
-    "spmm_short_kernel(dq)", "spmm_piece_kernel(dq)", "spmm_empty_rows_kernel"};
+    "spmm_short_kernel(dq)", "spmm_piece_kernel(dq)", "spmm_empty_rows_kernel", "spmm_band_kernel", "band_restage_kernel"};
 
 // ---- plain streaming copy: the attainable-bandwidth yardstick and the counter calibration -----
 __global__ __launch_bounds__(256) void stream_copy_kernel(const float4 *__restrict__ src, float4 *__restrict__ dst,

@@ -42,6 +42,8 @@ enum KernelId {
     K_FUSED_SHORT,
     K_FUSED_PIECE,
     K_SPMM_EMPTY_ROWS,
+    K_SPMM_BAND,
+    K_SPMM_BAND_RESTAGE,
     K_COUNT
 };
 

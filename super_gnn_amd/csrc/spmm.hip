@@ -24,6 +24,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <functional>
+#include <memory>
 #include <mutex>
 #include <vector>
 
@@ -190,29 +191,25 @@ __device__ __forceinline__ uint32_t group_ballot(bool pred) {
         return (uint32_t)m;  // only the low 32 lanes carry row flags
     } else {
         const int base = threadIdx.x & 63 & ~(G - 1);
-        return (uint32_t)(m >> base) & (G == 32 ? 0xffffffffu : ((1u << G) - 1u));
+        return (uint32_t)(m >> base) & (uint32_t)((1ull << G) - 1ull);
     }
 }
 
 // Rows per chunk: each of the first nr+1 lanes of the group holds one rowptr entry.
 __host__ __device__ constexpr int chunk_row_limit(int G) { return (G < 32 ? G : 32) - 1; }
 
-template <int VEC, int G, int NV, int BITS>
-__global__ __launch_bounds__(kBlock) void spmm_short_kernel(
-    const int64_t *__restrict__ rowptr, const int32_t *__restrict__ col, const float *__restrict__ val,
-    const DenseSrc dense, float *__restrict__ out, const int4 *__restrict__ chunks, int n_chunks, int F,
-    int64_t ldo, int accumulate, const float *__restrict__ row_div, uint32_t nblocks) {
-    constexpr int GPB = kBlock / G;
+// One lane group walks one chunk of consecutive rows for the feature columns [f_lo, f_hi) (both multiples
+// of VEC).  RP is the row-pointer type: the caller's int64 array, or the 32-bit per-band row pointers of a
+// band schedule.
+template <int VEC, int G, int NV, int BITS, typename RP, int UF = 0>
+__device__ __forceinline__ void short_chunk_body(
+    const RP *__restrict__ rowptr, const int32_t *__restrict__ col, const float *__restrict__ val,
+    const DenseSrc &dense, float *__restrict__ out, int4 ch, int f_lo, int f_hi,
+    int64_t ldo, int accumulate, const float *__restrict__ row_div, int lig) {
     constexpr int TILE = G * VEC * NV;
     // gathers in flight per lane group: 6 keeps the kernel at 75 VGPRs (6 waves per SIMD); 8 costs 83 (5 waves)
-    constexpr int U = NV == 1 ? 6 : unroll_of(NV);
-    const uint32_t lb = xcd_contiguous_block(blockIdx.x, nblocks);
-    const int gid = threadIdx.x / G, lig = threadIdx.x % G;
-    const int ci = (int)lb * GPB + gid;
-    if (ci >= n_chunks) return;
-    // A chunk record is (first row, row count, first edge, edge count): the column/weight loads
-    // depend on it alone and are issued before the row pointers come back.
-    int4 ch = chunks[ci];
+    constexpr int U = UF > 0 ? UF : NV == 1 ? 6 : unroll_of(NV);
+    const int F = f_hi;
     if constexpr (G == 64) {
         ch.x = __builtin_amdgcn_readfirstlane(ch.x);
         ch.y = __builtin_amdgcn_readfirstlane(ch.y);
@@ -240,7 +237,7 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
     const uint32_t mask = group_ballot<G>(lig < nr && rel_next > rel);  // bit i: row rb+i has edges
     const float mydiv = (row_div && lig < nr) ? row_div[rb + lig] : 1.0f;
 
-    for (int f0 = 0; f0 < F; f0 += TILE) {
+    for (int f0 = f_lo; f0 < F; f0 += TILE) {
         int off[NV];
         bool act[NV];
         float acc[NV][VEC], nxt_old[NV][VEC];
@@ -268,7 +265,7 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
 
         int nc = nc0, ns = ns0;
         float nw = nw0;
-        if (f0 > 0 && lig < E) {  // a later feature tile walks the chunk's edges again
+        if (f0 > f_lo && lig < E) {  // a later feature tile walks the chunk's edges again
             nc = __builtin_nontemporal_load(colp + lig);
             if (valp) nw = __builtin_nontemporal_load(valp + lig);
             if constexpr ((BITS & kEdgeSlots) != 0) ns = __builtin_nontemporal_load(slotp + lig);
@@ -337,6 +334,325 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
             vec_store_nt<VEC>(out + (int64_t)(rb + cur) * ldo + off[v], acc[v]);
         }
     }
+}
+
+template <int VEC, int G, int NV, int BITS>
+__global__ __launch_bounds__(kBlock) void spmm_short_kernel(
+    const int64_t *__restrict__ rowptr, const int32_t *__restrict__ col, const float *__restrict__ val,
+    const DenseSrc dense, float *__restrict__ out, const int4 *__restrict__ chunks, int n_chunks, int F,
+    int64_t ldo, int accumulate, const float *__restrict__ row_div, uint32_t nblocks) {
+    constexpr int GPB = kBlock / G;
+    const uint32_t lb = xcd_contiguous_block(blockIdx.x, nblocks);
+    const int gid = threadIdx.x / G, lig = threadIdx.x % G;
+    const int ci = (int)lb * GPB + gid;
+    if (ci >= n_chunks) return;
+    // A chunk record is (first row, row count, first edge, edge count): the column/weight loads
+    // depend on it alone and are issued before the row pointers come back.
+    short_chunk_body<VEC, G, NV, BITS, int64_t>(rowptr, col, val, dense, out, chunks[ci], 0, F, ldo, accumulate, row_div, lig);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Band schedule (dense-degree matrices whose dense operand does not fit the L2 caches).
+//
+// The column space is cut into bands of band_cols columns; band b of the matrix is a CSR matrix of its
+// own (32-bit row pointers, edges stored band-major), and the product is a sequence of launches, one per
+// band, each accumulating its band's contribution onto `out` in place.  Inside one launch the eight XCDs
+// split the FEATURE axis: workgroup i runs on XCD i % 8 and only touches feature slice (i % 8) % n_slices,
+// so an XCD's L2 has to hold band_cols x (slice bytes) of the dense operand -- sized to fit -- and every
+// gather after the first touch of a dense row slice is an L2 hit.  All workgroups of a launch work on the
+// same band (the kernel boundary is the synchronisation), the accumulators travel through `out` between
+// bands (read-modify-write of one row slice per band, a stream), and a row's edges are still summed in CSR
+// order with one fma per edge starting from the old value: with column-sorted rows the result is the
+// reference's, bit for bit, whatever the row length.
+// ------------------------------------------------------------------------------------------------
+// Rows per chunk and staged (row offset, val) pairs per chunk of the band kernel.
+#ifndef SGNN_BAND_ROWS
+#define SGNN_BAND_ROWS 10
+#endif
+#ifndef SGNN_BAND_EDGES
+#define SGNN_BAND_EDGES 128
+#endif
+#ifndef SGNN_BAND_U
+#define SGNN_BAND_U 12
+#endif
+constexpr int kBandRows = SGNN_BAND_ROWS;
+constexpr int kBandEdges = SGNN_BAND_EDGES;
+constexpr int kBandWindow = SGNN_BAND_U;  // gathers in flight per lane group
+constexpr int kBandPad = 16;              // staging entries past the last pair (>= the gather window)
+static_assert(kBandWindow <= kBandPad, "gather window wider than the staging pad");
+__host__ __device__ constexpr int band_group_floats(int tile_stride) { return kBandRows * tile_stride + 2 * (kBandEdges + kBandPad); }
+
+// The dense operand restaged for the band kernel: xs[slice][column][slice_pad floats], slice_pad a multiple of
+// 16 floats.  Every row of a slice then starts on a 64-byte boundary, a group of slice_pad / 4 lanes reads it
+// with aligned 128-bit loads, and four neighbouring lanes cover exactly one 64-byte sector.  That matters
+// because the L1 looks up one sector per cycle: gathered straight out of rows of 602 floats (2408 bytes, only
+// 8-byte aligned) a wave instruction of three 304-byte slices touched 23 sectors and held the address path for
+// 36 cycles; restaged it touches 15.  One pass over X per product (about 2 % of the product's time).
+// Floats past the end of a slice or of the row are zero.
+__global__ __launch_bounds__(kBlock) void band_restage_kernel(const float *__restrict__ x, int64_t ldx, float *__restrict__ xs,
+                                                               int64_t K, int F, int slice_floats, int slice_pad, int n_slices) {
+    const int vpr = slice_pad / 4;  // float4 per restaged row
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= (int64_t)n_slices * K * vpr) return;
+    const int v = (int)(i % vpr);
+    const int64_t sc = i / vpr;
+    const int64_t c = sc % K;
+    const int sl = (int)(sc / K);
+    const int f0 = sl * slice_floats + 4 * v;
+    const float *row = x + c * ldx;
+    float r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = (4 * v + e < slice_floats && f0 + e < F) ? row[f0 + e] : 0.0f;
+    reinterpret_cast<float4 *>(xs)[i] = make_float4(r[0], r[1], r[2], r[3]);
+}
+
+// Old / new values of `out` for one lane: nf (0..4) floats at p.  EVEN: rows start on 8-byte boundaries and F is
+// even, so nf is 4 or 2 and 128-bit accesses that need only 8-byte alignment are used (a lane with two floats
+// loads the four floats that END at p + 2 and keeps the upper two, so no access crosses the end of its row).
+template <bool EVEN>
+__device__ __forceinline__ void out_load(float (&r)[4], const float *p, int nf) {
+    if constexpr (EVEN) {
+        typedef float f4 __attribute__((ext_vector_type(4), aligned(8)));
+        const bool half = nf == 2;
+        const f4 v = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(p - (half ? 2 : 0)));
+        r[0] = half ? v.z : v.x;
+        r[1] = half ? v.w : v.y;
+        r[2] = v.z;
+        r[3] = v.w;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = e < nf ? __builtin_nontemporal_load(p + e) : 0.0f;
+    }
+}
+template <bool EVEN>
+__device__ __forceinline__ void out_store(float *p, const float (&r)[4], int nf) {
+    if constexpr (EVEN) {
+        typedef float f4 __attribute__((ext_vector_type(4), aligned(8)));
+        typedef float f2 __attribute__((ext_vector_type(2), aligned(8)));
+        if (nf == 2) {
+            f2 v = {r[0], r[1]};
+            __builtin_nontemporal_store(v, reinterpret_cast<f2 *>(p));
+        } else {
+            f4 v = {r[0], r[1], r[2], r[3]};
+            __builtin_nontemporal_store(v, reinterpret_cast<f4 *>(p));
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (e < nf) __builtin_nontemporal_store(r[e], p + e);
+    }
+}
+
+// One lane group per chunk of consecutive rows (at most kBandRows rows and kBandEdges edges).  A group is
+// G = slice_pad / 4 lanes (any value from 16 to 64, not only powers of two), one float4 of the restaged slice
+// each, and a wavefront carries 64 / G groups: a vector memory instruction occupies a CU's address path for as
+// long whether 20 or 64 of its lanes are active, so what a gather costs is decided by how many gathers share one
+// instruction.  At F = 602 a slice is 76 floats padded to 80, G = 20, and three gathers travel together.
+// Three phases per chunk:
+//   1. everything that comes from HBM is requested at once: the old `out` values of all the chunk's rows for
+//      this feature slice go to LDS (the output tile of the chunk), and so do its (row offset, val) pairs;
+//   2. the gather loop: a rolling window of kBandWindow gathers of dense-row slices, all of them L2 hits, one fma
+//      per edge in CSR order; a row boundary swaps the accumulator through the LDS tile.  Nothing slow sits in
+//      the vector memory queue during this phase: loads return in order, and one HBM-latency load between two
+//      gathers would stall every gather behind it;
+//   3. the tile rows that received edges are written back.
+// A tile column belongs to one lane and a group to one wavefront: the kernel has no workgroup barrier.
+template <bool EVEN, bool OFF32>
+__global__ __launch_bounds__(kBlock) void spmm_band_kernel(
+    const int32_t *__restrict__ rowptr_b, const int32_t *__restrict__ col_bm, const float *__restrict__ val_bm,
+    const float *__restrict__ xs, int64_t K, float *__restrict__ out, const int4 *__restrict__ chunks, int n_chunks, int F,
+    int64_t ldo, int slice_floats, int slice_pad, int n_slices, int G) {
+    extern __shared__ float band_lds[];
+    constexpr int U = kBandWindow;
+    const int tile_stride = G * 4;
+    const int gpw = 64 / G;                       // groups per wavefront
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int gsub = lane / G, lig = lane - gsub * G;
+    const int gbase = gsub * G;                   // first lane of this group inside the wavefront
+    const int gid = wave * gpw + gsub;            // group inside the workgroup
+    const int xcd = blockIdx.x % kNumXCD;
+    const int slice = xcd % n_slices, rg = xcd / n_slices, n_rg = kNumXCD / n_slices;
+    const int ci = ((int)(blockIdx.x / kNumXCD) * n_rg + rg) * ((kBlock / 64) * gpw) + gid;
+    const int f_lo = slice * slice_floats;        // first feature column of this slice
+    const int vpr = slice_pad / 4;                // float4 per restaged row
+    const bool valid = gsub < gpw && ci < n_chunks && f_lo < F;
+    float *tile = band_lds + (size_t)(gsub < gpw ? gid : 0) * band_group_floats(tile_stride);
+    int *lkey = reinterpret_cast<int *>(tile + kBandRows * tile_stride);
+    float *lval = reinterpret_cast<float *>(lkey + kBandEdges + kBandPad);
+    const float *xslice = xs + (int64_t)slice * K * slice_pad;
+
+    int4 ch = make_int4(0, 0, 0, 0);
+    if (valid) ch = chunks[ci];
+    const int rb = ch.x, nr = ch.y, E = ch.w;  // rows rb .. rb+nr-1 (first and last non-empty in this band), E edges
+    const int64_t B = ch.z;
+    const int32_t *colp = col_bm + B;
+    const float *valp = val_bm ? val_bm + B : nullptr;
+    // Lane i of the group holds rowptr[rb+i] relative to the chunk's first edge (lanes >= nr hold the end).
+    int rel = 0;
+    if (valid) rel = (int)(rowptr_b[rb + (lig < nr ? lig : nr)] - B);
+    const int rel_next = __shfl(rel, lane + 1 < 64 ? lane + 1 : 63);
+    const unsigned long long bal = __ballot(valid && lig < nr && rel_next > rel);
+    const uint32_t mask = (uint32_t)(bal >> gbase) & ((1u << kBandRows) - 1u);  // bit i: row rb+i has edges in this band
+
+    for (int t0 = 0; t0 < vpr; t0 += G) {             // slices wider than 64 float4 are walked in tiles
+        const int vi = t0 + lig;                      // this lane's float4 of the slice
+        const int off = f_lo + 4 * vi;                // its first feature column
+        int nf = slice_floats - 4 * vi < F - off ? slice_floats - 4 * vi : F - off;
+        nf = !valid || vi >= vpr || nf < 0 ? 0 : nf > 4 ? 4 : nf;  // floats of `out` this lane owns (EVEN: 0, 2 or 4)
+        const bool act = nf > 0;
+        // This lane's column of the tile.  Lanes that own nothing point at column 0 and never write (a write
+        // through "their" offset would land in the next row or in the staged pairs).
+        float *tcol = tile + (act ? lig * 4 : 0);
+        // ---- phase 1: old out values of the chunk's rows -> LDS tile -------------------------------------
+        if (act) {
+            for (int r0 = 0; r0 < nr; r0 += 6) {
+                float old[6][4];
+#pragma unroll
+                for (int k = 0; k < 6; ++k) {
+                    const int r = r0 + k < nr ? r0 + k : nr - 1;
+                    out_load<EVEN>(old[k], out + (int64_t)(rb + r) * ldo + off, nf);
+                }
+#pragma unroll
+                for (int k = 0; k < 6; ++k) {
+                    if (r0 + k < nr) *reinterpret_cast<float4 *>(tcol + (r0 + k) * tile_stride) = make_float4(old[k][0], old[k][1], old[k][2], old[k][3]);
+                }
+            }
+        }
+        // ---- phase 2: gathers ------------------------------------------------------------------------------
+        if (valid) {
+            // every lane of the group loads: the restaged rows are padded, so a lane that owns nothing reads zeros
+            const float *xlane = xslice + 4 * (vi < vpr ? vi : t0);
+            int cur = __builtin_ctz(mask);
+            int cur_end = __shfl(rel, gbase + cur + 1);
+            float4 acc = *reinterpret_cast<const float4 *>(tcol + cur * tile_stride);
+            // The chunk's (row offset, val) pairs are staged in LDS, kBandEdges at a time (more than one round only
+            // for a row longer than that).  A group lives inside one wavefront, whose LDS operations execute in
+            // order: a wavefront-level fence is all the staging needs.
+            for (int seg = 0; seg < E; seg += kBandEdges) {
+                const int se = E - seg < kBandEdges ? E - seg : kBandEdges;
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                // four pairs per lane and load (these are the only loads of the gather phase that miss the L2, and a
+                // miss delays every gather queued behind it); U entries of padding repeat the last pair, so the
+                // window below never clamps an index
+                for (int i = 4 * lig; i < se + U; i += 4 * G) {
+                    int c[4];
+                    float w[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+                    if (i + 4 <= se) {
+                        typedef int i4 __attribute__((ext_vector_type(4), aligned(4)));
+                        typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
+                        const i4 cv = __builtin_nontemporal_load(reinterpret_cast<const i4 *>(colp + seg + i));
+                        c[0] = cv.x; c[1] = cv.y; c[2] = cv.z; c[3] = cv.w;
+                        if (valp) {
+                            const f4 wv4 = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(valp + seg + i));
+                            w[0] = wv4.x; w[1] = wv4.y; w[2] = wv4.z; w[3] = wv4.w;
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int k = i + e < se ? i + e : se - 1;
+                            c[e] = __builtin_nontemporal_load(colp + seg + k);
+                            if (valp) w[e] = __builtin_nontemporal_load(valp + seg + k);
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (i + e < se + U) {
+                            lkey[i + e] = OFF32 ? (int)((uint32_t)c[e] * (uint32_t)slice_pad * 4u) : c[e];
+                            lval[i + e] = w[e];
+                        }
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                // A rolling window of U gathers: slot u is refilled with the edge U further on as soon as its value
+                // has been consumed, so U - 1 gathers are in flight at all times (loads return in order).
+                float4 xv[U];
+                float wv[U];
+                auto gather = [&](int u, int key) {
+                    const float *p;
+                    if constexpr (OFF32) p = reinterpret_cast<const float *>(reinterpret_cast<const char *>(xlane) + (uint32_t)key);
+                    else p = xlane + (int64_t)key * slice_pad;
+                    xv[u] = *reinterpret_cast<const float4 *>(p);
+                };
+                auto consume = [&](int edge, int u) {
+                    if (edge == cur_end) {  // first edge of the next non-empty row: swap accumulators through the tile
+                        if (act) *reinterpret_cast<float4 *>(tcol + cur * tile_stride) = acc;
+                        const uint32_t rest = mask & ~((2u << cur) - 1u);
+                        cur = __builtin_ctz(rest);
+                        cur_end = __shfl(rel, gbase + cur + 1);
+                        acc = *reinterpret_cast<const float4 *>(tcol + cur * tile_stride);
+                    }
+                    acc.x = fmaf(wv[u], xv[u].x, acc.x);
+                    acc.y = fmaf(wv[u], xv[u].y, acc.y);
+                    acc.z = fmaf(wv[u], xv[u].z, acc.z);
+                    acc.w = fmaf(wv[u], xv[u].w, acc.w);
+                };
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    wv[u] = lval[u];
+                    gather(u, lkey[u]);
+                }
+                int base = 0;
+                // full rounds: every slot holds a real edge and is refilled unconditionally (no branch around a load:
+                // the compiler then counts outstanding loads exactly instead of draining the queue at every join)
+                for (; base + U < se; base += U) {
+                    const int *lk = lkey + base + U;
+                    const float *lv = lval + base + U;
+                    int kn[U];
+                    float wn[U];
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {  // the next round's pairs, read from LDS ahead of their use
+                        kn[u] = lk[u];
+                        wn[u] = lv[u];
+                    }
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        consume(seg + base + u, u);
+                        wv[u] = wn[u];
+                        gather(u, kn[u]);
+                    }
+                }
+                // last round: the window drains
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    if (base + u < se) consume(seg + base + u, u);
+                }
+            }
+            if (act) *reinterpret_cast<float4 *>(tcol + cur * tile_stride) = acc;
+        }
+        // ---- phase 3: rows that received edges go back to out ---------------------------------------------
+        if (act) {
+            uint32_t m = mask;
+            while (m) {
+                const int r = __builtin_ctz(m);
+                m &= m - 1;
+                const float4 t = *reinterpret_cast<const float4 *>(tcol + r * tile_stride);
+                const float v[4] = {t.x, t.y, t.z, t.w};
+                out_store<EVEN>(out + (int64_t)(rb + r) * ldo + off, v, nf);
+            }
+        }
+    }
+}
+
+// out[r, 0..F) = 0 (overwrite mode of the band schedule) or out[r, :] /= row_div[r] (mean epilogue), for all rows.
+template <int VEC, bool DIV>
+__global__ __launch_bounds__(kBlock) void rows_fill_or_divide_kernel(float *__restrict__ out, int64_t M, int F, int64_t ldo,
+                                                                     const float *__restrict__ row_div) {
+    const int nvec = F / VEC;
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= M * nvec) return;
+    const int64_t r = i / nvec;
+    float *p = out + r * ldo + (i - r * nvec) * VEC;
+    float a[VEC];
+    if constexpr (DIV) {
+        vec_load_nt<VEC>(a, p);
+        const float d = row_div[r];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) a[k] = a[k] / d;
+    } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) a[k] = 0.0f;
+    }
+    vec_store_nt<VEC>(p, a);
 }
 
 // Rows without edges, only needed when they must be written: overwrite mode (zeros) or the mean
@@ -596,6 +912,68 @@ __global__ __launch_bounds__(kBlock) void permute_values_kernel(const float *__r
 }
 
 // ------------------------------------------------------------------------------------------------
+// Band schedule, plan-time kernels.
+// ------------------------------------------------------------------------------------------------
+// flag = 1 if some row's columns are not in non-decreasing order (16 lanes per row).
+__global__ __launch_bounds__(kBlock) void check_rows_sorted_kernel(const int64_t *__restrict__ rowptr,
+                                                                   const int32_t *__restrict__ col, int64_t M,
+                                                                   int *__restrict__ flag) {
+    const int64_t r = (int64_t)blockIdx.x * (kBlock / 16) + threadIdx.x / 16;
+    if (r >= M) return;
+    const int64_t b = rowptr[r], e = rowptr[r + 1];
+    bool bad = false;
+    for (int64_t i = b + (threadIdx.x % 16); i + 1 < e; i += 16) bad |= col[i] > col[i + 1];
+    if (bad) atomicOr(flag, 1);
+}
+
+// lo[r, b] = index of row r's first edge whose column is >= b * band_cols (b = 0 .. n_bands), and the
+// per-band edge counts transposed, cnt_t[b, r] = lo[r, b+1] - lo[r, b].  Rows are column-sorted.
+__global__ __launch_bounds__(kBlock) void band_bounds_kernel(const int64_t *__restrict__ rowptr,
+                                                             const int32_t *__restrict__ col, int64_t M, int n_bands,
+                                                             int band_cols, int32_t *__restrict__ lo) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= M * (n_bands + 1)) return;
+    const int64_t r = i / (n_bands + 1);
+    const int b = (int)(i - r * (n_bands + 1));
+    int64_t a = rowptr[r], z = rowptr[r + 1];
+    if (b == n_bands) a = z;
+    else if (b > 0) {
+        const int64_t key = (int64_t)b * band_cols;
+        while (a < z) {
+            const int64_t mid = (a + z) >> 1;
+            if (col[mid] < key) a = mid + 1; else z = mid;
+        }
+    }
+    lo[i] = (int32_t)a;
+}
+__global__ __launch_bounds__(kBlock) void band_counts_kernel(const int32_t *__restrict__ lo, int64_t M, int n_bands,
+                                                             int32_t *__restrict__ cnt_t) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= M * n_bands) return;
+    const int b = (int)(i / M);
+    const int64_t r = i - (int64_t)b * M;
+    cnt_t[i] = lo[r * (n_bands + 1) + b + 1] - lo[r * (n_bands + 1) + b];
+}
+
+// Copies the edges into band-major order: band b's edges of row r go to rowptr_bm[b, r] ... in CSR order.
+__global__ __launch_bounds__(kBlock) void band_scatter_kernel(const int64_t *__restrict__ rowptr,
+                                                              const int32_t *__restrict__ col, int64_t M, int n_bands,
+                                                              int band_cols, const int32_t *__restrict__ lo,
+                                                              const int32_t *__restrict__ rowptr_bm,
+                                                              int32_t *__restrict__ col_bm, int32_t *__restrict__ eperm_bm) {
+    const int64_t r = (int64_t)blockIdx.x * (kBlock / 16) + threadIdx.x / 16;
+    if (r >= M) return;
+    const int64_t b0 = rowptr[r], e0 = rowptr[r + 1];
+    for (int64_t i = b0 + (threadIdx.x % 16); i < e0; i += 16) {
+        const int32_t c = col[i];
+        const int b = c / band_cols;
+        const int64_t dst = (int64_t)rowptr_bm[(int64_t)b * (M + 1) + r] + (i - lo[r * (n_bands + 1) + b]);
+        col_bm[dst] = c;
+        eperm_bm[dst] = (int32_t)i;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Launch tables.
 // ------------------------------------------------------------------------------------------------
 struct ShortArgs {
@@ -728,6 +1106,23 @@ static int scratch_for_current_device(float **out) {
     return SGNN_OK;
 }
 
+// The matrix cut into column bands, each band a CSR matrix of its own (see spmm_band_kernel).
+struct BandSchedule {
+    int band_cols = 0, n_bands = 0;
+    int32_t *rowptr_bm = nullptr;      // [n_bands * (M+1)] absolute offsets into col_bm / val_bm
+    int32_t *col_bm = nullptr;         // [nnz] columns, band-major
+    int32_t *eperm_bm = nullptr;       // [nnz] CSR index of each band-major edge
+    float *val_bm = nullptr;           // [nnz] edge values in band-major order
+    uint64_t val_gen = 0;              // plan bind generation val_bm was filled under (0 = not from a bound array)
+    int64_t M = 0, K = 0;
+    int4 *chunks = nullptr;            // all bands' chunks, band after band: (first row, rows, first edge, edges)
+    std::vector<int64_t> chunk_off;    // [n_bands + 1] each band's range in chunks
+    ~BandSchedule() {
+        (void)hipFree(rowptr_bm); (void)hipFree(col_bm); (void)hipFree(eperm_bm); (void)hipFree(val_bm);
+        (void)hipFree(chunks);
+    }
+};
+
 struct sgnn_spmm_plan {
     int device = 0;
     int64_t M = 0, K = 0, nnz = 0;
@@ -756,7 +1151,13 @@ struct sgnn_spmm_plan {
     // rows without edges
     int32_t *empty_rows = nullptr;
     int64_t n_empty = 0;
-    // Short-row chunks, one list per chunk row limit (7, 15, 31), built on first use.
+    // Band schedules (dense-degree matrices), built on first use for a band width.
+    int cols_sorted = -1;           // -1 unknown, 0 some row's columns are out of order, 1 every row is column-sorted
+    uint64_t bind_gen = 1;          // bumped by every sgnn_spmm_plan_bind_values
+    std::vector<BandSchedule *> bands;
+    float *band_xs = nullptr;       // the dense operand restaged slice by slice (see band_restage_kernel), grown on demand
+    size_t band_xs_floats = 0;
+    // Short-row chunks, one list per chunk row limit (7, 15, 31).
     std::vector<int64_t> h_rowptr;
     int4 *chunks[3] = {nullptr, nullptr, nullptr};
     int64_t n_chunks[3] = {-1, -1, -1};
@@ -819,6 +1220,8 @@ extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     (void)hipFree(p->partial);
     (void)hipFree(p->empty_rows);
     for (int i = 0; i < 3; ++i) (void)hipFree(p->chunks[i]);
+    for (BandSchedule *b : p->bands) delete b;
+    (void)hipFree(p->band_xs);
     delete p;
     return SGNN_OK;
 }
@@ -1035,6 +1438,257 @@ extern "C" int sgnn_spmm_reference_overwrites(int64_t nnz, int64_t M, int64_t K,
     return (sparsity <= 0.0001f && F > 256) ? 1 : 0;
 }
 
+// ------------------------------------------------------------------------------------------------
+// Band schedule, host side.
+// ------------------------------------------------------------------------------------------------
+constexpr int kBandL2BudgetKB = 4096;   // per-XCD bytes of the restaged dense operand in one band: the whole 4 MB L2 measured best (the other streams pass through)
+constexpr double kBandMinRowEdges = 6;  // average edges per row and band below which the per-band read-modify-write of out dominates
+constexpr int64_t kBandMinDenseBytes = (int64_t)48 << 20;  // a dense operand this small lives in the L2s anyway
+
+struct BandShape {
+    bool even;         // X-independent: out rows on 8-byte boundaries, F even and >= 4 (128-bit accesses to out)
+    int n_slices;      // feature slices = XCDs that split the feature axis (8, 4, 2 or 1)
+    int slice_floats;  // feature columns per slice (a multiple of 4)
+    int slice_pad;     // floats per restaged slice row (a multiple of 16: rows on 64-byte boundaries)
+    int G;             // lanes per group: slice_pad / 4, at least 16, at most 64 (wider slices are walked in tiles)
+    int band_cols, n_bands;
+};
+
+// How a product of feature width F would be cut into feature slices and column bands.
+static BandShape band_shape(const sgnn_spmm_plan *p, int64_t F, bool even_out) {
+    BandShape b{};
+    b.even = even_out && F % 2 == 0 && F >= 4;
+    const int nvec = (int)((F + 3) / 4);
+    b.n_slices = kNumXCD;
+    while (b.n_slices > 1 && (nvec + b.n_slices - 1) / b.n_slices < 16) b.n_slices /= 2;
+    b.slice_floats = 4 * ((nvec + b.n_slices - 1) / b.n_slices);
+    b.slice_pad = (b.slice_floats + 15) / 16 * 16;
+    b.G = std::max(16, std::min(64, b.slice_pad / 4));
+    int cols = env_int("SGNN_SPMM_BAND_COLS", 0);
+    if (cols <= 0)
+        cols = (int)std::max<int64_t>(256, (int64_t)env_int("SGNN_SPMM_BAND_KB", kBandL2BudgetKB) * 1024 / (b.slice_pad * 4) / 256 * 256);
+    b.band_cols = cols;
+    b.n_bands = (int)std::max<int64_t>(1, (p->K + cols - 1) / cols);
+    return b;
+}
+
+// Whether the band schedule is the one to use: the dense operand does not fit the caches, and every row has
+// enough edges per band to pay for carrying its accumulator through `out` from band to band.
+static bool band_wanted(const sgnn_spmm_plan *p, int64_t F, const BandShape &b) {
+    const int mode = env_int("SGNN_SPMM_BAND", -1);
+    if (mode == 0 || p->nnz == 0 || p->M == 0) return false;
+    if (mode > 0) return true;
+    if (b.n_bands < 3 || p->K * F * 4 < kBandMinDenseBytes) return false;
+    return (double)p->nnz / (double)p->M / (double)b.n_bands >= kBandMinRowEdges;
+}
+
+static int band_rows_sorted(sgnn_spmm_plan *p, hipStream_t st, bool *sorted) {
+    if (p->cols_sorted < 0) {
+        DevTmp<int> flag;
+        SGNN_HIP_CHECK(hipMalloc(&flag.p, sizeof(int)));
+        SGNN_HIP_CHECK(hipMemsetAsync(flag.p, 0, sizeof(int), st));
+        hipLaunchKernelGGL(check_rows_sorted_kernel, dim3((uint32_t)((p->M + 15) / 16)), dim3(kBlock), 0, st, p->rowptr, p->col,
+                           p->M, flag.p);
+        SGNN_HIP_CHECK(hipGetLastError());
+        int h = 0;
+        SGNN_HIP_CHECK(hipMemcpyAsync(&h, flag.p, sizeof(int), hipMemcpyDeviceToHost, st));
+        SGNN_HIP_CHECK(hipStreamSynchronize(st));
+        p->cols_sorted = h ? 0 : 1;
+    }
+    *sorted = p->cols_sorted == 1;
+    return SGNN_OK;
+}
+
+// The chunk list of every band: consecutive rows, at most kBandRows rows and kBandEdges edges (one row may have
+// more), first and last row non-empty in the band.
+static int band_build_chunks(BandSchedule *bs, const std::vector<int32_t> &h_rowptr_bm, hipStream_t st) {
+    // a chunk's (col, val) pairs should fit the kernel's staging area; only a single row longer than that spills
+    int cap = env_int("SGNN_SPMM_BAND_CHUNK_EDGES", 0);
+    if (cap <= 0 || cap > kBandEdges) cap = kBandEdges;
+    const int64_t M = bs->M;
+    std::vector<int4> out;
+    bs->chunk_off.assign((size_t)bs->n_bands + 1, 0);
+    for (int b = 0; b < bs->n_bands; ++b) {
+        const int32_t *rp = h_rowptr_bm.data() + (size_t)b * (size_t)(M + 1);
+        int64_t m = 0;
+        while (m < M) {
+            if (rp[m + 1] == rp[m]) { ++m; continue; }
+            const int64_t start = m;
+            int64_t last = m, edges = 0;
+            while (m < M && m - start < kBandRows) {
+                const int64_t d = rp[m + 1] - rp[m];
+                if (m > start && edges + d > cap) break;
+                if (d > 0) last = m;
+                edges += d;
+                ++m;
+            }
+            out.push_back(make_int4((int)start, (int)(last - start + 1), rp[start], rp[last + 1] - rp[start]));
+        }
+        bs->chunk_off[(size_t)b + 1] = (int64_t)out.size();
+    }
+    if (!out.empty()) {
+        SGNN_HIP_CHECK(hipMalloc(&bs->chunks, sizeof(int4) * out.size()));
+        SGNN_HIP_CHECK(hipMemcpyAsync(bs->chunks, out.data(), sizeof(int4) * out.size(), hipMemcpyHostToDevice, st));
+        SGNN_HIP_CHECK(hipStreamSynchronize(st));
+    }
+    return SGNN_OK;
+}
+
+static int band_build(sgnn_spmm_plan *p, int band_cols, int n_bands, hipStream_t st, BandSchedule **out) {
+    const int64_t M = p->M, nnz = p->nnz;
+    std::unique_ptr<BandSchedule> bs(new BandSchedule());
+    bs->band_cols = band_cols;
+    bs->n_bands = n_bands;
+    bs->M = M;
+    bs->K = p->K;
+    SGNN_REQUIRE((int64_t)n_bands * (M + 1) < INT32_MAX && M * ((int64_t)n_bands + 1) < INT32_MAX * (int64_t)4,
+                 "band schedule too large (%d bands x %lld rows)", n_bands, (long long)M);
+    DevTmp<int32_t> lo, cnt_t;
+    const int64_t n_lo = M * ((int64_t)n_bands + 1), n_cnt = M * (int64_t)n_bands;
+    SGNN_HIP_CHECK(hipMalloc(&lo.p, sizeof(int32_t) * (size_t)n_lo));
+    SGNN_HIP_CHECK(hipMalloc(&cnt_t.p, sizeof(int32_t) * (size_t)n_cnt));
+    hipLaunchKernelGGL(band_bounds_kernel, dim3((uint32_t)((n_lo + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, p->rowptr, p->col, M,
+                       n_bands, band_cols, lo.p);
+    hipLaunchKernelGGL(band_counts_kernel, dim3((uint32_t)((n_cnt + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, lo.p, M, n_bands,
+                       cnt_t.p);
+    SGNN_HIP_CHECK(hipGetLastError());
+    std::vector<int32_t> h_cnt((size_t)n_cnt);
+    SGNN_HIP_CHECK(hipMemcpyAsync(h_cnt.data(), cnt_t.p, sizeof(int32_t) * h_cnt.size(), hipMemcpyDeviceToHost, st));
+    SGNN_HIP_CHECK(hipStreamSynchronize(st));
+    std::vector<int32_t> rp((size_t)n_bands * (size_t)(M + 1));
+    int64_t run = 0;
+    for (int b = 0; b < n_bands; ++b) {
+        int32_t *row = rp.data() + (size_t)b * (size_t)(M + 1);
+        const int32_t *c = h_cnt.data() + (size_t)b * (size_t)M;
+        for (int64_t r = 0; r < M; ++r) {
+            row[r] = (int32_t)run;
+            run += c[r];
+        }
+        row[M] = (int32_t)run;
+    }
+    if (run != nnz) return fail(SGNN_ERR_RANGE, "band schedule: %lld of %lld edges fall into the bands", (long long)run, (long long)nnz);
+    SGNN_HIP_CHECK(hipMalloc(&bs->rowptr_bm, sizeof(int32_t) * rp.size()));
+    SGNN_HIP_CHECK(hipMemcpyAsync(bs->rowptr_bm, rp.data(), sizeof(int32_t) * rp.size(), hipMemcpyHostToDevice, st));
+    SGNN_HIP_CHECK(hipMalloc(&bs->col_bm, sizeof(int32_t) * (size_t)nnz));
+    SGNN_HIP_CHECK(hipMalloc(&bs->eperm_bm, sizeof(int32_t) * (size_t)nnz));
+    SGNN_HIP_CHECK(hipMalloc(&bs->val_bm, sizeof(float) * (size_t)nnz));
+    hipLaunchKernelGGL(band_scatter_kernel, dim3((uint32_t)((M + 15) / 16)), dim3(kBlock), 0, st, p->rowptr, p->col, M, n_bands,
+                       band_cols, lo.p, bs->rowptr_bm, bs->col_bm, bs->eperm_bm);
+    SGNN_HIP_CHECK(hipGetLastError());
+    SGNN_HIP_CHECK(hipStreamSynchronize(st));
+    const int rc = band_build_chunks(bs.get(), rp, st);
+    if (rc != SGNN_OK) return rc;
+    *out = bs.release();
+    return SGNN_OK;
+}
+
+template <bool EVEN>
+static int launch_band(const BandSchedule *bs, const BandShape &sh, int b, const float *val_bm, const float *xs, float *out,
+                       int F, int64_t ldo, hipStream_t st) {
+    const int64_t c0 = bs->chunk_off[(size_t)b], c1 = bs->chunk_off[(size_t)b + 1];
+    if (c1 == c0) return SGNN_OK;
+    const int gpb = (kBlock / 64) * (64 / sh.G);  // lane groups per workgroup
+    const int n_rg = kNumXCD / sh.n_slices;
+    const int64_t wgs = (c1 - c0 + gpb - 1) / gpb;
+    const uint32_t nb = (uint32_t)((wgs + n_rg - 1) / n_rg) * kNumXCD;
+    const size_t lds = sizeof(float) * (size_t)gpb * (size_t)band_group_floats(sh.G * 4);
+    // every restaged row of a slice within 4 GB of the slice's start: 32-bit gather offsets
+    const bool off32 = (uint64_t)bs->K * (uint64_t)sh.slice_pad * 4u < ((uint64_t)1 << 32);
+    auto kernel = off32 ? spmm_band_kernel<EVEN, true> : spmm_band_kernel<EVEN, false>;
+    static size_t lds_allowed[2] = {48 * 1024, 48 * 1024};  // per instantiation
+    if (lds > lds_allowed[off32]) {
+        SGNN_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        lds_allowed[off32] = lds;
+    }
+    hipLaunchKernelGGL(kernel, dim3(nb), dim3(kBlock), lds, st, bs->rowptr_bm + (size_t)b * (size_t)(bs->M + 1), bs->col_bm, val_bm,
+                       xs, bs->K, out, bs->chunks + c0, (int)(c1 - c0), F, ldo, sh.slice_floats, sh.slice_pad, sh.n_slices, sh.G);
+    return SGNN_OK;
+}
+
+template <int VEC>
+static void launch_fill_or_divide(float *out, int64_t M, int F, int64_t ldo, const float *row_div, hipStream_t st) {
+    const int64_t n = M * (F / VEC);
+    const uint32_t nb = (uint32_t)((n + kBlock - 1) / kBlock);
+    if (row_div) hipLaunchKernelGGL((rows_fill_or_divide_kernel<VEC, true>), dim3(nb), dim3(kBlock), 0, st, out, M, F, ldo, row_div);
+    else hipLaunchKernelGGL((rows_fill_or_divide_kernel<VEC, false>), dim3(nb), dim3(kBlock), 0, st, out, M, F, ldo, row_div);
+}
+
+// The product through the band schedule.  may_build = false (the non-allocating entry point): use a schedule
+// only if an earlier call has built it; *done tells whether the product was carried out here.
+static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *val, const DenseSrc &dense, float *out, int64_t F,
+                         int64_t ldo, int accumulate, const float *row_div, hipStream_t st, bool may_build, bool *done) {
+    *done = false;
+    BandSchedule *bs = nullptr;
+    for (BandSchedule *c : p->bands)
+        if (c->band_cols == sh.band_cols) bs = c;
+    const size_t xs_floats = (size_t)sh.n_slices * (size_t)p->K * (size_t)sh.slice_pad;
+    if (bs == nullptr || xs_floats > p->band_xs_floats) {
+        if (!may_build) return SGNN_OK;
+        bool sorted = false;
+        int rc = band_rows_sorted(p, st, &sorted);
+        if (rc != SGNN_OK) return rc;
+        if (!sorted) return SGNN_OK;  // band edges of a row would not be contiguous: the other schedules take it
+        if (bs == nullptr) {
+            if ((rc = band_build(p, sh.band_cols, sh.n_bands, st, &bs)) != SGNN_OK) return rc;
+            p->bands.push_back(bs);
+        }
+        if (xs_floats > p->band_xs_floats) {
+            SGNN_HIP_CHECK(hipDeviceSynchronize());  // the old workspace may still be read by queued work
+            (void)hipFree(p->band_xs);
+            p->band_xs = nullptr;
+            p->band_xs_floats = 0;
+            SGNN_HIP_CHECK(hipMalloc(&p->band_xs, xs_floats * sizeof(float)));
+            p->band_xs_floats = xs_floats;
+        }
+    }
+    const float *val_bm = nullptr;
+    if (val != nullptr) {
+        const bool bound = val == p->bound_val;
+        if (!(bound && bs->val_gen == p->bind_gen)) {
+            hipLaunchKernelGGL(permute_values_kernel, dim3((uint32_t)((p->nnz + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, val,
+                               bs->eperm_bm, bs->val_bm, p->nnz);
+            bs->val_gen = bound ? p->bind_gen : 0;
+        }
+        val_bm = bs->val_bm;
+    }
+    const int iF = (int)F;
+    {
+        ProfScope prof(K_SPMM_BAND_RESTAGE, st);
+        const int64_t n = (int64_t)sh.n_slices * p->K * (sh.slice_pad / 4);
+        hipLaunchKernelGGL(band_restage_kernel, dim3((uint32_t)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, dense.x, dense.ldx,
+                           p->band_xs, p->K, iF, sh.slice_floats, sh.slice_pad, sh.n_slices);
+    }
+    const int ev = sh.even ? 2 : 1;  // vector width of the fill / divide passes
+    if (!accumulate) {
+        if (ev == 2) launch_fill_or_divide<2>(out, p->M, iF, ldo, nullptr, st);
+        else launch_fill_or_divide<1>(out, p->M, iF, ldo, nullptr, st);
+    }
+    {
+        ProfScope prof(K_SPMM_BAND, st);
+        for (int b = 0; b < bs->n_bands; ++b) {
+            const int rc = sh.even ? launch_band<true>(bs, sh, b, val_bm, p->band_xs, out, iF, ldo, st)
+                                   : launch_band<false>(bs, sh, b, val_bm, p->band_xs, out, iF, ldo, st);
+            if (rc != SGNN_OK) return rc;
+        }
+    }
+    if (row_div) {
+        if (ev == 2) launch_fill_or_divide<2>(out, p->M, iF, ldo, row_div, st);
+        else launch_fill_or_divide<1>(out, p->M, iF, ldo, row_div, st);
+    }
+    SGNN_HIP_CHECK(hipGetLastError());
+    *done = true;
+    return SGNN_OK;
+}
+
+extern "C" int sgnn_spmm_plan_schedule(const sgnn_spmm_plan *p, int64_t F, int64_t info[4]) {
+    SGNN_REQUIRE(p != nullptr && info != nullptr, "null argument");
+    SGNN_REQUIRE(F > 0 && F < (1 << 24), "feature width F=%lld out of range", (long long)F);
+    const BandShape sh = band_shape(p, F, true);
+    info[0] = (band_wanted(p, F, sh) && p->cols_sorted != 0) ? 1 : 0;
+    info[1] = sh.band_cols; info[2] = sh.n_bands; info[3] = sh.n_slices;
+    return SGNN_OK;
+}
+
 // scratch != null: the call must not allocate.  The piece partials then go to `scratch` (scratch_floats
 // floats) instead of the plan's own, growable buffer, and nothing is created on the way.
 static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, int bits, float *out, int64_t F,
@@ -1079,6 +1733,14 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     } else if (F % 2 == 0 && dense.ldx % 2 == 0 && ldo % 2 == 0 && aligned(dense.x, 8) && aligned(out, 8)) {
         vec = 2;
     }
+    if (bits == 0) {
+        const BandShape sh = band_shape(p, F, ldo % 2 == 0 && aligned(out, 8));
+        if (band_wanted(p, F, sh)) {
+            bool done = false;
+            const int rc = spmm_run_band(p, sh, val, dense, out, F, ldo, accumulate, row_div, st, scratch == nullptr, &done);
+            if (rc != SGNN_OK || done) return rc;
+        }
+    }
     const int nvec = (int)(F / vec);
     const int gw = group_width(nvec);
     const int which = gw == 8 ? 0 : gw == 16 ? 1 : 2;
@@ -1119,7 +1781,12 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
 extern "C" int sgnn_spmm_plan_bind_values(sgnn_spmm_plan *p, const float *val, sgnn_stream_t stream) {
     SGNN_REQUIRE(p != nullptr, "plan is null");
     p->bound_val = nullptr;
-    if (val == nullptr || !p->partitioned || p->long_edges == 0) return SGNN_OK;  // nothing to regroup
+    ++p->bind_gen;  // band schedules refill their value copies on their next use
+    if (val == nullptr) return SGNN_OK;
+    if (!p->partitioned || p->long_edges == 0) {  // nothing to regroup for the piece path
+        p->bound_val = val;
+        return SGNN_OK;
+    }
     if (p->val_long == nullptr) SGNN_HIP_CHECK(hipMalloc(&p->val_long, sizeof(float) * (size_t)p->long_edges));
     const int64_t nb = (p->long_edges + kBlock - 1) / kBlock;
     hipLaunchKernelGGL(permute_values_kernel, dim3((uint32_t)nb), dim3(kBlock), 0, (hipStream_t)stream, val, p->eperm,

@@ -124,6 +124,12 @@ class SpmmPlan:
                 "partitioned", "top_share_ppm")
         return dict(zip(keys, list(buf)))
 
+    def schedule(self, F):
+        """Which schedule a product of feature width F takes (sgnn_spmm_plan_schedule)."""
+        buf = (ctypes.c_int64 * 4)()
+        check(lib.sgnn_spmm_plan_schedule(self._h, int(F), buf))
+        return dict(zip(("band", "band_cols", "n_bands", "n_slices"), list(buf)))
+
     def run(self, value, mat, out, accumulate=True, row_div=None):
         """out (+)= A @ mat on the current stream.  value None = all ones."""
         _want(mat, torch.float32, "mat")

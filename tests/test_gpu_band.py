@@ -1,0 +1,170 @@
+"""The band schedule of the SpMM (column bands x feature slices per XCD, one launch per band) against
+the CPU oracle.  It sums every row's edges in CSR order with one fma per edge starting from the old
+out value, so with column-sorted rows the result must equal the reference's BIT FOR BIT for every row
+length -- stronger than the rel 1e-5 / abs 1e-6 bar.  The schedule is forced here (it is normally
+chosen only for dense-degree matrices that do not fit the caches) with small bands, so that many bands,
+ragged last bands and empty (row, band) pairs occur at sizes the oracle finishes in a blink."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from _util import random_csr
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    import super_gnn_amd  # noqa: F401
+    from super_gnn_amd import supergnn_ops
+    return supergnn_ops
+
+
+def _force(monkeypatch, cols):
+    monkeypatch.setenv("SGNN_SPMM_BAND", "1")
+    monkeypatch.setenv("SGNN_SPMM_BAND_COLS", str(cols))
+
+
+@pytest.mark.parametrize("M,K,F,deg,cols", [
+    (700, 900, 602, 40, 128),     # the wide odd width: float2 lanes, 8 slices of 38 vectors, 8 bands
+    (500, 1000, 128, 30, 100),    # float4, 2 slices x 4 row groups; band width not a power of two
+    (300, 800, 256, 25, 256),     # 4 slices x 2 row groups
+    (257, 600, 64, 20, 64),       # one slice, 8 row groups
+    (300, 500, 123, 20, 70),      # scalar lanes
+    (200, 400, 100, 15, 50),      # float4 with a ragged last slice
+    (150, 300, 2052, 9, 40),      # slices wider than one register tile
+    (90, 200, 4, 6, 16), (90, 200, 1, 6, 16), (64, 100, 10, 5, 7),
+    (400, 5000, 602, 12, 37),     # 136 bands, most (row, band) pairs empty
+])
+def test_band_schedule_bit_identical_to_oracle(M, K, F, deg, cols, monkeypatch):
+    ops = _ops()
+    _force(monkeypatch, cols)
+    rowptr, col, val = random_csr(M, K, deg, seed=M + F, empty_frac=0.1, hubs=3, hub_deg=min(K, 700))
+    rng = np.random.default_rng(F)
+    x = rng.standard_normal((K, F), dtype=np.float32)
+    init = rng.standard_normal((M, F), dtype=np.float32)
+    dev = torch.device("cuda:0")
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    sch = plan.schedule(F)
+    assert sch["band"] == 1 and sch["band_cols"] == cols and sch["n_bands"] == -(-K // cols)
+    w, xd = torch.from_numpy(val).to(dev), torch.from_numpy(x).to(dev)
+    deg_f = np.maximum(np.diff(rowptr), 1).astype(np.float32)
+    div = torch.from_numpy(deg_f).to(dev)
+
+    want = init.copy(); orc.spmm_accumulate(rowptr, col, val, x, want)
+    out = torch.from_numpy(init.copy()).to(dev)
+    plan.run(w, xd, out, accumulate=True)
+    assert np.array_equal(out.cpu().numpy(), want), "accumulate"
+    out2 = torch.from_numpy(init.copy()).to(dev)
+    plan.run(w, xd, out2, accumulate=True)     # second call: the weights are bound to the plan now
+    assert torch.equal(out, out2)
+
+    # overwrite + mean: (A x) / deg for every row, rows without edges zero
+    want0 = np.zeros_like(init); orc.spmm_accumulate(rowptr, col, val, x, want0)
+    orc.row_divide(want0, deg_f)
+    out3 = torch.from_numpy(init.copy()).to(dev)
+    plan.run(w, xd, out3, accumulate=False, row_div=div)
+    assert np.array_equal(out3.cpu().numpy(), want0), "overwrite + mean"
+
+    # unit weights (val == NULL), accumulate + mean: (old + A x) / deg, also for rows without edges
+    ones = np.ones_like(val)
+    want1 = init.copy(); orc.spmm_accumulate(rowptr, col, ones, x, want1)
+    orc.row_divide(want1, deg_f)
+    out4 = torch.from_numpy(init.copy()).to(dev)
+    plan.run(None, xd, out4, accumulate=True, row_div=div)
+    assert np.array_equal(out4.cpu().numpy(), want1), "unit weights + mean"
+
+
+def test_band_schedule_equals_row_class_schedule_and_honours_rebinding(monkeypatch):
+    ops = _ops()
+    dev = torch.device("cuda:0")
+    M, K, F = 3000, 2000, 128
+    rowptr, col, val = random_csr(M, K, 60, seed=5, hubs=4, hub_deg=1500)
+    x = torch.randn(K, F, generator=torch.Generator().manual_seed(1)).to(dev)
+    w = torch.from_numpy(val).to(dev)
+    rp, cl = torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev)
+    monkeypatch.setenv("SGNN_SPMM_BAND", "0")
+    ref = torch.zeros(M, F, device=dev)
+    ops.SpmmPlan(rp, cl, K).run(w, x, ref, accumulate=True)
+    _force(monkeypatch, 300)
+    plan = ops.SpmmPlan(rp, cl, K)
+    out = torch.zeros(M, F, device=dev)
+    for _ in range(3):                          # 2nd call binds, 3rd reuses the bound copy
+        out.zero_()
+        plan.run(w, x, out, accumulate=True)
+    short = torch.from_numpy(np.diff(rowptr) <= 128).to(dev)
+    assert torch.equal(out[short], ref[short])                    # both schedules: reference order on short rows
+    assert torch.allclose(out, ref, rtol=1e-5, atol=1e-5)
+    # in-place edit of the bound weights: the version counter moves, the plan must not use its stale copy
+    w.mul_(2.0)
+    out2 = torch.zeros(M, F, device=dev)
+    plan.run(w, x, out2, accumulate=True)
+    assert torch.equal(out2, out * 2.0)
+    # another tensor of weights altogether
+    w3 = torch.rand_like(w)
+    out3 = torch.zeros(M, F, device=dev)
+    plan.run(w3, x, out3, accumulate=True)
+    want3 = np.zeros((M, F), np.float32)
+    orc.spmm_accumulate(rowptr, col, w3.cpu().numpy(), x.cpu().numpy(), want3)
+    assert np.array_equal(out3.cpu().numpy(), want3)
+
+
+def test_unsorted_rows_keep_the_row_class_schedule(monkeypatch):
+    ops = _ops()
+    _force(monkeypatch, 64)
+    dev = torch.device("cuda:0")
+    M, K, F = 400, 500, 64
+    rowptr, col, val = random_csr(M, K, 30, seed=9, dup=True)    # columns in random order inside each row
+    assert any(np.any(np.diff(col[rowptr[r]:rowptr[r + 1]]) < 0) for r in range(M))
+    x = np.random.default_rng(2).standard_normal((K, F), dtype=np.float32)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    out = torch.zeros(M, F, device=dev)
+    plan.run(torch.from_numpy(val).to(dev), torch.from_numpy(x).to(dev), out, accumulate=True)
+    want = np.zeros((M, F), np.float32); orc.spmm_accumulate(rowptr, col, val, x, want)
+    assert np.array_equal(out.cpu().numpy(), want)               # all rows short: CSR order either way
+    assert plan.schedule(F)["band"] == 0                          # the plan has seen that rows are unsorted
+
+
+def test_band_schedule_with_leading_dimensions_through_the_c_abi(monkeypatch):
+    ops = _ops()
+    from super_gnn_amd._lib import lib, check
+    _force(monkeypatch, 90)
+    dev = torch.device("cuda:0")
+    M, K, F = 600, 700, 602
+    rowptr, col, val = random_csr(M, K, 35, seed=31, empty_frac=0.05)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    g = torch.Generator().manual_seed(3)
+    xw = torch.randn(K, F + 6, generator=g).to(dev)
+    ow = torch.randn(M, F + 10, generator=g).to(dev)
+    w = torch.from_numpy(val).to(dev)
+    got = ow.clone()
+    check(lib.sgnn_spmm_csr_f32(plan._h, w.data_ptr(), xw.data_ptr() + 8, got.data_ptr() + 16, F, F + 6, F + 10, 1, None,
+                                torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    want = ow[:, 4:4 + F].cpu().numpy().copy()
+    orc.spmm_accumulate(rowptr, col, val, xw[:, 2:2 + F].contiguous().cpu().numpy(), want)
+    assert np.array_equal(got[:, 4:4 + F].cpu().numpy(), want)
+    keep = torch.ones(F + 10, dtype=torch.bool, device=dev); keep[4:4 + F] = False
+    assert torch.equal(got[:, keep], ow[:, keep])
+
+
+def test_full_size_community_graph_takes_the_band_schedule_and_matches_oracle():
+    # the dense-degree configuration at full size with real-valued features: 233 k nodes, ~114 M edges, F = 602
+    from super_gnn_amd import synth
+    ops = _ops()
+    dev = torch.device("cuda:0")
+    n, F = 233_000, 602
+    rowptr, col = synth.sbm_graph(n, 50, 0.03048, 0.001524, seed=3, device=dev)
+    g = torch.Generator(device=dev); g.manual_seed(4)
+    x = torch.rand(n, F, generator=g, device=dev) * 2 - 1
+    plan = ops.SpmmPlan(rowptr, col, n)
+    sch = plan.schedule(F)
+    print(f"\n[cfg3] schedule {sch}", flush=True)
+    assert sch["band"] == 1 and sch["n_bands"] >= 8
+    out = torch.zeros(n, F, device=dev)
+    plan.run(None, x, out, accumulate=True)
+    torch.cuda.synchronize()
+    rp, cl = rowptr.cpu().numpy(), col.cpu().numpy().astype(np.int64)
+    want = np.zeros((n, F), np.float32)
+    orc.spmm_accumulate(rp, cl, np.ones(cl.shape[0], np.float32), x.cpu().numpy(), want)
+    assert np.array_equal(out.cpu().numpy(), want), "band schedule: the reference's fma chain, bit for bit"
