@@ -1,20 +1,33 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident in
-HBM: by default the headline configuration, a weighted-sum SpMM (out += A @ X, GCN-normalised edge
-weights) over an R-MAT power-law graph with 2.45 M nodes / ~62 M stored edges at F = 128 fp32.
-The same run also reports, as extras, the mean-aggregation variant, the int8/int4/int2
-quantize+pack and unpack+dequantize kernels on 1 M x 256 boundary rows, a plain streaming copy (the
-attainable-bandwidth yardstick), and a CPU baseline timed on this machine's host cores.
+HBM.  The default workload is the headline configuration: a weighted-sum SpMM (out += A @ X,
+GCN-normalised edge weights) over an R-MAT power-law graph with 2.45 M nodes / ~62 M stored edges
+at F = 128 fp32.  Unless --no-extras is given the same run also measures, as entries of
+``extra["workloads"]`` with their own kernel times and roofline objects: the dense-degree
+community graph at F = 602 (``sbm``), the pre/post-aggregation partition with int2-packed remote
+rows (``prepost``), the small CPU-runnable case (``small``), the int8/int4/int2 quantize+pack and
+unpack+dequantize kernels on 1 M x 256 and 2 M x 128 boundary rows (``quant``), a streaming copy
+(the attainable-bandwidth yardstick) and the CPU baselines timed on this machine's host cores.
+Any of them can be made the headline of the line with --workload.
+
+Roofline objects: ``achieved`` is HBM-side bytes per launch of the dominant kernel (rocprofv3
+FETCH_SIZE + WRITE_SIZE, read from the ``traffic:`` lines of the summaries under profiles/) divided
+by that kernel's average duration, measured here with HIP events on the launch stream; ``frac`` is
+that over the 8 TB/s peak and is therefore at most 1.  The gather-model rate (algorithmic bytes,
+cache hits counted as if they were memory traffic; it can exceed the peak) is reported beside it as
+``gather_model``.  Without a measured traffic figure for the workload ``achieved``/``frac`` are null.
 
 Prints ONE JSON line on stdout (everything else goes to stderr).
 """
 import argparse
+import glob
 import json
 import os
+import re
 import sys
 import time
 
@@ -24,19 +37,59 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this file (see profiles/), scaled by what the same counters read for sgnn_stream_copy_f32 of a
-# known size.  Keyed by workload name; None = not measured.
-MEASURED_TRAFFIC_BYTES = {
-    # spmm_piece_kernel (values bound to the plan): FETCH_SIZE 4041502 x 2.000 + WRITE_SIZE 860068 x 1.000 (KiB per launch)
-    "rmat_2450000n_62000000e_F128_gcn_weighted_sum": 9_157_000_000,
-    # quant_pack_rows16_kernel<2,...>: FETCH_SIZE 500052 x 2.000 + WRITE_SIZE 76196 x 1.000
-    "quant_pack_int2_1000000x256": 1_102_000_000,
-}
-
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+# ---------------------------------------------------------------------------------------------------
+# measured traffic: "traffic: workload=<w> kernel=<k> fetch_bytes=<n> write_bytes=<n> [l2_hit=<x>]" lines
+# of the rocprofv3 summaries under profiles/ (each summary names the command that produced it)
+# ---------------------------------------------------------------------------------------------------
+def load_measured_traffic():
+    table = {}
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.txt"))):
+        for line in open(path):
+            if not line.startswith("traffic:"):
+                continue
+            kv = dict(re.findall(r"(\w+)=(\S+)", line))
+            try:
+                table[(kv["workload"], kv["kernel"])] = {
+                    "bytes": int(kv["fetch_bytes"]) + int(kv["write_bytes"]),
+                    "fetch_bytes": int(kv["fetch_bytes"]), "write_bytes": int(kv["write_bytes"]),
+                    "l2_hit": float(kv["l2_hit"]) if "l2_hit" in kv else None,
+                    "source": "profiles/" + os.path.basename(path)}
+            except (KeyError, ValueError):
+                continue
+    return table
+
+
+TRAFFIC = load_measured_traffic()
+
+
+def roofline(workload, kernel, kernel_ms, algorithmic_bytes, launches_per_step=1):
+    """Roofline object of one kernel.  ``kernel_ms`` is per step (all launches of the kernel in one step)."""
+    t = TRAFFIC.get((workload, kernel))
+    ach = t["bytes"] / kernel_ms / 1e6 if t else None
+    gm = algorithmic_bytes / kernel_ms / 1e6
+    return {"bound": "hbm", "achieved": round(ach, 1) if ach else None, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(ach / HBM_PEAK_GBPS, 4) if ach else None,
+            "traffic": t["bytes"] if t else None, "traffic_source": t["source"] if t else None,
+            "l2_hit_rate": t["l2_hit"] if t else None,
+            "kernel": kernel, "kernel_ms_per_step": round(kernel_ms, 5), "launches_per_step": launches_per_step,
+            "gather_model": {"algorithmic_bytes": int(algorithmic_bytes), "GBps": round(gm, 1),
+                             "frac_of_peak": round(gm / HBM_PEAK_GBPS, 4)}}
+
+
+def step_roofline(workload, per_kernel_ms):
+    """All kernels of a step together: measured traffic summed over the kernels that have a figure."""
+    have = {k: TRAFFIC[(workload, k)] for k in per_kernel_ms if (workload, k) in TRAFFIC}
+    if not have:
+        return None
+    total = sum(v["bytes"] for v in have.values())
+    ms = sum(per_kernel_ms[k] for k in have)
+    return {"traffic": total, "kernels": sorted(have), "kernel_ms_sum": round(ms, 5), "GBps": round(total / ms / 1e6, 1),
+            "frac": round(total / ms / 1e6 / HBM_PEAK_GBPS, 4)}
 
 
 def spmm_gather_bytes(nnz, rows, F, weighted, accumulate, mean, empty_rows=0):
@@ -50,6 +103,11 @@ def spmm_gather_bytes(nnz, rows, F, weighted, accumulate, mean, empty_rows=0):
     touched = rows - (empty_rows if accumulate else 0)
     per_touched = 4 * F + (4 * F if accumulate else 0) + (4 if mean else 0)
     return nnz * per_edge + rows * 8 + touched * per_touched
+
+
+def spmm_compulsory_bytes(nnz, M, K, F, weighted):
+    """Each array once: 4KF + 4MF (+4MF read when accumulating is not counted) + 4nnz (+4nnz) + 8(M+1)."""
+    return 4 * K * F + 4 * M * F + 4 * nnz + (4 * nnz if weighted else 0) + 8 * (M + 1)
 
 
 def quant_bytes(rows, F, bits):
@@ -67,6 +125,23 @@ def time_steps(fn, steps, warmup):
         fn()
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def profiled_steps(fn, steps, warmup):
+    """(ms per step, {kernel: ms per step}, {kernel: launches per step}) with the library's HIP-event profiler."""
+    from super_gnn_amd import _lib
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    _lib.profile_start()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    prof = _lib.profile_stop()
+    return ms, {k: v[1] / steps for k, v in prof.items()}, {k: v[0] / steps for k, v in prof.items()}
 
 
 def time_reps_events(fn, reps, warmup, flush=None):
@@ -112,10 +187,13 @@ def build_headline_graph(nodes, und_edges, F, device):
     return rowptr, col, w, x
 
 
+# ---------------------------------------------------------------------------------------------------
+# CPU baselines (reported, never the target): the reference's own x86 extension when oracle/_ref is
+# loadable on this host, else the C restatement
+# ---------------------------------------------------------------------------------------------------
 def cpu_baseline_spmm(rowptr, col, w, x, target_edges=1 << 40, reps=10):
     """Time the CPU path on the same graph (all rows unless target_edges bounds the sample to the
-    leading rows holding that many edges), gathering from the full X.  Uses the reference's own x86
-    extension when oracle/_ref is loadable on this host, else the C restatement."""
+    leading rows holding that many edges), gathering from the full X."""
     import numpy as np
     import torch
     from oracle import oracle as orc
@@ -148,24 +226,424 @@ def cpu_baseline_spmm(rowptr, col, w, x, target_edges=1 << 40, reps=10):
         run()
         ts.append(time.perf_counter() - t0)
     t = float(np.median(ts))
-    return {"value": nnz / t / 1e9, "unit": "GEdges/s", "cores": int(T), "kind": kind,
+    return {"value": nnz / t / 1e9, "unit": "GEdges/s", "cores": int(T), "host_cpu_count": os.cpu_count(), "kind": kind,
             "sample": f"{m} of {rp.numel() - 1} rows ({nnz} edges) of the same graph, full X, F={F}, 1 warm-up + median of {reps}",
             "ms": t * 1e3}
 
 
 def cpu_baseline_quant(x, bits, rows=200_000, reps=3):
+    """(port, reference-or-None).  The port is the C restatement of the ARM kernel the live path calls
+    (params + codes + packing, quantization_arm.cpp:79-301).  The reference figure times the x86 build of
+    the reference, whose quantize_tensor packs given (min, scale) vectors (quantization_x86.cpp:17-110); the
+    torch amin/amax/scale computation that has to precede it is inside the timed region."""
     import numpy as np
+    import torch
     from oracle import oracle as orc
-    xs = x[:rows].cpu().numpy()
-    orc.quant_rows(xs, [0, rows], bits)
-    ts = []
-    for _ in range(reps):
-        t0 = time.perf_counter()
-        orc.quant_rows(xs, [0, rows], bits)
-        ts.append(time.perf_counter() - t0)
-    t = float(np.median(ts))
-    return {"value": quant_bytes(rows, xs.shape[1], bits) / t / 1e9, "unit": "GB/s", "cores": orc.num_threads(),
-            "kind": "port", "sample": f"first {rows} rows, int{bits}, median of {reps}"}
+    xs_t = x[:rows].cpu().contiguous()
+    xs = xs_t.numpy()
+    F = xs.shape[1]
+
+    def med(fn):
+        fn()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return float(np.median(ts))
+
+    t = med(lambda: orc.quant_rows(xs, [0, rows], bits))
+    port = {"value": quant_bytes(rows, F, bits) / t / 1e9, "unit": "GB/s", "cores": orc.num_threads(),
+            "host_cpu_count": os.cpu_count(), "kind": "port", "sample": f"first {rows} rows x {F}, int{bits}, median of {reps}"}
+    ref = orc.ref_ops()
+    refd = None
+    if ref is not None:
+        epb = 8 // bits
+        q = torch.zeros(((rows + epb - 1) // epb) * F, dtype=torch.uint8)
+
+        def run():
+            mn = xs_t.amin(dim=1)
+            sc = (xs_t.amax(dim=1) - mn) / float((1 << bits) - 1)
+            sc = torch.where(sc == 0, torch.ones_like(sc), sc)
+            ref.quantize_tensor(xs_t, q, mn, sc, bits)
+
+        t = med(run)
+        refd = {"value": quant_bytes(rows, F, bits) / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+                "host_cpu_count": os.cpu_count(), "kind": "reference",
+                "sample": f"first {rows} rows x {F}, int{bits}: torch amin/amax/scale + the x86 extension's quantize_tensor, median of {reps}"}
+    return port, refd
+
+
+# ---------------------------------------------------------------------------------------------------
+# workloads: each returns a dict with metric / value / unit / config / ms_per_step / dtype / roofline /
+# cpu_baseline / extra
+# ---------------------------------------------------------------------------------------------------
+def wl_copy(args, ctx):
+    import torch
+    from super_gnn_amd import _lib
+    n_copy = 256 * 1024 * 1024  # 1 GiB in + 1 GiB out
+    src = torch.empty(n_copy, device=ctx["dev"]).normal_()
+    dst = torch.empty_like(src)
+    fn = lambda: _lib.check(_lib.lib.sgnn_stream_copy_f32(src.data_ptr(), dst.data_ptr(), n_copy, ctx["stream"]()))  # noqa: E731
+    ms, per_k, _ = profiled_steps(fn, args.steps, args.warmup)
+    b = 2 * 4 * n_copy
+    k_ms = per_k["stream_copy_kernel"]
+    return {"metric": "stream copy GB/s", "value": round(b / ms / 1e6, 2), "unit": "GB/s",
+            "config": {"workload": "stream_copy_1GiB"}, "ms_per_step": ms, "dtype": "f32",
+            "roofline": {"bound": "hbm", "achieved": round(b / k_ms / 1e6, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": round(b / k_ms / 1e6 / HBM_PEAK_GBPS, 4), "traffic": b, "traffic_source": "by construction",
+                         "kernel": "stream_copy_kernel", "kernel_ms_per_step": round(k_ms, 5)},
+            "cpu_baseline": None, "extra": {}}
+
+
+def quant_case(ops, x, bits, steps, warmup):
+    """Quantize+pack and unpack+dequantize of x at one width: times, rates, rooflines."""
+    import torch
+    n, F = x.shape
+    epb = 8 // bits
+    seg = torch.tensor([0, n], dtype=torch.int32)
+    q = torch.empty((n + epb - 1) // epb, F, dtype=torch.uint8, device=x.device)
+    p = torch.empty(n, 2, device=x.device)
+    d = torch.empty(n, F, device=x.device)
+    wl = f"quant_pack_int{bits}_{n}x{F}"
+    b = quant_bytes(n, F, bits)
+    ms_q, kq, _ = profiled_steps(lambda: ops.quantize_tensor_for_all_procs(x, q, p, seg, 1, bits), steps, warmup)
+    ms_d, kd, _ = profiled_steps(lambda: ops.dequantize_tensor_for_all_procs(q, d, p, seg, 1, bits), steps, warmup)
+    kq_ms, kd_ms = kq["quant_pack_rows_kernel"], kd["unpack_dequant_rows_kernel"]
+    return {"workload": wl, "bytes": b, "quant_ms": ms_q, "dequant_ms": ms_d,
+            "quant_GBps_wall": round(b / ms_q / 1e6, 1), "dequant_GBps_wall": round(b / ms_d / 1e6, 1),
+            "quant_roofline": roofline(wl, "quant_pack_rows_kernel", kq_ms, b),
+            "dequant_roofline": roofline(wl.replace("quant_pack", "unpack_dequant"), "unpack_dequant_rows_kernel", kd_ms, b)}
+
+
+def wl_quant(args, ctx, rows=None, feat=None, headline=True):
+    from super_gnn_amd import synth, supergnn_ops as ops
+    n, F = rows or args.quant_rows, feat or args.quant_feat
+    xq = synth.boundary_features(n, F, seed=5, device=ctx["dev"])
+    cases = {}
+    for bits in (8, 4, 2):
+        if headline and args.no_extras and bits != args.bits:
+            continue
+        c = quant_case(ops, xq, bits, args.steps if (headline and bits == args.bits) else 10, args.warmup if headline else 3)
+        cases[bits] = c
+        log(f"[bench] {n}x{F} int{bits}: quantize+pack kernel {c['quant_roofline']['gather_model']['GBps']:.0f} GB/s "
+            f"({c['quant_roofline']['kernel_ms_per_step'] * 1e3:.1f} us), unpack+dequant kernel "
+            f"{c['dequant_roofline']['gather_model']['GBps']:.0f} GB/s ({c['dequant_roofline']['kernel_ms_per_step'] * 1e3:.1f} us)")
+    main = cases[args.bits]
+    cpu_port = cpu_ref = None
+    if not args.no_cpu:
+        cpu_port, cpu_ref = cpu_baseline_quant(xq, args.bits)
+    extra = {f"int{b}": {k: v for k, v in c.items() if k != "workload"} for b, c in cases.items()}
+    if cpu_ref is not None:
+        extra["cpu_port"] = cpu_port
+    # the quantizer's algorithmic bytes ARE its compulsory traffic (one read, one write): the roofline fraction of
+    # a kernel without a traffic figure falls back to them
+    rf = main["quant_roofline"]
+    if rf["achieved"] is None:
+        rf = dict(rf, achieved=rf["gather_model"]["GBps"], frac=rf["gather_model"]["frac_of_peak"],
+                  traffic_source="algorithmic bytes (one read + one write per element; no reuse to credit)")
+    return {"metric": f"quantize-pack GB/s at int{args.bits}", "value": round(main["bytes"] / main["quant_ms"] / 1e6, 2),
+            "unit": "GB/s", "config": {"workload": main["workload"], "rows": n, "F": F, "bits": args.bits},
+            "ms_per_step": main["quant_ms"], "dtype": "f32->u8", "roofline": rf,
+            "cpu_baseline": cpu_ref or cpu_port, "extra": extra}
+
+
+def wl_rmat(args, ctx):
+    import torch
+    from super_gnn_amd import supergnn_ops as ops
+    dev, F = ctx["dev"], args.feat
+    extra = {}
+    if args.uniform_rows:
+        g = torch.Generator(device=dev); g.manual_seed(11)
+        M, dg = args.uniform_rows, args.uniform_degree
+        col = torch.sort(torch.randint(0, args.nodes, (M, dg), generator=g, device=dev), dim=1).values
+        col = col.reshape(-1).to(torch.int32).contiguous()
+        rowptr = torch.arange(M + 1, device=dev, dtype=torch.int64) * dg
+        w = torch.rand(col.numel(), generator=g, device=dev)
+        x = torch.randn(args.nodes, F, generator=g, device=dev)
+    else:
+        rowptr, col, w, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
+    M, nnz = rowptr.numel() - 1, col.numel()
+    t0 = time.perf_counter()
+    plan = ops.SpmmPlan(rowptr, col, x.shape[0], long_row_threshold=args.long_threshold, piece_edges=args.piece_edges)
+    torch.cuda.synchronize()
+    info = plan.info()
+    extra["plan_build_ms"] = round((time.perf_counter() - t0) * 1e3, 1)
+    extra["plan"] = {k: info[k] for k in ("long_rows", "pieces", "long_edges", "long_row_threshold", "piece_edges", "partitioned")}
+    log(f"[bench] plan: {extra['plan']} built in {extra['plan_build_ms']} ms")
+    out = torch.zeros(M, F, device=dev)
+    step = lambda: plan.run(w, x, out, accumulate=True)  # noqa: E731
+    ms, per_kernel, launches = profiled_steps(step, args.steps, args.warmup)
+    log(f"[bench] weighted sum: {ms:.3f} ms/step, {nnz / ms / 1e6:.2f} GEdges/s, kernels (ms per step) "
+        f"{ {k: round(v, 4) for k, v in per_kernel.items()} }")
+    short_edges = nnz - info["long_edges"]
+    short_rows = M - info["long_rows"]
+    n_empty = int(((rowptr[1:] - rowptr[:-1]) == 0).sum())
+    b_short = spmm_gather_bytes(short_edges, short_rows, F, weighted=True, accumulate=True, mean=False, empty_rows=n_empty)
+    b_total = spmm_gather_bytes(nnz, M, F, weighted=True, accumulate=True, mean=False, empty_rows=n_empty)
+    extra["empty_rows"] = n_empty
+    dom = max(per_kernel, key=per_kernel.get)
+    if dom == "spmm_short_kernel":
+        dom_bytes = b_short
+    elif dom == "spmm_piece_kernel":
+        # per edge: dense row + col + val (the per-unit figure of the gather model); the kernel's own
+        # bookkeeping (edge permutation, piece partial sums) is overhead, not algorithmic traffic
+        dom_bytes = info["long_edges"] * (4 * F + 8)
+    else:
+        dom_bytes = b_total
+    wl = (f"rmat_{M}n_{nnz}e_F{F}_gcn_weighted_sum" if not args.uniform_rows
+          else f"uniform_{M}x{args.nodes}_deg{args.uniform_degree}_F{F}")
+    if not args.no_extras:
+        deg = (rowptr[1:] - rowptr[:-1]).clamp(min=1).to(torch.float32)
+        out2 = torch.zeros(M, F, device=dev)
+        ms_mean = time_steps(lambda: plan.run(None, x, out2, accumulate=True, row_div=deg), 10, 3)
+        extra["spmm_mean_GEdges_per_s"] = round(nnz / ms_mean / 1e6, 3)
+        extra["spmm_mean_gather_GBps"] = round(spmm_gather_bytes(nnz, M, F, False, True, True, empty_rows=n_empty) / ms_mean / 1e6, 1)
+        del out2
+        scratch = torch.empty(192 * 1024 * 1024, device=dev)   # 768 MB > 8 x 4 MB L2 + 256 MB Infinity Cache
+        extra["spmm_warm"] = time_reps_events(step, 20, 5)
+        extra["spmm_cache_flushed"] = time_reps_events(step, 20, 2, flush=lambda: scratch.fill_(1.0))
+        log(f"[bench] weighted sum per repetition: warm {extra['spmm_warm']}, caches flushed before each {extra['spmm_cache_flushed']}")
+        del scratch
+    # one-time preparation, like the plan itself: the unchanged weight tensor was bound during warm-up
+    extra["edge_values_bound_to_plan"] = plan._bound is not None
+    extra["gather_model_total"] = {"algorithmic_bytes": int(b_total), "GBps": round(b_total / ms / 1e6, 1),
+                                   "frac_of_peak": round(b_total / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    extra["compulsory_bytes"] = int(spmm_compulsory_bytes(nnz, M, x.shape[0], F, True))
+    extra["spmm_GFLOPs"] = round(2.0 * nnz * F / ms / 1e6, 1)
+    extra["kernel_ms_per_step"] = {k: round(v, 5) for k, v in per_kernel.items()}
+    extra["step_roofline"] = step_roofline(wl, per_kernel)
+    extra["kernel_rooflines"] = {k: roofline(wl, k, v, b_short if k == "spmm_short_kernel" else info["long_edges"] * (4 * F + 8)
+                                             if k == "spmm_piece_kernel" else 0, launches[k])
+                                 for k, v in per_kernel.items() if (wl, k) in TRAFFIC}
+    return {"metric": "SpMM GEdges/s + % HBM roofline (F=128 fp32); quantize-pack GB/s at int2",
+            "value": round(nnz / ms / 1e6, 4), "unit": "GEdges/s",
+            "config": {"workload": wl, "nodes": M, "edges": nnz, "F": F, "aggregation": "weighted_sum",
+                       "accumulate": True, "index_dtype": "int32"},
+            "ms_per_step": ms, "dtype": "f32", "roofline": roofline(wl, dom, per_kernel[dom], dom_bytes, launches[dom]),
+            "cpu_baseline": None if args.no_cpu else cpu_baseline_spmm(rowptr, col, w, x), "extra": extra}
+
+
+def wl_small(args, ctx):
+    """The small CPU-runnable configuration: cache-resident, so GEdges/s only."""
+    import torch
+    from super_gnn_amd import supergnn_ops as ops
+    dev = ctx["dev"]
+    N, F = 10_000, 128
+    g = torch.Generator().manual_seed(0)
+    col = torch.randint(0, N, (N, 16), generator=g)
+    col = torch.sort(torch.cat([col, torch.arange(N).unsqueeze(1)], dim=1), dim=1).values.reshape(-1)
+    rowptr = 17 * torch.arange(N + 1, dtype=torch.int64)
+    x = torch.randn(N, F, generator=g)
+    w = torch.ones(col.numel())
+    d_rowptr, d_col, d_w, d_x = rowptr.to(dev), col.to(torch.int32).to(dev), w.to(dev), x.to(dev)
+    plan = ops.SpmmPlan(d_rowptr, d_col, N)
+    out = torch.zeros(N, F, device=dev)
+    ms, per_k, _ = profiled_steps(lambda: plan.run(d_w, d_x, out, accumulate=True), max(args.steps, 50), max(args.warmup, 10))
+    k_ms = per_k["spmm_short_kernel"]
+    nnz = col.numel()
+    b = spmm_gather_bytes(nnz, N, F, weighted=True, accumulate=True, mean=False)
+    xq = torch.randn(2000, F, generator=g).to(dev)
+    q = torch.empty(2000, F, dtype=torch.uint8, device=dev); pq = torch.empty(2000, 2, device=dev)
+    seg1 = torch.tensor([0, 2000], dtype=torch.int32)
+    ms_q = time_steps(lambda: ops.quantize_tensor_for_all_procs(xq, q, pq, seg1, 1, 8), 50, 10)
+    extra = {"kernel_ms": round(k_ms, 5), "kernel_GEdges_per_s": round(nnz / k_ms / 1e6, 2),
+             "kernel_gather_GBps_cache_resident": round(b / k_ms / 1e6, 1),
+             "quant_int8_2000x128_us_per_call": round(ms_q * 1e3, 2)}
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline_spmm(rowptr, col, w, x, reps=20)
+        nt = torch.get_num_threads()
+        torch.set_num_threads(1)
+        cpu1 = cpu_baseline_spmm(rowptr, col, w, x, reps=5)
+        torch.set_num_threads(nt)
+        extra["cpu_1_thread_GEdges_per_s"] = round(cpu1["value"], 4)
+    log(f"[bench] small: {ms * 1e3:.1f} us/step wall, kernel {k_ms * 1e3:.1f} us = {nnz / k_ms / 1e6:.1f} GEdges/s; int8 quantize 2000x128 {ms_q * 1e3:.1f} us/call")
+    return {"metric": "SpMM GEdges/s (10k nodes x 17 edges, F=128, cache-resident)", "value": round(nnz / ms / 1e6, 4),
+            "unit": "GEdges/s", "config": {"workload": f"small_uniform_{N}n_{nnz}e_F{F}_sum"}, "ms_per_step": ms,
+            "dtype": "f32", "roofline": None, "cpu_baseline": cpu, "extra": extra}
+
+
+def wl_prepost(args, ctx):
+    """One partition in pre/post-aggregation mode: remote rows arrive int2-packed."""
+    import torch
+    from super_gnn_amd import synth, supergnn_ops as ops
+    dev, F, bits = ctx["dev"], args.feat, args.bits
+    Ml, Kr = args.local_nodes, args.remote_nodes
+    t0 = time.perf_counter()
+    rp_l, col_l = synth.rmat_graph(Ml, args.local_und_edges, seed=6, device=dev)
+    g = torch.Generator(device=dev); g.manual_seed(7)
+    # remote edges: rows follow the local degree distribution, columns uniform over the boundary set
+    deg_l = (rp_l[1:] - rp_l[:-1]).to(torch.float32)
+    rows_r = torch.multinomial(deg_l + 0.05, args.remote_edges, replacement=True, generator=g)
+    cols_r = torch.randint(0, Kr, (args.remote_edges,), generator=g, device=dev)
+    rp_r, col_r = synth.csr_from_pairs(rows_r, cols_r, Ml, Kr, dedupe=True)
+    del rows_r, cols_r, deg_l
+    x_l = torch.randn(Ml, F, generator=g, device=dev)
+    x_r = torch.randn(Kr, F, generator=g, device=dev)
+    torch.cuda.synchronize()
+    log(f"[bench] prepost: local {Ml} rows / {col_l.numel()} edges, remote {Kr} cols / {col_r.numel()} edges, "
+        f"built in {time.perf_counter() - t0:.1f}s")
+    P = 8
+    wr = torch.tensor([Kr * i // P for i in range(P + 1)], dtype=torch.int32)
+    epb = 8 // bits
+    npk = sum((int(wr[i + 1] - wr[i]) + epb - 1) // epb for i in range(P))
+    q = torch.empty(npk, F, dtype=torch.uint8, device=dev)
+    prm = torch.empty(Kr, 2, device=dev)
+    ops.quantize_tensor_for_all_procs(x_r, q, prm, wr, P, bits)
+    del x_r
+    plan_l = ops.SpmmPlan(rp_l, col_l, Ml)
+    plan_r = ops.SpmmPlan(rp_r, col_r, Kr)
+    segs = ops.quant_segments(wr, bits)
+    out = torch.zeros(Ml, F, device=dev)
+    recv = torch.empty(Kr, F, device=dev)
+    ms_local, k_local, _ = profiled_steps(lambda: plan_l.run(None, x_l, out, accumulate=True), args.steps, args.warmup)
+
+    def separate():
+        ops.dequantize_tensor_for_all_procs(q, recv, prm, wr, P, bits)
+        plan_r.run(None, recv, out, accumulate=True)
+
+    ms_sep = time_steps(separate, args.steps, args.warmup)
+    ms_fused, k_fused, launches = profiled_steps(
+        lambda: plan_r.run_quantized(None, q, prm, segs, bits, out, accumulate=True), args.steps, args.warmup)
+    nl, nr = col_l.numel(), col_r.numel()
+    dom = max(k_fused, key=k_fused.get)
+    info_r = plan_r.info()
+    dom_edges = info_r["long_edges"] if "piece" in dom else nr - info_r["long_edges"]
+    dom_bytes = dom_edges * (F + 16)  # per remote edge: one packed row of F bytes + params + col/val
+    total = ms_local + ms_fused
+    wl = f"prepost_{Ml}n_{nl}e_local_{Kr}c_{nr}e_remote_int{bits}_F{F}"
+    extra = {"local_spmm_ms": round(ms_local, 4), "remote_separate_ms": round(ms_sep, 4),
+             "remote_fused_ms": round(ms_fused, 4), "fused_speedup_on_remote_step": round(ms_sep / ms_fused, 3),
+             "local_GEdges_per_s": round(nl / ms_local / 1e6, 3),
+             "local_kernel_ms_per_step": {k: round(v, 5) for k, v in k_local.items()},
+             "fused_kernel_ms_per_step": {k: round(v, 5) for k, v in k_fused.items()},
+             "fused_step_roofline": step_roofline(wl, k_fused)}
+    log(f"[bench] prepost: local SpMM {ms_local:.3f} ms; remote: separate {ms_sep:.3f} ms vs fused {ms_fused:.3f} ms")
+    return {"metric": "SpMM GEdges/s, pre/post-aggregation partition (local fp32 + int2-packed remote rows, fused)",
+            "value": round((nl + nr) / total / 1e6, 4), "unit": "GEdges/s",
+            "config": {"workload": wl, "F": F, "bits": bits}, "ms_per_step": total, "dtype": "f32",
+            "roofline": roofline(wl, dom, k_fused[dom], dom_bytes, launches[dom]), "cpu_baseline": None, "extra": extra}
+
+
+def wl_sbm(args, ctx):
+    """Dense-degree community graph, wide odd feature rows (the band schedule)."""
+    import torch
+    from super_gnn_amd import synth, supergnn_ops as ops
+    dev, F = ctx["dev"], 602
+    n = args.sbm_nodes // 50 * 50
+    t0 = time.perf_counter()
+    rowptr, col = synth.sbm_graph(n, 50, 0.03048, 0.001524, seed=3, device=dev)
+    g = torch.Generator(device=dev); g.manual_seed(4)
+    x = torch.rand(n, F, generator=g, device=dev) * 2 - 1
+    torch.cuda.synchronize()
+    nnz = col.numel()
+    log(f"[bench] sbm: {n} nodes, {nnz} edges (avg degree {nnz / n:.0f}), built in {time.perf_counter() - t0:.1f}s")
+    plan = ops.SpmmPlan(rowptr, col, n, long_row_threshold=args.long_threshold, piece_edges=args.piece_edges)
+    info, sched = plan.info(), plan.schedule(F)
+    out = torch.zeros(n, F, device=dev)
+    ms, per_kernel, launches = profiled_steps(lambda: plan.run(None, x, out, accumulate=True), args.steps, args.warmup)
+    dom = max(per_kernel, key=per_kernel.get)
+    b_total = spmm_gather_bytes(nnz, n, F, weighted=False, accumulate=True, mean=False,
+                                empty_rows=int(((rowptr[1:] - rowptr[:-1]) == 0).sum()))
+    dom_edges = nnz if dom == "spmm_band_kernel" else info["long_edges"] if "piece" in dom else nnz - info["long_edges"]
+    dom_bytes = dom_edges * (4 * F + 4)
+    wl = f"sbm_{n}n_{nnz}e_F{F}_sum"
+    extra = {"kernel_ms_per_step": {k: round(v, 5) for k, v in per_kernel.items()},
+             "launches_per_step": {k: round(v, 2) for k, v in launches.items()}, "schedule": sched,
+             "plan": {k: info[k] for k in ("long_rows", "pieces", "long_edges")},
+             "gather_model_total": {"algorithmic_bytes": int(b_total), "GBps": round(b_total / ms / 1e6, 1),
+                                    "frac_of_peak": round(b_total / ms / 1e6 / HBM_PEAK_GBPS, 4)},
+             "compulsory_bytes": int(spmm_compulsory_bytes(nnz, n, n, F, False)), "step_roofline": step_roofline(wl, per_kernel)}
+    log(f"[bench] sbm sum: {ms:.3f} ms/step, {nnz / ms / 1e6:.2f} GEdges/s, schedule {sched}, kernels (ms per step) "
+        f"{ {k: round(v, 4) for k, v in per_kernel.items()} }")
+    return {"metric": "SpMM GEdges/s (dense-degree community graph, F=602 fp32)", "value": round(nnz / ms / 1e6, 4),
+            "unit": "GEdges/s", "config": {"workload": wl, "F": F}, "ms_per_step": ms, "dtype": "f32",
+            "roofline": roofline(wl, dom, per_kernel[dom], dom_bytes, launches[dom]), "cpu_baseline": None, "extra": extra}
+
+
+def wl_aggregate(args, ctx):
+    """One GraphSAGE-style aggregation (forward + backward) over P partitions of the headline graph."""
+    import torch
+    from super_gnn_amd.aggregator import LoopbackWorld
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    dev, F = ctx["dev"], args.feat
+    rowptr, col, w, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
+    t0 = time.perf_counter()
+    graphs = build_loopback_partitions(rowptr, col, w, args.parts, F, num_bits=args.exchange_bits,
+                                       is_pre_delay=bool(args.pre), device=dev)
+    log(f"[bench] {args.parts} partitions built in {time.perf_counter() - t0:.1f}s; rows exchanged per direction: "
+        f"{sum(sum(g.comm_splits.send_splits) for g in graphs)}")
+    world = LoopbackWorld(graphs, args.exchange_bits, bool(args.pre))
+    feats = [x[g.node_range[0]:g.node_range[1]].clone().requires_grad_() for g in graphs]
+    grads = [torch.randn(g.node_range[1] - g.node_range[0], F, device=dev) for g in graphs]
+
+    def step():
+        outs = world.aggregate(feats)
+        torch.autograd.backward(outs, grads)
+        for f in feats:
+            f.grad = None
+
+    ms = time_steps(step, args.steps, args.warmup)
+    ms_fwd = time_steps(lambda: world.aggregate([f.detach() for f in feats]), args.steps, args.warmup)
+    nnz = col.numel()
+    extra = {"forward_ms": round(ms_fwd, 4), "forward_backward_ms": round(ms, 4),
+             "rows_exchanged": sum(sum(g.comm_splits.send_splits) for g in graphs)}
+    log(f"[bench] aggregate fwd {ms_fwd:.3f} ms, fwd+bwd {ms:.3f} ms ({2 * nnz / ms / 1e6:.2f} GEdges/s)")
+    return {"metric": "aggregation layer GEdges/s (forward+backward, loop-back exchange)",
+            "value": round(2 * nnz / ms / 1e6, 4), "unit": "GEdges/s",
+            "config": {"workload": f"aggregate_rmat_{args.nodes}n_{nnz}e_F{F}_P{args.parts}_bits{args.exchange_bits}_pre{args.pre}"},
+            "ms_per_step": ms, "dtype": "f32", "roofline": None, "cpu_baseline": None, "extra": extra}
+
+
+def wl_sage(args, ctx):
+    """One training epoch of a 3-layer GraphSAGE over P partitions (examples/graphsage/sage.py:213-232)."""
+    import torch
+    from super_gnn_amd.aggregator import LoopbackWorld
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    from super_gnn_amd.layers import LoopbackSAGE
+    dev = ctx["dev"]
+    F, H, C = args.feat, args.hidden, args.classes
+    rowptr, col, _, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
+    graphs = build_loopback_partitions(rowptr, col, None, args.parts, max(F, H, C), num_bits=args.exchange_bits,
+                                       is_pre_delay=bool(args.pre), device=dev)
+    world = LoopbackWorld(graphs, args.exchange_bits, bool(args.pre),
+                          params_wire_dtype=torch.bfloat16 if args.exchange_bits in (2, 4, 8) else None)
+    torch.manual_seed(0)
+    model = LoopbackSAGE(F, H, C, num_layers=3, dropout=0.5).to(dev)
+    model.reset_parameters()
+    opt = torch.optim.Adam(model.parameters(), lr=0.01)
+    feats = [x[g.node_range[0]:g.node_range[1]] for g in graphs]
+    labels = torch.randint(0, C, (rowptr.numel() - 1,), device=dev)
+
+    def epoch():
+        model.train()
+        opt.zero_grad()
+        out = torch.cat(model(world, feats))
+        # nll_loss(out, labels) written as a gather: torch's nll_loss kernels reduce 2.45 M rows in a
+        # single workgroup (5 ms forward, 4 ms backward)
+        loss = -out.gather(1, labels.view(-1, 1)).mean()
+        loss.backward()
+        opt.step()
+
+    ms = time_steps(epoch, args.steps, args.warmup)
+    nnz = col.numel()
+    log(f"[bench] sage epoch {ms:.3f} ms (3 layers {F}-{H}-{H}-{C}, P={args.parts}, bits={args.exchange_bits}, pre={args.pre})")
+    return {"metric": "GraphSAGE training epoch time (3 layers, full graph, loop-back exchange)",
+            "value": round(1000.0 / ms, 4), "unit": "epochs/s",
+            "config": {"workload": f"sage_rmat_{args.nodes}n_{nnz}e_F{F}_H{H}_C{C}_P{args.parts}_bits{args.exchange_bits}_pre{args.pre}"},
+            "ms_per_step": ms, "dtype": "f32", "roofline": None, "cpu_baseline": None, "extra": {}}
+
+
+WORKLOADS = {"rmat": wl_rmat, "quant": wl_quant, "copy": wl_copy, "prepost": wl_prepost, "sbm": wl_sbm,
+             "aggregate": wl_aggregate, "sage": wl_sage, "small": wl_small}
+
+
+def brief(r):
+    """A workload's result as an entry of extra["workloads"]."""
+    return {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "config": r["config"],
+            "ms_per_step": round(r["ms_per_step"], 5), "roofline": r["roofline"], "cpu_baseline": r["cpu_baseline"],
+            "extra": r["extra"]}
 
 
 def main():
@@ -176,9 +654,10 @@ def main():
     ap.add_argument("--uniform-rows", type=int, default=0, help="diagnostic: replace the R-MAT graph by uniform random "
                     "rows of --uniform-degree neighbours over --nodes columns")
     ap.add_argument("--uniform-degree", type=int, default=25)
-    ap.add_argument("--workload", default="rmat", choices=["rmat", "quant", "copy", "prepost", "sbm", "aggregate", "sage", "small"],
+    ap.add_argument("--workload", default="rmat", choices=sorted(WORKLOADS),
                     help="rmat: headline SpMM (default); quant: int2 quantize+pack as the step; copy: streaming copy; "
-                         "prepost: one partition with packed remote rows, fused vs separate; sbm: dense-degree graph, F=602")
+                         "prepost: one partition with packed remote rows, fused vs separate; sbm: dense-degree graph, F=602; "
+                         "small: the CPU-runnable case; aggregate / sage: the aggregation layer and a GraphSAGE epoch")
     ap.add_argument("--local-nodes", type=int, default=8_000_000)
     ap.add_argument("--remote-nodes", type=int, default=2_000_000)
     ap.add_argument("--local-und-edges", type=int, default=160_000_000)
@@ -197,8 +676,8 @@ def main():
     ap.add_argument("--bits", type=int, default=2)
     ap.add_argument("--long-threshold", type=int, default=0, help="SpMM plan: rows longer than this are split (0 = default)")
     ap.add_argument("--piece-edges", type=int, default=0, help="SpMM plan: minimum edges per long-row piece (0 = default)")
-    ap.add_argument("--no-extras", action="store_true", help="skip the extra kernels (used under rocprofv3)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-extras", action="store_true", help="only the chosen workload (used under rocprofv3)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build runs one partition on ONE GPU; there is no multi-GPU path to time "
@@ -207,358 +686,34 @@ def main():
 
     import torch
     import super_gnn_amd  # noqa: F401  (raises if libsgnn_hip.so is missing)
-    from super_gnn_amd import _lib, synth, supergnn_ops as ops
+    from super_gnn_amd import supergnn_ops as ops
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    dev = torch.device("cuda:0")
-    stream = ops._stream
+    ctx = {"dev": torch.device("cuda:0"), "stream": ops._stream}
 
-    extra = {}
-    # ---- streaming copy yardstick --------------------------------------------------------------
-    n_copy = 256 * 1024 * 1024  # 1 GiB in + 1 GiB out
-    src = torch.empty(n_copy, device=dev).normal_()
-    dst = torch.empty_like(src)
-    copy_fn = lambda: _lib.check(_lib.lib.sgnn_stream_copy_f32(src.data_ptr(), dst.data_ptr(), n_copy, stream()))  # noqa: E731
-    if args.workload == "copy" or not args.no_extras:
-        ms = time_steps(copy_fn, 10, 3)
-        extra["stream_copy_GBps"] = round(2 * 4 * n_copy / ms / 1e6, 1)
-        log(f"[bench] stream copy: {extra['stream_copy_GBps']} GB/s (read+write)")
-
-    result = None
-    if args.workload == "copy":
-        _lib.profile_start()
-        ms = time_steps(copy_fn, args.steps, args.warmup)
-        prof = _lib.profile_stop()
-        n, tot = prof["stream_copy_kernel"]
-        ach = 2 * 4 * n_copy / (tot / n) / 1e6
-        result = {"metric": "stream copy GB/s", "value": round(2 * 4 * n_copy / ms / 1e6, 2), "unit": "GB/s",
-                  "config": {"workload": "stream_copy_1GiB"}, "ms_per_step": ms, "dtype": "f32",
-                  "roofline": {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                               "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": "stream_copy_kernel"},
-                  "cpu_baseline": None}
-    del src, dst
-
-    # ---- quantize / dequantize sweep -----------------------------------------------------------
-    if args.workload == "quant" or not args.no_extras:
-        n, F = args.quant_rows, args.quant_feat
-        xq = synth.boundary_features(n, F, seed=5, device=dev)
-        seg = torch.tensor([0, n], dtype=torch.int32)
-        d = torch.empty(n, F, device=dev)
-        for bits in (8, 4, 2):
-            if args.workload == "quant" and args.no_extras and bits != args.bits:
+    result = WORKLOADS[args.workload](args, ctx)
+    extra = result.pop("extra")
+    if not args.no_extras:
+        others = {}
+        saved = (args.steps, args.warmup)
+        args.steps, args.warmup = min(args.steps, 10), min(args.warmup, 3)
+        for name in ("copy", "quant", "sbm", "prepost", "small"):
+            if name == args.workload:
                 continue
-            epb = 8 // bits
-            q = torch.empty((n + epb - 1) // epb, F, dtype=torch.uint8, device=dev)
-            p = torch.empty(n, 2, device=dev)
-            qf = lambda: ops.quantize_tensor_for_all_procs(xq, q, p, seg, 1, bits)  # noqa: E731
-            df = lambda: ops.dequantize_tensor_for_all_procs(q, d, p, seg, 1, bits)  # noqa: E731
-            is_main = args.workload == "quant" and bits == args.bits
-            st, wu = (args.steps, args.warmup) if is_main else (10, 3)
-            _lib.profile_start()
-            ms_q = time_steps(qf, st, wu)
-            prof = _lib.profile_stop()
-            ms_d = time_steps(df, 10, 3)
-            b = quant_bytes(n, F, bits)
-            extra[f"quant_pack_int{bits}_GBps"] = round(b / ms_q / 1e6, 1)
-            extra[f"unpack_dequant_int{bits}_GBps"] = round(b / ms_d / 1e6, 1)
-            log(f"[bench] int{bits}: quantize+pack {b / ms_q / 1e6:.0f} GB/s ({ms_q:.3f} ms), "
-                f"unpack+dequant {b / ms_d / 1e6:.0f} GB/s ({ms_d:.3f} ms)")
-            if is_main:
-                nl, tot = prof["quant_pack_rows_kernel"]
-                ach = b / (tot / nl) / 1e6
-                wl = f"quant_pack_int{bits}_{n}x{F}"
-                result = {"metric": f"quantize-pack GB/s at int{bits}", "value": round(b / ms_q / 1e6, 2),
-                          "unit": "GB/s", "config": {"workload": wl, "rows": n, "F": F, "bits": bits},
-                          "ms_per_step": ms_q, "dtype": "f32->u8",
-                          "roofline": {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS,
-                                       "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBPS, 4),
-                                       "traffic": MEASURED_TRAFFIC_BYTES.get(wl), "kernel": "quant_pack_rows_kernel",
-                                       "kernel_avg_ms": round(tot / nl, 5), "algorithmic_bytes": b},
-                          "cpu_baseline": None if args.no_cpu else cpu_baseline_quant(xq, bits)}
-        if not args.no_cpu and args.workload != "quant":
-            extra["cpu_quant_pack_int2"] = cpu_baseline_quant(xq, 2)
-        del xq, d
-
-    # ---- headline SpMM -------------------------------------------------------------------------
-    if args.workload == "rmat":
-        F = args.feat
-        if args.uniform_rows:
-            g = torch.Generator(device=dev); g.manual_seed(11)
-            M, dg = args.uniform_rows, args.uniform_degree
-            col = torch.sort(torch.randint(0, args.nodes, (M, dg), generator=g, device=dev), dim=1).values
-            col = col.reshape(-1).to(torch.int32).contiguous()
-            rowptr = torch.arange(M + 1, device=dev, dtype=torch.int64) * dg
-            w = torch.rand(col.numel(), generator=g, device=dev)
-            x = torch.randn(args.nodes, F, generator=g, device=dev)
-        else:
-            rowptr, col, w, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
-        M, nnz = rowptr.numel() - 1, col.numel()
-        t0 = time.perf_counter()
-        plan = ops.SpmmPlan(rowptr, col, x.shape[0], long_row_threshold=args.long_threshold, piece_edges=args.piece_edges)
-        torch.cuda.synchronize()
-        info = plan.info()
-        extra["plan_build_ms"] = round((time.perf_counter() - t0) * 1e3, 1)
-        extra["plan"] = {k: info[k] for k in ("long_rows", "pieces", "long_edges", "long_row_threshold", "piece_edges", "partitioned")}
-        log(f"[bench] plan: {extra['plan']} built in {extra['plan_build_ms']} ms")
-        out = torch.zeros(M, F, device=dev)
-        step = lambda: plan.run(w, x, out, accumulate=True)  # noqa: E731
-        _lib.profile_start()
-        ms = time_steps(step, args.steps, args.warmup)
-        prof = _lib.profile_stop()
-        per_kernel = {k: round(v[1] / v[0], 5) for k, v in prof.items()}
-        log(f"[bench] weighted sum: {ms:.3f} ms/step, {nnz / ms / 1e6:.2f} GEdges/s, kernels (avg ms) {per_kernel}")
-        # dominant kernel: the short-row kernel; its share of the algorithmic bytes
-        short_edges = nnz - info["long_edges"]
-        short_rows = M - info["long_rows"]
-        n_empty = int(((rowptr[1:] - rowptr[:-1]) == 0).sum())
-        b_short = spmm_gather_bytes(short_edges, short_rows, F, weighted=True, accumulate=True, mean=False, empty_rows=n_empty)
-        b_total = spmm_gather_bytes(nnz, M, F, weighted=True, accumulate=True, mean=False, empty_rows=n_empty)
-        extra["empty_rows"] = n_empty
-        dom = max(prof, key=lambda k: prof[k][1])
-        dom_ms = prof[dom][1] / prof[dom][0]
-        if dom == "spmm_short_kernel":
-            dom_bytes = b_short
-        elif dom == "spmm_piece_kernel":
-            # per edge: dense row + col + val (the per-unit figure of the gather model); the kernel's own
-            # bookkeeping (edge permutation, piece partial sums) is overhead, not algorithmic traffic
-            dom_bytes = info["long_edges"] * (4 * F + 8)
-        else:
-            dom_bytes = b_total
-        ach = dom_bytes / dom_ms / 1e6
-        wl = f"rmat_{M}n_{nnz}e_F{F}_gcn_weighted_sum" if not args.uniform_rows else f"uniform_{M}x{args.nodes}_deg{args.uniform_degree}_F{F}"
-        # mean aggregation (unit weights + fused /deg) as an extra
-        if not args.no_extras:
-            deg = (rowptr[1:] - rowptr[:-1]).clamp(min=1).to(torch.float32)
-            out2 = torch.zeros(M, F, device=dev)
-            ms_mean = time_steps(lambda: plan.run(None, x, out2, accumulate=True, row_div=deg), 10, 3)
-            extra["spmm_mean_GEdges_per_s"] = round(nnz / ms_mean / 1e6, 3)
-            extra["spmm_mean_gather_GBps"] = round(spmm_gather_bytes(nnz, M, F, False, True, True, empty_rows=n_empty) / ms_mean / 1e6, 1)
-            del out2
-        if not args.no_extras:
-            scratch = torch.empty(192 * 1024 * 1024, device=dev)   # 768 MB > 8 x 4 MB L2 + 256 MB Infinity Cache
-            extra["spmm_warm"] = time_reps_events(step, 20, 5)
-            extra["spmm_cache_flushed"] = time_reps_events(step, 20, 2, flush=lambda: scratch.fill_(1.0))
-            log(f"[bench] weighted sum per repetition: warm {extra['spmm_warm']}, caches flushed before each {extra['spmm_cache_flushed']}")
-            del scratch
-        # one-time preparation, like the plan itself: the unchanged weight tensor was bound during warm-up
-        extra["edge_values_bound_to_plan"] = plan._bound is not None
-        extra["spmm_total_gather_GBps"] = round(b_total / ms / 1e6, 1)
-        extra["spmm_total_frac_of_hbm_peak"] = round(b_total / ms / 1e6 / HBM_PEAK_GBPS, 4)
-        extra["spmm_GFLOPs"] = round(2.0 * nnz * F / ms / 1e6, 1)
-        extra["kernel_avg_ms"] = per_kernel
-        result = {"metric": "SpMM GEdges/s + % HBM roofline (F=128 fp32); quantize-pack GB/s at int2",
-                  "value": round(nnz / ms / 1e6, 4), "unit": "GEdges/s",
-                  "config": {"workload": wl, "nodes": M, "edges": nnz, "F": F, "aggregation": "weighted_sum",
-                             "accumulate": True, "index_dtype": "int32"},
-                  "ms_per_step": ms, "dtype": "f32",
-                  "roofline": {"bound": "hbm", "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                               "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(wl),
-                               "kernel": dom, "kernel_avg_ms": round(dom_ms, 5), "algorithmic_bytes": int(dom_bytes)},
-                  "cpu_baseline": None if args.no_cpu else cpu_baseline_spmm(rowptr, col, w, x)}
-
-    # ---- the small CPU-runnable configuration: cache-resident, so GEdges/s only -----------------
-    if args.workload == "small":
-        N, F = 10_000, 128
-        g = torch.Generator().manual_seed(0)
-        col = torch.randint(0, N, (N, 16), generator=g)
-        col = torch.sort(torch.cat([col, torch.arange(N).unsqueeze(1)], dim=1), dim=1).values.reshape(-1)
-        rowptr = 17 * torch.arange(N + 1, dtype=torch.int64)
-        x = torch.randn(N, F, generator=g)
-        w = torch.ones(col.numel())
-        d_rowptr, d_col, d_w, d_x = rowptr.to(dev), col.to(torch.int32).to(dev), w.to(dev), x.to(dev)
-        plan = ops.SpmmPlan(d_rowptr, d_col, N)
-        out = torch.zeros(N, F, device=dev)
-        step = lambda: plan.run(d_w, d_x, out, accumulate=True)  # noqa: E731
-        _lib.profile_start()
-        ms = time_steps(step, args.steps, args.warmup)
-        prof = _lib.profile_stop()
-        k_ms = prof["spmm_short_kernel"][1] / prof["spmm_short_kernel"][0]
-        nnz = col.numel()
-        b = spmm_gather_bytes(nnz, N, F, weighted=True, accumulate=True, mean=False)
-        xq = torch.randn(2000, F, generator=g).to(dev)
-        q = torch.empty(2000, F, dtype=torch.uint8, device=dev); pq = torch.empty(2000, 2, device=dev)
-        seg1 = torch.tensor([0, 2000], dtype=torch.int32)
-        ms_q = time_steps(lambda: ops.quantize_tensor_for_all_procs(xq, q, pq, seg1, 1, 8), 50, 10)
-        cpu = None
-        if not args.no_cpu:
-            cpu = cpu_baseline_spmm(rowptr, col, w, x, reps=20)
-            nt = torch.get_num_threads()
-            torch.set_num_threads(1); os.environ["OMP_NUM_THREADS"] = "1"
-            cpu1 = cpu_baseline_spmm(rowptr, col, w, x, reps=5)
-            torch.set_num_threads(nt)
-            extra["cpu_1_thread_GEdges_per_s"] = round(cpu1["value"], 4)
-        extra.update({"kernel_ms": round(k_ms, 5), "kernel_GEdges_per_s": round(nnz / k_ms / 1e6, 2),
-                      "kernel_gather_GBps_cache_resident": round(b / k_ms / 1e6, 1),
-                      "quant_int8_2000x128_us_per_call": round(ms_q * 1e3, 2)})
-        log(f"[bench] small: {ms * 1e3:.1f} us/step wall, kernel {k_ms * 1e3:.1f} us = {nnz / k_ms / 1e6:.1f} GEdges/s; int8 quantize 2000x128 {ms_q * 1e3:.1f} us/call")
-        result = {"metric": "SpMM GEdges/s (10k nodes x 17 edges, F=128, cache-resident)", "value": round(nnz / ms / 1e6, 4),
-                  "unit": "GEdges/s", "config": {"workload": f"small_uniform_{N}n_{nnz}e_F{F}_sum"}, "ms_per_step": ms,
-                  "dtype": "f32", "roofline": None, "cpu_baseline": cpu}
-
-    # ---- one partition in pre/post-aggregation mode: remote rows arrive int2-packed -------------
-    if args.workload == "prepost":
-        F, bits = args.feat, args.bits
-        Ml, Kr = args.local_nodes, args.remote_nodes
-        t0 = time.perf_counter()
-        rp_l, col_l = synth.rmat_graph(Ml, args.local_und_edges, seed=6, device=dev)
-        g = torch.Generator(device=dev); g.manual_seed(7)
-        # remote edges: rows follow the local degree distribution, columns uniform over the boundary set
-        deg_l = (rp_l[1:] - rp_l[:-1]).to(torch.float32)
-        rows_r = torch.multinomial(deg_l + 0.05, args.remote_edges, replacement=True, generator=g)
-        cols_r = torch.randint(0, Kr, (args.remote_edges,), generator=g, device=dev)
-        rp_r, col_r = synth.csr_from_pairs(rows_r, cols_r, Ml, Kr, dedupe=True)
-        del rows_r, cols_r, deg_l
-        x_l = torch.randn(Ml, F, generator=g, device=dev)
-        x_r = torch.randn(Kr, F, generator=g, device=dev)
-        torch.cuda.synchronize()
-        log(f"[bench] prepost: local {Ml} rows / {col_l.numel()} edges, remote {Kr} cols / {col_r.numel()} edges, "
-            f"built in {time.perf_counter() - t0:.1f}s")
-        P = 8
-        wr = torch.tensor([Kr * i // P for i in range(P + 1)], dtype=torch.int32)
-        epb = 8 // bits
-        npk = sum((int(wr[i + 1] - wr[i]) + epb - 1) // epb for i in range(P))
-        q = torch.empty(npk, F, dtype=torch.uint8, device=dev)
-        prm = torch.empty(Kr, 2, device=dev)
-        ops.quantize_tensor_for_all_procs(x_r, q, prm, wr, P, bits)
-        del x_r
-        plan_l = ops.SpmmPlan(rp_l, col_l, Ml)
-        plan_r = ops.SpmmPlan(rp_r, col_r, Kr)
-        segs = ops.quant_segments(wr, bits)
-        out = torch.zeros(Ml, F, device=dev)
-        recv = torch.empty(Kr, F, device=dev)
-        ms_local = time_steps(lambda: plan_l.run(None, x_l, out, accumulate=True), args.steps, args.warmup)
-
-        def separate():
-            ops.dequantize_tensor_for_all_procs(q, recv, prm, wr, P, bits)
-            plan_r.run(None, recv, out, accumulate=True)
-
-        ms_sep = time_steps(separate, args.steps, args.warmup)
-        _lib.profile_start()
-        ms_fused = time_steps(lambda: plan_r.run_quantized(None, q, prm, segs, bits, out, accumulate=True), args.steps, args.warmup)
-        prof = _lib.profile_stop()
-        nl, nr = col_l.numel(), col_r.numel()
-        per_kernel = {k: round(v[1] / v[0], 5) for k, v in prof.items()}
-        dom = max(prof, key=lambda k: prof[k][1])
-        info_r = plan_r.info()
-        dom_edges = info_r["long_edges"] if "piece" in dom else nr - info_r["long_edges"]
-        dom_bytes = dom_edges * (F + 16)  # survey figure for a remote edge: one packed row of F bytes + params + col/val
-        dom_ms = prof[dom][1] / prof[dom][0]
-        extra.update({"local_spmm_ms": round(ms_local, 4), "remote_separate_ms": round(ms_sep, 4),
-                      "remote_fused_ms": round(ms_fused, 4), "fused_speedup_on_remote_step": round(ms_sep / ms_fused, 3),
-                      "local_GEdges_per_s": round(nl / ms_local / 1e6, 3), "kernel_avg_ms": per_kernel})
-        log(f"[bench] local SpMM {ms_local:.3f} ms; remote: separate {ms_sep:.3f} ms vs fused {ms_fused:.3f} ms")
-        total = ms_local + ms_fused
-        result = {"metric": "SpMM GEdges/s, pre/post-aggregation partition (local fp32 + int2-packed remote rows, fused)",
-                  "value": round((nl + nr) / total / 1e6, 4), "unit": "GEdges/s",
-                  "config": {"workload": f"prepost_{Ml}n_{nl}e_local_{Kr}c_{nr}e_remote_int{bits}_F{F}", "F": F, "bits": bits},
-                  "ms_per_step": total, "dtype": "f32",
-                  "roofline": {"bound": "hbm", "achieved": round(dom_bytes / dom_ms / 1e6, 1), "peak": HBM_PEAK_GBPS,
-                               "unit": "GB/s", "frac": round(dom_bytes / dom_ms / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None,
-                               "kernel": dom, "kernel_avg_ms": round(dom_ms, 5), "algorithmic_bytes": int(dom_bytes)},
-                  "cpu_baseline": None}
-
-    # ---- dense-degree community graph, wide odd feature rows --------------------------------------
-    if args.workload == "sbm":
-        F = 602
-        n = args.sbm_nodes // 50 * 50
-        t0 = time.perf_counter()
-        rowptr, col = synth.sbm_graph(n, 50, 0.03048, 0.001524, seed=3, device=dev)
-        g = torch.Generator(device=dev); g.manual_seed(4)
-        x = torch.rand(n, F, generator=g, device=dev) * 2 - 1
-        torch.cuda.synchronize()
-        nnz = col.numel()
-        log(f"[bench] sbm: {n} nodes, {nnz} edges (avg degree {nnz / n:.0f}), built in {time.perf_counter() - t0:.1f}s")
-        plan = ops.SpmmPlan(rowptr, col, n, long_row_threshold=args.long_threshold, piece_edges=args.piece_edges)
-        info = plan.info()
-        out = torch.zeros(n, F, device=dev)
-        _lib.profile_start()
-        ms = time_steps(lambda: plan.run(None, x, out, accumulate=True), args.steps, args.warmup)
-        prof = _lib.profile_stop()
-        per_kernel = {k: round(v[1] / v[0], 5) for k, v in prof.items()}
-        dom = max(prof, key=lambda k: prof[k][1])
-        dom_ms = prof[dom][1] / prof[dom][0]
-        dom_edges = info["long_edges"] if "piece" in dom else nnz - info["long_edges"]
-        dom_bytes = dom_edges * (4 * F + 4)
-        b_total = spmm_gather_bytes(nnz, n, F, weighted=False, accumulate=True, mean=False,
-                                    empty_rows=int(((rowptr[1:] - rowptr[:-1]) == 0).sum()))
-        extra.update({"kernel_avg_ms": per_kernel, "plan": {k: info[k] for k in ("long_rows", "pieces", "long_edges")},
-                      "spmm_total_gather_GBps": round(b_total / ms / 1e6, 1)})
-        log(f"[bench] sbm sum: {ms:.3f} ms/step, {nnz / ms / 1e6:.2f} GEdges/s, {b_total / ms / 1e6:.0f} GB/s gather model, {per_kernel}")
-        result = {"metric": "SpMM GEdges/s (dense-degree community graph, F=602 fp32)", "value": round(nnz / ms / 1e6, 4),
-                  "unit": "GEdges/s", "config": {"workload": f"sbm_{n}n_{nnz}e_F{F}_sum", "F": F}, "ms_per_step": ms,
-                  "dtype": "f32",
-                  "roofline": {"bound": "hbm", "achieved": round(dom_bytes / dom_ms / 1e6, 1), "peak": HBM_PEAK_GBPS,
-                               "unit": "GB/s", "frac": round(dom_bytes / dom_ms / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None,
-                               "kernel": dom, "kernel_avg_ms": round(dom_ms, 5), "algorithmic_bytes": int(dom_bytes)},
-                  "cpu_baseline": None}
-
-    # ---- one GraphSAGE-style aggregation (forward + backward) over P partitions of the headline graph ----
-    if args.workload == "aggregate":
-        from super_gnn_amd.aggregator import LoopbackWorld
-        from super_gnn_amd.data_manager import build_loopback_partitions
-        F = args.feat
-        rowptr, col, w, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
-        t0 = time.perf_counter()
-        graphs = build_loopback_partitions(rowptr, col, w, args.parts, F, num_bits=args.exchange_bits,
-                                           is_pre_delay=bool(args.pre), device=dev)
-        log(f"[bench] {args.parts} partitions built in {time.perf_counter() - t0:.1f}s; rows exchanged per direction: "
-            f"{sum(sum(g.comm_splits.send_splits) for g in graphs)}")
-        world = LoopbackWorld(graphs, args.exchange_bits, bool(args.pre))
-        feats = [x[g.node_range[0]:g.node_range[1]].clone().requires_grad_() for g in graphs]
-        grads = [torch.randn(g.node_range[1] - g.node_range[0], F, device=dev) for g in graphs]
-
-        def step():
-            outs = world.aggregate(feats)
-            torch.autograd.backward(outs, grads)
-            for f in feats:
-                f.grad = None
-
-        ms = time_steps(step, args.steps, args.warmup)
-        ms_fwd = time_steps(lambda: world.aggregate([f.detach() for f in feats]), args.steps, args.warmup)
-        nnz = col.numel()
-        extra.update({"forward_ms": round(ms_fwd, 4), "forward_backward_ms": round(ms, 4),
-                      "rows_exchanged": sum(sum(g.comm_splits.send_splits) for g in graphs)})
-        log(f"[bench] aggregate fwd {ms_fwd:.3f} ms, fwd+bwd {ms:.3f} ms ({2 * nnz / ms / 1e6:.2f} GEdges/s)")
-        result = {"metric": "aggregation layer GEdges/s (forward+backward, loop-back exchange)",
-                  "value": round(2 * nnz / ms / 1e6, 4), "unit": "GEdges/s",
-                  "config": {"workload": f"aggregate_rmat_{args.nodes}n_{nnz}e_F{F}_P{args.parts}_bits{args.exchange_bits}_pre{args.pre}"},
-                  "ms_per_step": ms, "dtype": "f32", "roofline": None, "cpu_baseline": None}
-
-    # ---- one training epoch of a 3-layer GraphSAGE over P partitions (examples/graphsage/sage.py:213-232) ----
-    if args.workload == "sage":
-        from super_gnn_amd.aggregator import LoopbackWorld
-        from super_gnn_amd.data_manager import build_loopback_partitions
-        from super_gnn_amd.layers import LoopbackSAGE
-        F, H, C = args.feat, args.hidden, args.classes
-        rowptr, col, _, x = build_headline_graph(args.nodes, args.und_edges, F, dev)
-        graphs = build_loopback_partitions(rowptr, col, None, args.parts, max(F, H, C), num_bits=args.exchange_bits,
-                                           is_pre_delay=bool(args.pre), device=dev)
-        world = LoopbackWorld(graphs, args.exchange_bits, bool(args.pre),
-                              params_wire_dtype=torch.bfloat16 if args.exchange_bits in (2, 4, 8) else None)
-        torch.manual_seed(0)
-        model = LoopbackSAGE(F, H, C, num_layers=3, dropout=0.5).to(dev)
-        model.reset_parameters()
-        opt = torch.optim.Adam(model.parameters(), lr=0.01)
-        feats = [x[g.node_range[0]:g.node_range[1]] for g in graphs]
-        labels = torch.randint(0, C, (rowptr.numel() - 1,), device=dev)
-
-        def epoch():
-            model.train()
-            opt.zero_grad()
-            out = torch.cat(model(world, feats))
-            # nll_loss(out, labels) written as a gather: torch's nll_loss kernels reduce 2.45 M rows in a
-            # single workgroup (5 ms forward, 4 ms backward)
-            loss = -out.gather(1, labels.view(-1, 1)).mean()
-            loss.backward()
-            opt.step()
-
-        ms = time_steps(epoch, args.steps, args.warmup)
-        nnz = col.numel()
-        log(f"[bench] sage epoch {ms:.3f} ms (3 layers {F}-{H}-{H}-{C}, P={args.parts}, bits={args.exchange_bits}, pre={args.pre})")
-        result = {"metric": "GraphSAGE training epoch time (3 layers, full graph, loop-back exchange)",
-                  "value": round(1000.0 / ms, 4), "unit": "epochs/s",
-                  "config": {"workload": f"sage_rmat_{args.nodes}n_{nnz}e_F{F}_H{H}_C{C}_P{args.parts}_bits{args.exchange_bits}_pre{args.pre}"},
-                  "ms_per_step": ms, "dtype": "f32", "roofline": None, "cpu_baseline": None}
+            torch.cuda.empty_cache()
+            t0 = time.perf_counter()
+            cpu_saved = args.no_cpu
+            args.no_cpu = args.no_cpu or name in ("sbm", "prepost")
+            others[name] = brief(WORKLOADS[name](args, ctx))
+            if name == "quant":   # the narrow rows the live path exchanges (F = 128), twice the rows for the same bytes
+                torch.cuda.empty_cache()
+                others["quant_F128"] = brief(wl_quant(args, ctx, rows=2 * args.quant_rows, feat=128, headline=False))
+            args.no_cpu = cpu_saved
+            log(f"[bench] extra workload {name}: {time.perf_counter() - t0:.1f}s")
+        args.steps, args.warmup = saved
+        extra["workloads"] = others
+        if "copy" in others:
+            extra["stream_copy_GBps"] = others["copy"]["value"]
 
     line = {"metric": result["metric"], "value": result["value"], "unit": result["unit"], "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(result["ms_per_step"], 5),

@@ -62,7 +62,7 @@ typedef struct sgnn_spmm_plan sgnn_spmm_plan;
  * Every col must lie in [0, K) and rowptr must be non-decreasing with rowptr[0] == 0: both are
  * checked (SGNN_ERR_RANGE).
  * long_row_threshold: rows with more edges take the long-row path (<= 0: default 128).
- * piece_edges: minimum edges per long-row piece (<= 0: default 32).
+ * piece_edges: minimum edges per long-row piece (<= 0: default 96).
  * Synchronises the stream (the work lists are built on the host). */
 int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int col_is_i64, int64_t M,
                           int64_t K, int64_t nnz, int long_row_threshold, int piece_edges,

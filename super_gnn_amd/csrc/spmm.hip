@@ -35,7 +35,7 @@ namespace sgnn {
 constexpr int kBlock = 256;
 constexpr int kDefaultLongThreshold = 128;  // rows with more edges go to the class-partitioned piece path
 constexpr int kChunkGroupsWanted = 16384;
-constexpr int kDefaultPieceEdges = 32;      // minimum edges per piece of a long row
+constexpr int kDefaultPieceEdges = 96;      // minimum edges per piece of a long row (a class run shorter than this stays one piece)
 constexpr int kPopularColumns = 16384;      // size of the "popular" column set the plan looks at
 constexpr double kPartitionMinShare = 0.02; // below this share of all edges (popularity ~uniform) leave the long rows as they are
 
