@@ -512,7 +512,8 @@ def wl_prepost(args, ctx):
     dom_edges = info_r["long_edges"] if "piece" in dom else nr - info_r["long_edges"]
     dom_bytes = dom_edges * (F + 16)  # per remote edge: one packed row of F bytes + params + col/val
     total = ms_local + ms_fused
-    wl = f"prepost_{Ml}n_{nl}e_local_{Kr}c_{nr}e_remote_int{bits}_F{F}"
+    # named by the requested sizes: the de-duplicated remote edge count varies by a few edges from run to run
+    wl = f"prepost_{Ml}n_{args.local_und_edges}ue_local_{Kr}c_{args.remote_edges}e_remote_int{bits}_F{F}"
     extra = {"local_spmm_ms": round(ms_local, 4), "remote_separate_ms": round(ms_sep, 4),
              "remote_fused_ms": round(ms_fused, 4), "fused_speedup_on_remote_step": round(ms_sep / ms_fused, 3),
              "local_GEdges_per_s": round(nl / ms_local / 1e6, 3),
@@ -522,7 +523,7 @@ def wl_prepost(args, ctx):
     log(f"[bench] prepost: local SpMM {ms_local:.3f} ms; remote: separate {ms_sep:.3f} ms vs fused {ms_fused:.3f} ms")
     return {"metric": "SpMM GEdges/s, pre/post-aggregation partition (local fp32 + int2-packed remote rows, fused)",
             "value": round((nl + nr) / total / 1e6, 4), "unit": "GEdges/s",
-            "config": {"workload": wl, "F": F, "bits": bits}, "ms_per_step": total, "dtype": "f32",
+            "config": {"workload": wl, "F": F, "bits": bits, "local_edges": nl, "remote_edges": nr}, "ms_per_step": total, "dtype": "f32",
             "roofline": roofline(wl, dom, k_fused[dom], dom_bytes, launches[dom]), "cpu_baseline": None, "extra": extra}
 
 

@@ -399,13 +399,17 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
         if (l16 == 0) store_params(pb, row[rl], mn, s);
     }
 
-    // Codes.  The reference's code is RNE(RN((x - zp) / scale)).  The quotient is first formed as
-    // (x - zp) * rcp(scale) with the 1-ulp hardware reciprocal: the product is within 1.5 * 2^-23
-    // relative of the true quotient and the IEEE quotient within 2^-24, both are below 256, so the two
-    // differ by less than 2^-13.  If the product is further than 2^-13 from every half-integer,
-    // rounding it gives the same integer as rounding the IEEE quotient; a lane that sees an element
-    // inside that guard band (about 1 in 4000), or a scale whose reciprocal is not a normal number,
-    // redoes its elements with the IEEE division.  The stored bytes are always the exact formula's.
+    // Codes.  The reference's code is RNE(RN(d / scale)) with d = RN(x - zp).  The quotient is first formed
+    // as RN(d * r) with r the hardware reciprocal of the scale (within 1 ulp of 1/scale): d * r differs from
+    // d / scale by at most 2^-23 relative, and each of the two roundings adds 2^-24, so the product and the
+    // IEEE quotient differ by less than 2^-22 relative -- in absolute terms less than qmax * 2^-22, since
+    // neither exceeds qmax = 2^bits - 1 by more than a rounding: 2^-14 at int8, 2^-18.1 at int4, 2^-20.4 at
+    // int2.  If the product is further than kGuard (twice that bound or more) from every half-integer,
+    // rounding it gives the same integer as rounding the IEEE quotient; a lane that sees an element inside
+    // the guard band (1 element in 4000 at int8, 1 in 33 000 at int4, 1 in 130 000 at int2), or a scale whose
+    // reciprocal is not a normal number, redoes its elements with the IEEE division.  The stored bytes are
+    // always the exact formula's.
+    constexpr float kGuard = BITS == 8 ? 0x1p-13f : BITS == 4 ? 0x1p-17f : 0x1p-19f;
     const int shift = (EPB - 1 - (d % EPB)) * BITS;
     uint32_t words[RL][NV];
 #pragma unroll
@@ -418,8 +422,10 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
                 for (int e = 0; e < VEC; ++e) {
                     const float qf = (xv[rl][v][e] - zp[rl]) * rinv[rl];
                     const float ri = rintf(qf);
-                    if (!(fabsf(qf - ri) < 0.5f - 0x1p-13f)) lane_exact = true;
-                    word |= (uint32_t)ri << (8 * e);
+                    if (!(fabsf(qf - ri) < 0.5f - kGuard)) lane_exact = true;  // also true for a NaN quotient
+                    // ri is an integer in [0, 255] whenever the lane stays on this path: one instruction
+                    // converts it and drops it into byte e of the word
+                    word = __builtin_amdgcn_cvt_pk_u8_f32(ri, e, word);
                 }
             }
             words[rl][v] = word;

@@ -266,8 +266,9 @@ def test_full_size_properties(bits):
     assert np.all(np.abs(d.cpu().numpy() - d_ref) <= dequant_atol(p_ref[:, 0], p_ref[:, 1], bits)[:, None])
 
 
+@pytest.mark.parametrize("F", [256, 128, 64])
 @pytest.mark.parametrize("bits", [8, 4, 2])
-def test_fast_quotient_equals_ieee_division(bits):
+def test_fast_quotient_equals_ieee_division(bits, F):
     """The kernel forms (x-zp)*RN(1/scale) and falls back to the IEEE division near half-integers;
     its bytes must equal those of the all-IEEE variant (SGNN_QUANT_EXACT_DIV=1) on the full-size
     input and on rows built to sit on rounding ties."""
@@ -276,13 +277,16 @@ def test_fast_quotient_equals_ieee_division(bits):
     ops = _ops()
     qmax = (1 << bits) - 1
     g = torch.Generator(device="cuda"); g.manual_seed(bits)
-    n, F = 1_000_000, 256
+    n = 256_000_000 // F
     x = synth.boundary_features(n, F, seed=5, device="cuda")
     # adversarial block: min 0, max qmax*s, values at (k + 0.5 +- tiny) * s for assorted scales s
     na = 4096
     s = torch.rand(na, 1, generator=g, device="cuda") * 3 + 0.01
     k = torch.randint(0, qmax, (na, F), generator=g, device="cuda").float()
+    # quotients a few ulps either side of the tie, and -- for the narrower guard bands of int4 / int2 -- up to
+    # and beyond the edge of the band (2^-13, 2^-17, 2^-19 absolute)
     eps = (torch.randint(-3, 4, (na, F), generator=g, device="cuda").float()) * 2.0 ** -22
+    eps[na // 2:] *= 2.0 ** torch.randint(0, 8, (na - na // 2, F), generator=g, device="cuda").float()
     adv = (k + 0.5) * (1 + eps) * s
     adv[:, 0] = 0.0
     adv[:, 1] = qmax * s[:, 0]
