@@ -39,17 +39,29 @@ class CommSplits(object):
 
 
 class CommBuffer(object):
-    """fp32 message buffers [sum(splits), F] (super_gnn/data_manager/CommBuffer.py:5-27)."""
+    """fp32 message buffers [sum(splits), F], plus bf16 copies of them in the 16-bit exchange mode (the
+    reference's attribute names say fp16, the dtype is bfloat16: super_gnn/data_manager/CommBuffer.py:5-27)."""
 
     def __init__(self, comm_splits: CommSplits, feat_len: int, bits: int, device="cuda") -> None:
         self.send_buf = torch.zeros((sum(comm_splits.send_splits), feat_len), dtype=torch.float32, device=device)
         self.recv_buf = torch.zeros((sum(comm_splits.recv_splits), feat_len), dtype=torch.float32, device=device)
+        self.send_buf_fp16 = None
+        self.recv_buf_fp16 = None
+        if bits == 16:
+            self.send_buf_fp16 = torch.zeros_like(self.send_buf, dtype=torch.bfloat16)
+            self.recv_buf_fp16 = torch.zeros_like(self.recv_buf, dtype=torch.bfloat16)
 
     def resize_buffer(self, comm_splits: CommSplits, feat_len: int, bits: int) -> None:
-        for name, n in (("send_buf", sum(comm_splits.send_splits)), ("recv_buf", sum(comm_splits.recv_splits))):
+        sizes = (("send_buf", sum(comm_splits.send_splits)), ("recv_buf", sum(comm_splits.recv_splits)))
+        for name, n in sizes:
             buf = getattr(self, name)
             if tuple(buf.shape) != (n, feat_len):
                 setattr(self, name, torch.zeros((n, feat_len), dtype=torch.float32, device=buf.device))
+        if bits == 16 and self.send_buf_fp16 is not None and self.recv_buf_fp16 is not None:
+            for name, n in sizes:
+                buf = getattr(self, name + "_fp16")
+                if tuple(buf.shape) != (n, feat_len):
+                    setattr(self, name + "_fp16", torch.zeros((n, feat_len), dtype=torch.bfloat16, device=buf.device))
 
 
 class CommBufferForQuantization(object):

@@ -12,7 +12,7 @@ import torch.nn.functional as F
 from torch import Tensor
 from torch.nn import LayerNorm, Linear, Parameter
 
-from .aggregator import LoopbackWorld
+from .aggregator import Aggregator, LoopbackWorld
 
 
 def _column_sum(g: Tensor) -> Tensor:
@@ -130,3 +130,72 @@ class LoopbackSAGE(torch.nn.Module):
             feats = [F.relu(x) for x in feats]
         feats = self.convs[-1](world, feats)
         return [F.log_softmax(x, dim=1) for x in feats]
+
+
+class DistSAGEConvGrad(torch.nn.Module):
+    """The reference's layer with the reference's constructor and call signatures
+    (super_gnn/layers/sageconv.py:15-89): ``conv(graph, local_nodes_feat, layer)`` aggregates through
+    ``Aggregator.apply(graph, feat, layer, num_bits, is_pre_delay, self.training)``, divides by
+    ``graph.in_degrees`` and returns ``lin_neigh(agg) + lin_self(feat) + bias``.  ``graph`` is whatever
+    ``Aggregator`` accepts: a partition that is the whole graph, or a LoopbackWorld of P partitions with the
+    node features of all of them stacked in partition order."""
+
+    def __init__(self, in_channels: int, out_channels: int, num_bits: int, is_pre_delay: bool,
+                 add_self_loops: bool = False, normalize: bool = True, bias: bool = True, **kwargs):
+        super().__init__()
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.add_self_loops, self.normalize = add_self_loops, normalize
+        self.num_bits, self.is_pre_delay = num_bits, is_pre_delay
+        self.lin_neigh = Linear(in_channels, out_channels, bias=False)
+        self.lin_self = Linear(in_channels, out_channels, bias=False)
+        if bias:
+            self.bias = Parameter(torch.zeros(out_channels))
+        else:
+            self.register_parameter("bias", None)
+
+    def reset_parameters(self):
+        gain = torch.nn.init.calculate_gain("relu")
+        torch.nn.init.xavier_uniform_(self.lin_neigh.weight, gain=gain)
+        torch.nn.init.xavier_uniform_(self.lin_self.weight, gain=gain)
+
+    def propagate(self, graph, local_nodes_feat, layer):
+        return Aggregator.apply(graph, local_nodes_feat, layer, self.num_bits, self.is_pre_delay, self.training)
+
+    def forward(self, graph, local_nodes_feat, layer) -> Tensor:
+        agg = self.propagate(graph, local_nodes_feat, layer)
+        deg = graph.in_degrees.reshape(-1, 1) if self.normalize else None
+        return _SageCombine.apply(agg, local_nodes_feat, deg, self.lin_neigh.weight, self.lin_self.weight, self.bias)
+
+
+class DistSAGE(torch.nn.Module):
+    """The model of the reference's training script with its constructor and call signatures
+    (examples/graphsage/sage.py:127-211; LayerNorm or no norm, no label augmentation)."""
+
+    def __init__(self, in_channels, hidden_channels, out_channels, num_layers=3, dropout=0.5, num_bits=32,
+                 is_pre_delay=False, norm_type="LayerNorm", is_label_augment=False):
+        super().__init__()
+        if is_label_augment:
+            raise NotImplementedError("label augmentation (MaskLabel) is outside the aggregation hot path")
+        if norm_type not in (None, "LayerNorm"):
+            raise NotImplementedError("only LayerNorm (the reference's default) or no normalisation")
+        dims = [in_channels] + [hidden_channels] * (num_layers - 1) + [out_channels]
+        self.convs = torch.nn.ModuleList(DistSAGEConvGrad(a, b, num_bits, is_pre_delay) for a, b in zip(dims[:-1], dims[1:]))
+        self.norms = torch.nn.ModuleList(LayerNorm(hidden_channels) for _ in range(num_layers - 1)) if norm_type else None
+        self.dropout, self.norm_type = dropout, norm_type
+
+    def reset_parameters(self):
+        for conv in self.convs:
+            conv.reset_parameters()
+        if self.norms is not None:
+            for norm in self.norms:
+                norm.reset_parameters()
+
+    def forward(self, graph, nodes_feats, labels=None, label_mask=None):
+        for i, conv in enumerate(self.convs[:-1]):
+            nodes_feats = conv(graph, nodes_feats, i)
+            nodes_feats = F.dropout(nodes_feats, p=self.dropout, training=self.training)
+            if self.norms is not None:
+                nodes_feats = self.norms[i](nodes_feats)
+            nodes_feats = F.relu(nodes_feats)
+        nodes_feats = self.convs[-1](graph, nodes_feats, len(self.convs) - 1)
+        return F.log_softmax(nodes_feats, dim=1)

@@ -4,8 +4,9 @@
 ``SPMM_backward(src, other, out)`` : out += A^T @ other
 
 The reference computes an nnz-balanced OpenMP row split on first use and caches it on the matrix
-(spmm_kernel.py:49-58); here the cached object is the GPU schedule (SpmmPlan).  The work-range
-getters/setters are still honoured so callers that inspect them keep working."""
+(spmm_kernel.py:49-58); here the object that matters is the GPU schedule (SpmmPlan), cached the same
+way.  The row split is still computed once per matrix and stored through the work-range setters, so
+callers that read ``get_work_range()`` see what the reference would have put there."""
 import torch
 
 from ..supergnn_ops import quant_segments, spmm
@@ -57,6 +58,8 @@ def SPMM_forward(src, other: torch.Tensor, out: torch.Tensor, accumulate=None) -
     rowptr, col, value = src.csr()
     col_splits = disribute_work_for_col(other, 1)
     row_splits, _ = src.get_work_range()
+    if row_splits.size(0) == 0:   # once per matrix, as the reference does (spmm_kernel.py:49-53)
+        row_splits = distribute_work_for_row(rowptr, value, torch.get_num_threads())
     src.set_work_range(row_splits, col_splits)
     if value is not None:
         value = value.to(other.dtype)
@@ -71,6 +74,8 @@ def SPMM_backward(src, other: torch.Tensor, out: torch.Tensor, accumulate=None) 
     value_T = src.storage.value_T()
     col_splits = disribute_work_for_col(other, 1)
     row_splits, _ = src.get_work_range_for_transpose()
+    if row_splits.size(0) == 0:   # spmm_kernel.py:82-85
+        row_splits = distribute_work_for_row(colptr, value_T, torch.get_num_threads())
     src.set_work_range_for_transpose(row_splits, col_splits)
     if value_T is not None:
         value_T = value_T.to(other.dtype)

@@ -286,3 +286,119 @@ def test_world_from_reference_partition_files(tmp_path):
             assert np.all(np.abs(got - want) <= 1e-4 + 1e-5 * np.abs(want))
         else:
             assert np.linalg.norm(got - want) / np.linalg.norm(want) < 0.01
+
+
+# ------------------------------------------------------------------------------------------------
+# the reference's own signatures: Aggregator.apply(graph, feat, layer, num_bits, is_pre_delay, is_training)
+# (super_gnn/aggregator.py:15-23) and DistSAGEConvGrad.forward(graph, feat, layer) (layers/sageconv.py:62-89)
+# ------------------------------------------------------------------------------------------------
+def _global_products(rowptr, col, w, x, G):
+    rp, c, v = rowptr.numpy(), col.numpy().astype(np.int64), w.numpy()
+    n = rp.shape[0] - 1
+    want = np.zeros((n, x.shape[1]), np.float32)
+    orc.spmm_accumulate(rp, c, v, x.numpy(), want)
+    AT = sp.csr_matrix((v, c, rp), shape=(n, n)).T.tocsr(); AT.sort_indices()
+    rpt, ct, vt = AT.indptr.astype(np.int64), AT.indices.astype(np.int64), AT.data.astype(np.float32)
+    want_g = np.zeros((n, x.shape[1]), np.float32)
+    orc.spmm_accumulate(rpt, ct, vt, G.numpy(), want_g)
+    return (rp, c, v, want), (rpt, ct, vt, want_g)
+
+
+@pytest.mark.parametrize("pre", [False, True])
+@pytest.mark.parametrize("P", [1, 4])
+def test_reference_signature_aggregator_equals_global_product(pre, P):
+    from super_gnn_amd.aggregator import Aggregator, LoopbackWorld
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    rowptr, col, w = _graph()
+    n, F = rowptr.numel() - 1, 64
+    graphs = build_loopback_partitions(rowptr, col, w, P, F, num_bits=32, is_pre_delay=pre)
+    # world_size == 1: the partition object itself is the graph argument; P > 1: the world of all partitions
+    graph = graphs[0] if P == 1 else LoopbackWorld(graphs, 32, pre)
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(n, F, generator=gen)
+    G = torch.randn(n, F, generator=gen)
+    feat = x.cuda().requires_grad_()
+    out = Aggregator.apply(graph, feat, 0, 32, pre, True)
+    assert out.shape == (n, F)
+    out.backward(G.cuda())
+    (rp, c, v, want), (rpt, ct, vt, want_g) = _global_products(rowptr, col, w, x, G)
+    assert_spmm_close(out.detach().cpu().numpy(), want, orc.spmm_f64(rp, c, v, x.numpy()), abs_sum64(rp, c, v, x.numpy()),
+                      np.diff(rp), what="forward")
+    assert_spmm_close(feat.grad.cpu().numpy(), want_g, orc.spmm_f64(rpt, ct, vt, G.numpy()), abs_sum64(rpt, ct, vt, G.numpy()),
+                      np.diff(rpt), what="backward")
+    # the work range the reference caches on the matrix on first use is there (spmm_kernel.py:49-58)
+    rs, cs = graphs[0].local_adj_t.get_work_range()
+    assert rs.numel() == torch.get_num_threads() + 1 and int(rs[0]) == 0 and int(rs[-1]) == graphs[0].local_adj_t.sparse_size(0)
+    assert cs.tolist() == [0, F]
+
+
+@pytest.mark.parametrize("bits,pre", [(8, False), (2, True), (16, True), (16, False)])
+def test_reference_signature_aggregator_equals_loopback_world(bits, pre):
+    """Same floats as the list-based world API; eval mode exchanges fp32 rows whatever num_bits says
+    (communicator.py:61-62); 16 ships bf16 copies of the boundary rows."""
+    from super_gnn_amd.aggregator import Aggregator, LoopbackWorld
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    rowptr, col, w = _graph(n=8000, und_edges=60000, seed=9)
+    n, F, P = rowptr.numel() - 1, 128, 4
+    graphs = build_loopback_partitions(rowptr, col, w, P, F, num_bits=bits, is_pre_delay=pre)
+    world = LoopbackWorld(graphs, bits, pre)
+    gen = torch.Generator().manual_seed(1)
+    x = torch.randn(n, F, generator=gen).cuda()
+    G = torch.randn(n, F, generator=gen).cuda()
+    feat = x.clone().requires_grad_()
+    out = Aggregator.apply(world, feat, 1, bits, pre, True)
+    out.backward(G)
+    if bits != 16:
+        feats = [x[g.node_range[0]:g.node_range[1]].clone().requires_grad_() for g in graphs]
+        outs = world.aggregate(feats)
+        torch.autograd.backward(outs, [G[g.node_range[0]:g.node_range[1]] for g in graphs])
+        assert torch.equal(out, torch.cat(outs))
+        assert torch.equal(feat.grad, torch.cat([f.grad for f in feats]))
+    else:
+        # bf16 rows: the exact result with every boundary row rounded to bf16 once, i.e. within 2^-8 relative of
+        # the fp32 exchange per contribution; and different from it (the rounding really happened)
+        exact = Aggregator.apply(LoopbackWorld(graphs, 32, pre), x, 1, 32, pre, True)
+        err = (out.detach() - exact).abs()
+        assert float(err.max()) > 0
+        xa = x.abs()
+        bound = Aggregator.apply(LoopbackWorld(graphs, 32, pre), xa, 1, 32, pre, True) * 2.0 ** -8 + 1e-6
+        assert bool((err <= bound).all())
+    # evaluation mode: fp32 exchange
+    ev = Aggregator.apply(world, x, 1, bits, pre, False)
+    ev32 = Aggregator.apply(LoopbackWorld(graphs, 32, pre), x, 1, 32, pre, True)
+    assert torch.equal(ev, ev32)
+    with pytest.raises(ValueError):
+        Aggregator.apply(world, x, 1, bits, not pre, True)
+    with pytest.raises(ValueError):
+        Aggregator.apply(graphs[0], x[:graphs[0].local_adj_t.sparse_size(0)], 1, bits, pre, True)  # a rank that has peers
+
+
+def test_reference_signature_sage_layer_and_model():
+    from super_gnn_amd.aggregator import LoopbackWorld
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    from super_gnn_amd.layers import DistSAGE, DistSAGEConvGrad, LoopbackSAGEConv
+    rowptr, col, _ = _graph(n=6000, und_edges=40000, seed=3)
+    n, F, H, P = rowptr.numel() - 1, 32, 48, 3
+    graphs = build_loopback_partitions(rowptr, col, None, P, max(F, H), num_bits=2, is_pre_delay=True)
+    world = LoopbackWorld(graphs, 2, True)
+    torch.manual_seed(0)
+    a = DistSAGEConvGrad(F, H, 2, True).cuda(); a.reset_parameters()
+    b = LoopbackSAGEConv(F, H).cuda()
+    b.load_state_dict(a.state_dict())
+    x = torch.randn(n, F, device="cuda")
+    ya = a(world, x, 0)
+    yb = torch.cat(b(world, [x[g.node_range[0]:g.node_range[1]] for g in graphs]))
+    assert torch.equal(ya, yb)
+    # the model trains through the reference's call sequence: model(graph, feats, labels, mask) -> log-probabilities
+    model = DistSAGE(F, H, 5, num_layers=3, dropout=0.0, num_bits=2, is_pre_delay=True).cuda()
+    model.reset_parameters()
+    labels = torch.randint(0, 5, (n,), device="cuda")
+    opt = torch.optim.Adam(model.parameters(), lr=0.01)
+    losses = []
+    for _ in range(8):
+        opt.zero_grad()
+        loss = torch.nn.functional.nll_loss(model(world, x, labels, None), labels)
+        loss.backward()
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert losses[-1] < losses[0]

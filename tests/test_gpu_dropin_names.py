@@ -103,3 +103,25 @@ def test_quantization_script_flow_with_reference_import_names(compat_path, bits)
         scale = (data_fp32.max(dim=1)[0] - data_fp32.min(dim=1)[0]) / (2 ** bits - 1)
         codes = torch.round((data_fp32 - data_fp32.min(dim=1, keepdim=True)[0]) / scale[:, None]).to(torch.uint8)
         assert torch.equal(data_int8.view(num_nodes, feat_len), codes)
+
+
+def test_aggregation_layer_with_reference_import_names(compat_path):
+    # the reference's layer code: `from super_gnn.aggregator import Aggregator`, `Aggregator.apply(graph, feat, layer,
+    # num_bits, is_pre_delay, training)` (layers/sageconv.py:56-60) on a partition that is the whole graph (world_size 1)
+    from super_gnn.aggregator import Aggregator
+    from super_gnn.data_manager import DistributedGraph
+    from super_gnn.layers.sageconv import DistSAGEConvGrad
+    from super_gnn_amd.data_manager import build_loopback_partitions
+    from super_gnn_amd import synth
+    rowptr, col = synth.uniform_degree_graph(3000, 9, seed=2)
+    graph = build_loopback_partitions(rowptr, col.to(torch.int64), None, 1, 64, num_bits=32, is_pre_delay=False)[0]
+    assert isinstance(graph, DistributedGraph)
+    x = torch.randn(3000, 64, generator=torch.Generator().manual_seed(0))
+    out = Aggregator.apply(graph, x.cuda(), 0, 32, False, True)
+    want = np.zeros((3000, 64), np.float32)
+    orc.spmm_accumulate(rowptr.numpy(), col.numpy().astype(np.int64), np.ones(col.numel(), np.float32), x.numpy(), want)
+    assert np.array_equal(out.cpu().numpy(), want)      # 10 edges per row: the reference's fma chain, bit for bit
+    conv = DistSAGEConvGrad(64, 16, 32, False).cuda()
+    y = conv(graph, x.cuda(), 0)
+    ref = (torch.from_numpy(want).cuda() / graph.in_degrees) @ conv.lin_neigh.weight.t() + x.cuda() @ conv.lin_self.weight.t() + conv.bias
+    assert torch.allclose(y, ref, rtol=1e-4, atol=1e-4)
