@@ -93,7 +93,11 @@ int sgnn_spmm_plan_schedule(const sgnn_spmm_plan *plan, int64_t F, int64_t info[
  * long rows' values in its own (regrouped) edge order, and later sgnn_spmm_csr_f32 /
  * sgnn_spmm_csr_dq*_f32 calls that pass the SAME pointer read that copy contiguously instead of
  * going through the edge permutation (-8 % on the long-row kernel of the power-law graph).  The
- * caller must bind again after changing the array's contents; val == NULL unbinds.  The reference
+ * caller must bind again after changing the array's contents (also after freeing it and getting the same
+ * address back from an allocator); val == NULL unbinds.  Nothing is ever bound implicitly: a run call
+ * only compares the pointer it is given with the bound one, and a different pointer is read in place.
+ * A plan holds per-call state (partial sums, the restaged operand, these copies): use it, and bind it,
+ * from one stream at a time, or order the streams yourself.  The reference
  * passes `value` on every call (super_gnn/ops/spmm_kernel.py:60-65) but never changes it after the
  * graph is built (DataProcessor.py:112,119), which is what this exploits. */
 int sgnn_spmm_plan_bind_values(sgnn_spmm_plan *plan, const float *val, sgnn_stream_t stream);
@@ -125,7 +129,10 @@ int sgnn_spmm_csr_f32(sgnn_spmm_plan *plan, const float *val, const float *x, fl
  *     rows never touch the scratch and have no limit;
  *   - every call on one GPU shares that GPU's scratch: two calls whose kernels may overlap in time
  *     (different streams, different host threads) race on it.  Calls queued on one stream are safe.
- *     Nothing in the scratch has to start at zero: each call writes every partial it later reads. */
+ *     Nothing in the scratch has to start at zero: each call writes every partial it later reads;
+ *   - a matrix that sgnn_spmm_plan_schedule reports as band-scheduled runs that schedule here only if an
+ *     earlier sgnn_spmm_csr_f32 call has already built it for a width >= F (building allocates); otherwise
+ *     the row-class kernels run, whose long rows are summed per piece instead of in one chain. */
 int sgnn_spmm_csr_f32_noalloc(sgnn_spmm_plan *plan, const float *val, const float *x, float *out,
                               int64_t F, int64_t ldx, int64_t ldo, int accumulate,
                               const float *row_div, sgnn_stream_t stream);
