@@ -108,6 +108,7 @@ class SpmmPlan:
         self.nnz = cl.numel()
         if self.M < 0:
             raise ValueError("rowptr must have at least one entry")
+        _destroy_plan_handle()   # handles parked during a graph capture
         h = ctypes.c_void_p()
         check(lib.sgnn_spmm_plan_create(_ptr(rp), _ptr(cl), int(cl.dtype == torch.int64), self.M, self.K, self.nnz,
                                         int(long_row_threshold), int(piece_edges), _stream(), ctypes.byref(h)))
@@ -221,10 +222,35 @@ class SpmmPlan:
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
         if h:
-            try:
-                lib.sgnn_spmm_plan_destroy(h)
-            except Exception:
-                pass
+            _destroy_plan_handle(h)
+
+
+# Plan handles whose owner died while a stream was being captured into a HIP graph.  Destroying a plan frees
+# device memory, and a free issued during a capture invalidates the capture (Python's cyclic collector may run a
+# plan's finaliser at any allocation, i.e. also in the middle of somebody's ``torch.cuda.graph`` block), so such
+# handles wait here until the next plan is created or destroyed outside a capture.
+_deferred_handles = []
+
+
+def _capturing():
+    try:
+        return torch.cuda.is_available() and torch.cuda.is_current_stream_capturing()
+    except Exception:
+        return False
+
+
+def _destroy_plan_handle(h=None):
+    try:
+        if _capturing():
+            if h:
+                _deferred_handles.append(h)
+            return
+        if h:
+            lib.sgnn_spmm_plan_destroy(h)
+        while _deferred_handles:
+            lib.sgnn_spmm_plan_destroy(_deferred_handles.pop())
+    except Exception:
+        pass
 
 
 def _cached_plan(rowptr, col, K):

@@ -365,6 +365,43 @@ def test_steady_state_calls_replay_from_a_captured_graph():
         assert torch.equal(out, want) and torch.equal(out_q, want_q), f"replay {i}"
 
 
+def test_plan_finalised_during_a_capture_does_not_invalidate_it():
+    """Python may run a dead plan's finaliser at any time, also inside someone's graph capture; freeing device
+    memory there would invalidate the capture, so the wrapper parks the handle until later."""
+    import gc
+    ops = _gpu()
+    dev = torch.device("cuda:0")
+    rowptr, col, val = random_csr(500, 400, 7, seed=11, hubs=2, hub_deg=300)
+    rp, cl = torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev)
+    x = torch.randn(400, 64, generator=torch.Generator().manual_seed(1)).to(dev)
+    v = torch.from_numpy(val).to(dev)
+    out = torch.zeros(500, 64, device=dev)
+    plan = ops.SpmmPlan(rp, cl, 400)
+    for _ in range(3):
+        out.zero_(); plan.run(v, x, out, accumulate=True)
+    torch.cuda.synchronize()
+    want = out.clone()
+
+    class Holder:
+        pass
+    gc.collect()                                                      # leftovers of earlier tests go now
+    h = Holder(); h.me = h; h.plan = ops.SpmmPlan(rp, cl, 400)      # a plan only the cyclic collector can reach
+    h.plan.run(v, x, torch.zeros(500, 64, device=dev), accumulate=True)
+    torch.cuda.synchronize()
+    del h
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gc.collect()                                                  # the dead plan's finaliser runs here
+        out.zero_(); plan.run(v, x, out, accumulate=True)
+    assert len(ops._deferred_handles) == 1
+    for i in range(2):
+        out.fill_(3.0); torch.cuda.synchronize()
+        graph.replay(); torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {i}"
+    ops.SpmmPlan(rp, cl, 400)                                         # creating a plan releases the parked handle
+    assert not ops._deferred_handles
+
+
 @pytest.mark.parametrize("tag", ["spmm_acc", "spmm_acc128", "spmm_ovw"])
 def test_committed_reference_extension_vectors(tag):
     # inputs and the outputs the reference's own x86 extension produced for them (tests/golden/make_ref_vectors.py);
