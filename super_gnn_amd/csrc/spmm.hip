@@ -1593,7 +1593,8 @@ static int launch_band(const BandSchedule *bs, const BandShape &sh, int b, const
     const uint32_t nb = (uint32_t)((wgs + n_rg - 1) / n_rg) * kNumXCD;
     const size_t lds = sizeof(float) * (size_t)gpb * (size_t)band_group_floats(sh.G * 4);
     // every restaged row of a slice within 4 GB of the slice's start: 32-bit gather offsets
-    const bool off32 = (uint64_t)bs->K * (uint64_t)sh.slice_pad * 4u < ((uint64_t)1 << 32);
+    // (SGNN_SPMM_BAND_OFF64=1 forces the 64-bit variant so that tests reach it at small sizes)
+    const bool off32 = (uint64_t)bs->K * (uint64_t)sh.slice_pad * 4u < ((uint64_t)1 << 32) && env_int("SGNN_SPMM_BAND_OFF64", 0) == 0;
     auto kernel = off32 ? spmm_band_kernel<EVEN, true> : spmm_band_kernel<EVEN, false>;
     static size_t lds_allowed[2] = {48 * 1024, 48 * 1024};  // per instantiation
     if (lds > lds_allowed[off32]) {

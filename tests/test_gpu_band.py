@@ -75,6 +75,25 @@ def test_band_schedule_bit_identical_to_oracle(M, K, F, deg, cols, monkeypatch):
     assert np.array_equal(out4.cpu().numpy(), want1), "unit weights + mean"
 
 
+@pytest.mark.parametrize("F", [602, 128, 37])
+def test_band_schedule_with_64_bit_gather_offsets(F, monkeypatch):
+    # operands of 4 GB and more per feature slice take a kernel variant with 64-bit row offsets; forced here
+    ops = _ops()
+    _force(monkeypatch, 96)
+    monkeypatch.setenv("SGNN_SPMM_BAND_OFF64", "1")
+    M, K = 333, 777
+    rowptr, col, val = random_csr(M, K, 30, seed=F, empty_frac=0.1, hubs=2, hub_deg=500)
+    rng = np.random.default_rng(F)
+    x = rng.standard_normal((K, F), dtype=np.float32)
+    init = rng.standard_normal((M, F), dtype=np.float32)
+    dev = torch.device("cuda:0")
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    want = init.copy(); orc.spmm_accumulate(rowptr, col, val, x, want)
+    out = torch.from_numpy(init.copy()).to(dev)
+    plan.run(torch.from_numpy(val).to(dev), torch.from_numpy(x).to(dev), out, accumulate=True)
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
 def test_band_schedule_equals_row_class_schedule_and_honours_rebinding(monkeypatch):
     ops = _ops()
     dev = torch.device("cuda:0")
