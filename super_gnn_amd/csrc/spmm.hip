@@ -1584,7 +1584,7 @@ static int band_build(sgnn_spmm_plan *p, int band_cols, int n_bands, hipStream_t
 
 template <bool EVEN>
 static int launch_band(const BandSchedule *bs, const BandShape &sh, int b, const float *val_bm, const float *xs, float *out,
-                       int F, int64_t ldo, hipStream_t st) {
+                       int F, int64_t ldo, hipStream_t st, int device) {
     const int64_t c0 = bs->chunk_off[(size_t)b], c1 = bs->chunk_off[(size_t)b + 1];
     if (c1 == c0) return SGNN_OK;
     const int gpb = (kBlock / 64) * (64 / sh.G);  // lane groups per workgroup
@@ -1596,10 +1596,16 @@ static int launch_band(const BandSchedule *bs, const BandShape &sh, int b, const
     // (SGNN_SPMM_BAND_OFF64=1 forces the 64-bit variant so that tests reach it at small sizes)
     const bool off32 = (uint64_t)bs->K * (uint64_t)sh.slice_pad * 4u < ((uint64_t)1 << 32) && env_int("SGNN_SPMM_BAND_OFF64", 0) == 0;
     auto kernel = off32 ? spmm_band_kernel<EVEN, true> : spmm_band_kernel<EVEN, false>;
-    static size_t lds_allowed[2] = {48 * 1024, 48 * 1024};  // per instantiation
-    if (lds > lds_allowed[off32]) {
-        SGNN_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        lds_allowed[off32] = lds;
+    // the dynamic-LDS limit of a kernel is a per-device setting: remember what each device has been told
+    static std::mutex mu;
+    static size_t lds_allowed[64][2];
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        size_t &allowed = lds_allowed[device & 63][off32];
+        if (lds > std::max<size_t>(allowed, 48 * 1024)) {
+            SGNN_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            allowed = lds;
+        }
     }
     hipLaunchKernelGGL(kernel, dim3(nb), dim3(kBlock), lds, st, bs->rowptr_bm + (size_t)b * (size_t)(bs->M + 1), bs->col_bm, val_bm,
                        xs, bs->K, out, bs->chunks + c0, (int)(c1 - c0), F, ldo, sh.slice_floats, sh.slice_pad, sh.n_slices, sh.G);
@@ -1667,8 +1673,8 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
     {
         ProfScope prof(K_SPMM_BAND, st);
         for (int b = 0; b < bs->n_bands; ++b) {
-            const int rc = sh.even ? launch_band<true>(bs, sh, b, val_bm, p->band_xs, out, iF, ldo, st)
-                                   : launch_band<false>(bs, sh, b, val_bm, p->band_xs, out, iF, ldo, st);
+            const int rc = sh.even ? launch_band<true>(bs, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device)
+                                   : launch_band<false>(bs, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device);
             if (rc != SGNN_OK) return rc;
         }
     }

@@ -230,3 +230,48 @@ def test_partition_builder_on_the_reference_tests_edge_lists():
         x = np.arange(N * 4, dtype=np.float32).reshape(N, 4)
         got = frm @ (to @ x[:10])
         assert np.array_equal(got, (A @ x)[10:])
+
+
+# ------------------------------------------------------------------------------------------------
+# Literals of the reference's tests/test_data_preprocessor.py (plain mode, no pre/post split): how the
+# remote sources of a rank are listed (ascending global id, grouped by owning rank: obtain_remote_nodes_list,
+# :17-29) and how in-degrees count local and remote edges with a floor of one (get_in_degrees, :107-114).
+# ------------------------------------------------------------------------------------------------
+def _csr_over_destinations(src, dst, N):
+    A = sp.coo_matrix((np.ones(len(src), np.float32), (dst, src)), shape=(N, N)).tocsr()
+    A.sort_indices()
+    return torch.from_numpy(A.indptr.astype(np.int64)), torch.from_numpy(A.indices.astype(np.int64)), torch.from_numpy(A.data)
+
+
+def test_remote_node_list_of_the_reference_tests_literal():
+    # three ranks owning nodes [0,3), [3,6), [6,9); rank 2 receives from sources 2, 5, 5, 4, 4, 4, 1.  The
+    # reference's expected values: remote nodes [1, 2, 4, 5], ranges [0, 2, 4, 4], per-rank counts [2, 2, 0].
+    src = [2, 5, 5, 4, 4, 4, 1]
+    dst = [6, 7, 8, 6, 7, 8, 7]
+    rowptr, col, val = _csr_over_destinations(src, dst, 9)
+    graphs = build_loopback_partitions(rowptr, col, val, 3, 4, num_bits=32, is_pre_delay=False, device="cpu",
+                                       bounds=torch.tensor([0, 3, 6, 9]))
+    g2 = graphs[2]
+    assert g2.comm_splits.recv_splits == [2, 2, 0]
+    remote_nodes = [1, 2, 4, 5]
+    R = _scipy(g2.remote_adj_t).toarray()
+    assert R.shape == (3, 4)
+    want = np.zeros((3, 4), np.float32)
+    for s, d in zip(src, dst):
+        want[d - 6, remote_nodes.index(s)] = 1.0
+    assert np.array_equal(R, want)
+    # the senders list exactly those nodes, in that order, as local ids
+    assert graphs[0].idx_nodes_send_to_others.tolist() == [1, 2] and graphs[0].comm_splits.send_splits == [0, 0, 2]
+    assert graphs[1].idx_nodes_send_to_others.tolist() == [1, 2] and graphs[1].comm_splits.send_splits == [0, 0, 2]
+
+
+def test_in_degrees_of_the_reference_tests_literal():
+    # five local nodes; local edges 1->0, 2->0, 3->1; remote edges from three nodes of another rank into 2, 3, 3.
+    # The reference's expected in-degrees: [2, 1, 1, 2, 1] (a node without in-edges counts as 1).
+    src = [1, 2, 3, 5, 6, 7]
+    dst = [0, 0, 1, 2, 3, 3]
+    rowptr, col, val = _csr_over_destinations(src, dst, 8)
+    graphs = build_loopback_partitions(rowptr, col, val, 2, 4, num_bits=32, is_pre_delay=False, device="cpu",
+                                       bounds=torch.tensor([0, 5, 8]))
+    assert graphs[0].in_degrees.reshape(-1).tolist() == [2.0, 1.0, 1.0, 2.0, 1.0]
+    assert graphs[1].in_degrees.reshape(-1).tolist() == [1.0, 1.0, 1.0]
