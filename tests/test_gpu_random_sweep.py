@@ -129,3 +129,52 @@ def test_fused_random_shapes(case):
         plan.run_quantized(w, q, prm, segs, bits, got, accumulate=accumulate, row_div=div)
     torch.cuda.synchronize()
     assert torch.equal(got, want), f"case {case}: bits={bits} F={F} M={M} K={K} deg={deg} hubs={hubs} P={P} bf16={bf16}"
+
+
+@pytest.mark.parametrize("case", range(30))
+def test_band_schedule_random_shapes(case, monkeypatch):
+    # the column-band schedule forced onto random matrices with random band widths: column-sorted rows must come
+    # out bit-identical to the oracle's CSR-order fma chain in every mode
+    from super_gnn_amd import supergnn_ops as ops
+    rng = np.random.default_rng(4000 + case)
+    M, K = int(rng.integers(1, 2000)), int(rng.integers(1, 2500))
+    F = int(rng.choice([1, 2, 5, 16, 48, 64, 100, 128, 200, 256, 301, 602, 640, 1030]))
+    deg = float(rng.choice([0.5, 3, 12, 50]))
+    hubs = int(rng.integers(0, 3)) if M > 8 else 0
+    cols = int(rng.choice([1, 7, 32, 100, 256, 1000, 4096]))
+    monkeypatch.setenv("SGNN_SPMM_BAND", "1")
+    monkeypatch.setenv("SGNN_SPMM_BAND_COLS", str(cols))
+    if case % 5 == 0:
+        monkeypatch.setenv("SGNN_SPMM_BAND_CHUNK_EDGES", str(int(rng.choice([8, 24, 64]))))
+    unsorted = case % 6 == 5                                  # rows in random column order: the schedule must step aside
+    rowptr, col, val = random_csr(M, K, deg, seed=4000 + case, empty_frac=float(rng.choice([0, 0.3, 0.9])), hubs=hubs,
+                                  hub_deg=int(rng.integers(100, 3000)), dup=unsorted)
+    x = rng.standard_normal((K, F)).astype(np.float32)
+    init = rng.standard_normal((M, F)).astype(np.float32)
+    accumulate, mean, weighted = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), bool(rng.integers(0, 3))
+    dev = torch.device("cuda:0")
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    assert plan.schedule(F)["band"] == 1
+    div = np.maximum(np.diff(rowptr), 1).astype(np.float32) if mean else None
+    v = val if weighted else np.ones(col.shape[0], np.float32)
+    xd = torch.from_numpy(x).to(dev)
+    out = torch.from_numpy(init.copy()).to(dev)
+    for _ in range(2 if case % 3 == 0 else 1):
+        out.copy_(torch.from_numpy(init))
+        plan.run(torch.from_numpy(val).to(dev) if weighted else None, xd, out, accumulate=accumulate,
+                 row_div=torch.from_numpy(div).to(dev) if mean else None)
+    want = init.copy() if accumulate else np.zeros_like(init)
+    orc.spmm_accumulate(rowptr, col, v, x, want)
+    if mean:
+        orc.row_divide(want, div)
+    what = f"case {case}: M={M} K={K} F={F} cols={cols} acc={accumulate} mean={mean}"
+    if not unsorted:
+        assert np.array_equal(out.cpu().numpy(), want), what
+        return
+    is_sorted = bool(np.all((np.diff(col) >= 0) | np.isin(np.arange(1, col.size), rowptr[1:-1]))) if col.size > 1 else True
+    assert plan.schedule(F)["band"] == int(is_sorted)          # known after the first product
+    base = init if accumulate else None
+    f64, asum = orc.spmm_f64(rowptr, col, v, x, base), abs_sum64(rowptr, col, v, x, base)
+    if mean:
+        f64, asum = f64 / div[:, None].astype(np.float64), asum / div[:, None].astype(np.float64)
+    assert_spmm_close(out.cpu().numpy(), want, f64, asum, np.diff(rowptr), what=what)
