@@ -13,7 +13,7 @@ def random_csr(M, K, avg_deg, seed, empty_frac=0.0, hubs=0, hub_deg=0, dup=False
     if empty_frac > 0:
         deg[rng.random(M) < empty_frac] = 0
     if hubs:
-        deg[rng.choice(M, size=hubs, replace=False)] = hub_deg
+        deg[rng.choice(M, size=min(hubs, M), replace=False)] = hub_deg
     rowptr = np.zeros(M + 1, dtype=np.int64)
     np.cumsum(deg, out=rowptr[1:])
     nnz = int(rowptr[-1])
