@@ -367,18 +367,22 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
 // ------------------------------------------------------------------------------------------------
 // Rows per chunk and staged (row offset, val) pairs per chunk of the band kernel.
 #ifndef SGNN_BAND_ROWS
-#define SGNN_BAND_ROWS 10
+#define SGNN_BAND_ROWS 11
 #endif
 #ifndef SGNN_BAND_EDGES
-#define SGNN_BAND_EDGES 128
+#define SGNN_BAND_EDGES 240
 #endif
 #ifndef SGNN_BAND_U
-#define SGNN_BAND_U 12
+#define SGNN_BAND_U 8
 #endif
 constexpr int kBandRows = SGNN_BAND_ROWS;
 constexpr int kBandEdges = SGNN_BAND_EDGES;
 constexpr int kBandWindow = SGNN_BAND_U;  // gathers in flight per lane group
 constexpr int kBandPad = 16;              // staging entries past the last pair (>= the gather window)
+#ifndef SGNN_BAND_BLOCK
+#define SGNN_BAND_BLOCK 256
+#endif
+constexpr int kBandBlock = SGNN_BAND_BLOCK;  // threads per workgroup of the band kernel
 static_assert(kBandWindow <= kBandPad, "gather window wider than the staging pad");
 __host__ __device__ constexpr int band_group_floats(int tile_stride) { return kBandRows * tile_stride + 2 * (kBandEdges + kBandPad); }
 
@@ -443,14 +447,21 @@ __device__ __forceinline__ void out_store(float *p, const float (&r)[4], int nf)
     }
 }
 
-// One lane group per chunk of consecutive rows (at most kBandRows rows and kBandEdges edges).  A group is
+// A chunk is a run of consecutive rows of one band: at most kBandRows rows and kBandEdges edges (a single row may
+// have more).  Its record is two int4: (first row, rows, first edge, edges) and the rows' edge offsets relative
+// to the first edge, one byte each (entries 0 .. rows; unused for a one-row chunk, whose offsets are 0 and edges).
+static_assert(kBandEdges <= 255 && kBandRows <= 11, "row offsets of a chunk are stored as bytes, twelve per record");
+constexpr int kBandKeyRounds = (kBandEdges + kBandPad + 63) / 64;  // staging loads per lane: four pairs per load, >= 16 lanes
+
+// One lane group per chunk.  A group is
 // G = slice_pad / 4 lanes (any value from 16 to 64, not only powers of two), one float4 of the restaged slice
 // each, and a wavefront carries 64 / G groups: a vector memory instruction occupies a CU's address path for as
 // long whether 20 or 64 of its lanes are active, so what a gather costs is decided by how many gathers share one
 // instruction.  At F = 602 a slice is 76 floats padded to 80, G = 20, and three gathers travel together.
 // Three phases per chunk:
-//   1. everything that comes from HBM is requested at once: the old `out` values of all the chunk's rows for
-//      this feature slice go to LDS (the output tile of the chunk), and so do its (row offset, val) pairs;
+//   1. everything that comes from HBM is requested in ONE batch right after the chunk's record has arrived, so a
+//      chunk pays two memory latencies in all: the old `out` values of all its rows for this feature slice go to
+//      LDS (the output tile of the chunk), and so do its (row offset, val) pairs;
 //   2. the gather loop: a rolling window of kBandWindow gathers of dense-row slices, all of them L2 hits, one fma
 //      per edge in CSR order; a row boundary swaps the accumulator through the LDS tile.  Nothing slow sits in
 //      the vector memory queue during this phase: loads return in order, and one HBM-latency load between two
@@ -458,10 +469,10 @@ __device__ __forceinline__ void out_store(float *p, const float (&r)[4], int nf)
 //   3. the tile rows that received edges are written back.
 // A tile column belongs to one lane and a group to one wavefront: the kernel has no workgroup barrier.
 template <bool EVEN, bool OFF32>
-__global__ __launch_bounds__(kBlock) void spmm_band_kernel(
-    const int32_t *__restrict__ rowptr_b, const int32_t *__restrict__ col_bm, const float *__restrict__ val_bm,
-    const float *__restrict__ xs, int64_t K, float *__restrict__ out, const int4 *__restrict__ chunks, int n_chunks, int F,
-    int64_t ldo, int slice_floats, int slice_pad, int n_slices, int G) {
+__global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
+    const int32_t *__restrict__ col_bm, const float *__restrict__ val_bm, const float *__restrict__ xs, int64_t K,
+    float *__restrict__ out, const int4 *__restrict__ chunks, int n_chunks, int F, int64_t ldo, int slice_floats,
+    int slice_pad, int n_slices, int G) {
     extern __shared__ float band_lds[];
     constexpr int U = kBandWindow;
     const int tile_stride = G * 4;
@@ -472,7 +483,7 @@ __global__ __launch_bounds__(kBlock) void spmm_band_kernel(
     const int gid = wave * gpw + gsub;            // group inside the workgroup
     const int xcd = blockIdx.x % kNumXCD;
     const int slice = xcd % n_slices, rg = xcd / n_slices, n_rg = kNumXCD / n_slices;
-    const int ci = ((int)(blockIdx.x / kNumXCD) * n_rg + rg) * ((kBlock / 64) * gpw) + gid;
+    const int ci = ((int)(blockIdx.x / kNumXCD) * n_rg + rg) * ((kBandBlock / 64) * gpw) + gid;
     const int f_lo = slice * slice_floats;        // first feature column of this slice
     const int vpr = slice_pad / 4;                // float4 per restaged row
     const bool valid = gsub < gpw && ci < n_chunks && f_lo < F;
@@ -481,15 +492,22 @@ __global__ __launch_bounds__(kBlock) void spmm_band_kernel(
     float *lval = reinterpret_cast<float *>(lkey + kBandEdges + kBandPad);
     const float *xslice = xs + (int64_t)slice * K * slice_pad;
 
-    int4 ch = make_int4(0, 0, 0, 0);
-    if (valid) ch = chunks[ci];
+    int4 ch = make_int4(0, 0, 0, 0), ch1 = make_int4(0, 0, 0, 0);
+    if (valid) {
+        ch = chunks[2 * (int64_t)ci];
+        ch1 = chunks[2 * (int64_t)ci + 1];
+    }
     const int rb = ch.x, nr = ch.y, E = ch.w;  // rows rb .. rb+nr-1 (first and last non-empty in this band), E edges
     const int64_t B = ch.z;
     const int32_t *colp = col_bm + B;
     const float *valp = val_bm ? val_bm + B : nullptr;
-    // Lane i of the group holds rowptr[rb+i] relative to the chunk's first edge (lanes >= nr hold the end).
+    // Lane i of the group holds the offset of row rb+i relative to the chunk's first edge (lanes >= nr hold the end).
     int rel = 0;
-    if (valid) rel = (int)(rowptr_b[rb + (lig < nr ? lig : nr)] - B);
+    if (valid) {
+        const int idx = lig < nr ? lig : nr;
+        const uint32_t word = (uint32_t)(idx < 4 ? ch1.x : idx < 8 ? ch1.y : ch1.z);
+        rel = nr == 1 ? (idx == 0 ? 0 : E) : (int)((word >> (8 * (idx & 3))) & 255u);
+    }
     const int rel_next = __shfl(rel, lane + 1 < 64 ? lane + 1 : 63);
     const unsigned long long bal = __ballot(valid && lig < nr && rel_next > rel);
     const uint32_t mask = (uint32_t)(bal >> gbase) & ((1u << kBandRows) - 1u);  // bit i: row rb+i has edges in this band
@@ -503,20 +521,61 @@ __global__ __launch_bounds__(kBlock) void spmm_band_kernel(
         // This lane's column of the tile.  Lanes that own nothing point at column 0 and never write (a write
         // through "their" offset would land in the next row or in the staged pairs).
         float *tcol = tile + (act ? lig * 4 : 0);
-        // ---- phase 1: old out values of the chunk's rows -> LDS tile -------------------------------------
-        if (act) {
-            for (int r0 = 0; r0 < nr; r0 += 6) {
-                float old[6][4];
+        // ---- phase 1: one batch of loads: old out values of the chunk's rows, the first kBandEdges pairs ----------
+        const int se0 = E < kBandEdges ? E : kBandEdges;
+        {
+            float old[kBandRows][4];
+            if (act) {
 #pragma unroll
-                for (int k = 0; k < 6; ++k) {
-                    const int r = r0 + k < nr ? r0 + k : nr - 1;
+                for (int k = 0; k < kBandRows; ++k) {
+                    const int r = k < nr ? k : nr - 1;
                     out_load<EVEN>(old[k], out + (int64_t)(rb + r) * ldo + off, nf);
                 }
+            }
+            // Four pairs per lane and load.  The window below gathers up to U pairs past the chunk's last one (never
+            // consumed): those are the next edges of the band-major arrays, valid columns all, and the arrays end
+            // in kBandPad + 4 zero entries.
+            int c[kBandKeyRounds][4];
+            float w[kBandKeyRounds][4];
+            if (valid) {
 #pragma unroll
-                for (int k = 0; k < 6; ++k) {
-                    if (r0 + k < nr) *reinterpret_cast<float4 *>(tcol + (r0 + k) * tile_stride) = make_float4(old[k][0], old[k][1], old[k][2], old[k][3]);
+                for (int q = 0; q < kBandKeyRounds; ++q) {
+                    const int i = 4 * lig + 4 * G * q;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) { c[q][e] = 0; w[q][e] = 1.0f; }
+                    if (i < se0 + U) {
+                        typedef int i4 __attribute__((ext_vector_type(4), aligned(4)));
+                        typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
+                        const i4 cv = __builtin_nontemporal_load(reinterpret_cast<const i4 *>(colp + i));
+                        c[q][0] = cv.x; c[q][1] = cv.y; c[q][2] = cv.z; c[q][3] = cv.w;
+                        if (valp) {
+                            const f4 wv4 = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(valp + i));
+                            w[q][0] = wv4.x; w[q][1] = wv4.y; w[q][2] = wv4.z; w[q][3] = wv4.w;
+                        }
+                    }
                 }
             }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // the previous tile's LDS reads are done
+            if (act) {
+#pragma unroll
+                for (int k = 0; k < kBandRows; ++k) {
+                    if (k < nr) *reinterpret_cast<float4 *>(tcol + k * tile_stride) = make_float4(old[k][0], old[k][1], old[k][2], old[k][3]);
+                }
+            }
+            if (valid) {
+#pragma unroll
+                for (int q = 0; q < kBandKeyRounds; ++q) {
+                    const int i = 4 * lig + 4 * G * q;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (i + e < se0 + U) {
+                            lkey[i + e] = OFF32 ? (int)((uint32_t)c[q][e] * (uint32_t)slice_pad * 4u) : c[q][e];
+                            lval[i + e] = w[q][e];
+                        }
+                    }
+                }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         }
         // ---- phase 2: gathers ------------------------------------------------------------------------------
         if (valid) {
@@ -530,39 +589,20 @@ __global__ __launch_bounds__(kBlock) void spmm_band_kernel(
             // order: a wavefront-level fence is all the staging needs.
             for (int seg = 0; seg < E; seg += kBandEdges) {
                 const int se = E - seg < kBandEdges ? E - seg : kBandEdges;
-                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-                // four pairs per lane and load (these are the only loads of the gather phase that miss the L2, and a
-                // miss delays every gather queued behind it); U entries of padding repeat the last pair, so the
-                // window below never clamps an index
-                for (int i = 4 * lig; i < se + U; i += 4 * G) {
-                    int c[4];
-                    float w[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-                    if (i + 4 <= se) {
-                        typedef int i4 __attribute__((ext_vector_type(4), aligned(4)));
-                        typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
-                        const i4 cv = __builtin_nontemporal_load(reinterpret_cast<const i4 *>(colp + seg + i));
-                        c[0] = cv.x; c[1] = cv.y; c[2] = cv.z; c[3] = cv.w;
-                        if (valp) {
-                            const f4 wv4 = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(valp + seg + i));
-                            w[0] = wv4.x; w[1] = wv4.y; w[2] = wv4.z; w[3] = wv4.w;
-                        }
-                    } else {
+                if (seg > 0) {   // a later round of a row longer than kBandEdges: stage its pairs now
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                    for (int i = 4 * lig; i < se + U; i += 4 * G) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const int k = i + e < se ? i + e : se - 1;
-                            c[e] = __builtin_nontemporal_load(colp + seg + k);
-                            if (valp) w[e] = __builtin_nontemporal_load(valp + seg + k);
+                            if (i + e < se + U) {
+                                const int cc = __builtin_nontemporal_load(colp + seg + i + e);
+                                lkey[i + e] = OFF32 ? (int)((uint32_t)cc * (uint32_t)slice_pad * 4u) : cc;
+                                lval[i + e] = valp ? __builtin_nontemporal_load(valp + seg + i + e) : 1.0f;
+                            }
                         }
                     }
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        if (i + e < se + U) {
-                            lkey[i + e] = OFF32 ? (int)((uint32_t)c[e] * (uint32_t)slice_pad * 4u) : c[e];
-                            lval[i + e] = w[e];
-                        }
-                    }
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                 }
-                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                 // A rolling window of U gathers: slot u is refilled with the edge U further on as soon as its value
                 // has been consumed, so U - 1 gathers are in flight at all times (loads return in order).
                 float4 xv[U];
@@ -1109,16 +1149,15 @@ static int scratch_for_current_device(float **out) {
 // The matrix cut into column bands, each band a CSR matrix of its own (see spmm_band_kernel).
 struct BandSchedule {
     int band_cols = 0, n_bands = 0;
-    int32_t *rowptr_bm = nullptr;      // [n_bands * (M+1)] absolute offsets into col_bm / val_bm
-    int32_t *col_bm = nullptr;         // [nnz] columns, band-major
+    int32_t *col_bm = nullptr;         // [nnz] columns, band-major (+ kBandPad + 4 zero entries)
     int32_t *eperm_bm = nullptr;       // [nnz] CSR index of each band-major edge
     float *val_bm = nullptr;           // [nnz] edge values in band-major order
     uint64_t val_gen = 0;              // plan bind generation val_bm was filled under (0 = not from a bound array)
     int64_t M = 0, K = 0;
-    int4 *chunks = nullptr;            // all bands' chunks, band after band: (first row, rows, first edge, edges)
-    std::vector<int64_t> chunk_off;    // [n_bands + 1] each band's range in chunks
+    int4 *chunks = nullptr;            // all bands' chunk records (two int4 each, see spmm_band_kernel), band after band
+    std::vector<int64_t> chunk_off;    // [n_bands + 1] each band's range of chunks
     ~BandSchedule() {
-        (void)hipFree(rowptr_bm); (void)hipFree(col_bm); (void)hipFree(eperm_bm); (void)hipFree(val_bm);
+        (void)hipFree(col_bm); (void)hipFree(eperm_bm); (void)hipFree(val_bm);
         (void)hipFree(chunks);
     }
 };
@@ -1522,9 +1561,18 @@ static int band_build_chunks(BandSchedule *bs, const std::vector<int32_t> &h_row
                 edges += d;
                 ++m;
             }
-            out.push_back(make_int4((int)start, (int)(last - start + 1), rp[start], rp[last + 1] - rp[start]));
+            const int nr = (int)(last - start + 1);
+            uint32_t w[3] = {0, 0, 0};   // offsets of rows start .. start + nr relative to the first edge, one byte each
+            if (nr > 1) {
+                for (int i = 0; i <= nr; ++i) {
+                    const uint32_t rel = (uint32_t)(rp[start + i] - rp[start]);   // <= cap <= 255
+                    w[i >> 2] |= rel << (8 * (i & 3));
+                }
+            }
+            out.push_back(make_int4((int)start, nr, rp[start], rp[last + 1] - rp[start]));
+            out.push_back(make_int4((int)w[0], (int)w[1], (int)w[2], 0));
         }
-        bs->chunk_off[(size_t)b + 1] = (int64_t)out.size();
+        bs->chunk_off[(size_t)b + 1] = (int64_t)(out.size() / 2);
     }
     if (!out.empty()) {
         SGNN_HIP_CHECK(hipMalloc(&bs->chunks, sizeof(int4) * out.size()));
@@ -1567,13 +1615,18 @@ static int band_build(sgnn_spmm_plan *p, int band_cols, int n_bands, hipStream_t
         row[M] = (int32_t)run;
     }
     if (run != nnz) return fail(SGNN_ERR_RANGE, "band schedule: %lld of %lld edges fall into the bands", (long long)run, (long long)nnz);
-    SGNN_HIP_CHECK(hipMalloc(&bs->rowptr_bm, sizeof(int32_t) * rp.size()));
-    SGNN_HIP_CHECK(hipMemcpyAsync(bs->rowptr_bm, rp.data(), sizeof(int32_t) * rp.size(), hipMemcpyHostToDevice, st));
-    SGNN_HIP_CHECK(hipMalloc(&bs->col_bm, sizeof(int32_t) * (size_t)nnz));
+    DevTmp<int32_t> rowptr_bm;   // [n_bands * (M+1)] where each (band, row) starts in the band-major arrays
+    SGNN_HIP_CHECK(hipMalloc(&rowptr_bm.p, sizeof(int32_t) * rp.size()));
+    SGNN_HIP_CHECK(hipMemcpyAsync(rowptr_bm.p, rp.data(), sizeof(int32_t) * rp.size(), hipMemcpyHostToDevice, st));
+    // the kernel reads up to kBandPad + 3 entries past a chunk's last pair: zero entries (column 0) close the arrays
+    const size_t tail = (size_t)kBandPad + 4;
+    SGNN_HIP_CHECK(hipMalloc(&bs->col_bm, sizeof(int32_t) * ((size_t)nnz + tail)));
     SGNN_HIP_CHECK(hipMalloc(&bs->eperm_bm, sizeof(int32_t) * (size_t)nnz));
-    SGNN_HIP_CHECK(hipMalloc(&bs->val_bm, sizeof(float) * (size_t)nnz));
+    SGNN_HIP_CHECK(hipMalloc(&bs->val_bm, sizeof(float) * ((size_t)nnz + tail)));
+    SGNN_HIP_CHECK(hipMemsetAsync(bs->col_bm + nnz, 0, sizeof(int32_t) * tail, st));
+    SGNN_HIP_CHECK(hipMemsetAsync(bs->val_bm + nnz, 0, sizeof(float) * tail, st));
     hipLaunchKernelGGL(band_scatter_kernel, dim3((uint32_t)((M + 15) / 16)), dim3(kBlock), 0, st, p->rowptr, p->col, M, n_bands,
-                       band_cols, lo.p, bs->rowptr_bm, bs->col_bm, bs->eperm_bm);
+                       band_cols, lo.p, rowptr_bm.p, bs->col_bm, bs->eperm_bm);
     SGNN_HIP_CHECK(hipGetLastError());
     SGNN_HIP_CHECK(hipStreamSynchronize(st));
     const int rc = band_build_chunks(bs.get(), rp, st);
@@ -1587,7 +1640,7 @@ static int launch_band(const BandSchedule *bs, const BandShape &sh, int b, const
                        int F, int64_t ldo, hipStream_t st, int device) {
     const int64_t c0 = bs->chunk_off[(size_t)b], c1 = bs->chunk_off[(size_t)b + 1];
     if (c1 == c0) return SGNN_OK;
-    const int gpb = (kBlock / 64) * (64 / sh.G);  // lane groups per workgroup
+    const int gpb = (kBandBlock / 64) * (64 / sh.G);  // lane groups per workgroup
     const int n_rg = kNumXCD / sh.n_slices;
     const int64_t wgs = (c1 - c0 + gpb - 1) / gpb;
     const uint32_t nb = (uint32_t)((wgs + n_rg - 1) / n_rg) * kNumXCD;
@@ -1607,8 +1660,8 @@ static int launch_band(const BandSchedule *bs, const BandShape &sh, int b, const
             allowed = lds;
         }
     }
-    hipLaunchKernelGGL(kernel, dim3(nb), dim3(kBlock), lds, st, bs->rowptr_bm + (size_t)b * (size_t)(bs->M + 1), bs->col_bm, val_bm,
-                       xs, bs->K, out, bs->chunks + c0, (int)(c1 - c0), F, ldo, sh.slice_floats, sh.slice_pad, sh.n_slices, sh.G);
+    hipLaunchKernelGGL(kernel, dim3(nb), dim3(kBandBlock), lds, st, bs->col_bm, val_bm, xs, bs->K, out, bs->chunks + 2 * c0,
+                       (int)(c1 - c0), F, ldo, sh.slice_floats, sh.slice_pad, sh.n_slices, sh.G);
     return SGNN_OK;
 }
 

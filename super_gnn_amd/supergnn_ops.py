@@ -221,8 +221,9 @@ class SpmmPlan:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
-            _destroy_plan_handle(h)
+        destroy = _destroy_plan_handle    # None once the interpreter has begun to tear the module down
+        if h and destroy is not None:
+            destroy(h)
 
 
 # Plan handles whose owner died while a stream was being captured into a HIP graph.  Destroying a plan frees
