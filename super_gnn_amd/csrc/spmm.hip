@@ -365,18 +365,23 @@ __global__ __launch_bounds__(kBlock) void spmm_short_kernel(
 // order with one fma per edge starting from the old value: with column-sorted rows the result is the
 // reference's, bit for bit, whatever the row length.
 // ------------------------------------------------------------------------------------------------
-// Rows per chunk and staged (row offset, val) pairs per chunk of the band kernel.
+// Upper limits of a chunk of the band kernel: rows, and staged (row offset, val) pairs.  What a launch uses is
+// decided from the lane-group shape and the LDS it leaves (band_chunk_caps).
 #ifndef SGNN_BAND_ROWS
-#define SGNN_BAND_ROWS 11
+#define SGNN_BAND_ROWS 16
 #endif
 #ifndef SGNN_BAND_EDGES
-#define SGNN_BAND_EDGES 240
+#define SGNN_BAND_EDGES 448
 #endif
 #ifndef SGNN_BAND_U
 #define SGNN_BAND_U 8
 #endif
 constexpr int kBandRows = SGNN_BAND_ROWS;
 constexpr int kBandEdges = SGNN_BAND_EDGES;
+// With edge values a chunk keeps twice the words per edge in flight and in LDS: lower limits keep the kernel's
+// registers (all of a chunk's HBM loads are in flight at once) within two waves per SIMD.
+constexpr int kBandRowsWeighted = kBandRows < 12 ? kBandRows : 12;
+constexpr int kBandEdgesWeighted = kBandEdges < 320 ? kBandEdges : 320;
 constexpr int kBandWindow = SGNN_BAND_U;  // gathers in flight per lane group
 constexpr int kBandPad = 16;              // staging entries past the last pair (>= the gather window)
 #ifndef SGNN_BAND_BLOCK
@@ -384,7 +389,10 @@ constexpr int kBandPad = 16;              // staging entries past the last pair 
 #endif
 constexpr int kBandBlock = SGNN_BAND_BLOCK;  // threads per workgroup of the band kernel
 static_assert(kBandWindow <= kBandPad, "gather window wider than the staging pad");
-__host__ __device__ constexpr int band_group_floats(int tile_stride) { return kBandRows * tile_stride + 2 * (kBandEdges + kBandPad); }
+// LDS floats of one lane group: the output tile, the staged row offsets of the edges and, for a weighted matrix, their values.
+__host__ __device__ constexpr int band_group_floats(int tile_stride, int rows_cap, int edge_cap, bool weighted) {
+    return rows_cap * tile_stride + (weighted ? 2 : 1) * (edge_cap + kBandPad);
+}
 
 // The dense operand restaged for the band kernel: xs[slice][column][slice_pad floats], slice_pad a multiple of
 // 16 floats.  Every row of a slice then starts on a 64-byte boundary, a group of slice_pad / 4 lanes reads it
@@ -447,11 +455,12 @@ __device__ __forceinline__ void out_store(float *p, const float (&r)[4], int nf)
     }
 }
 
-// A chunk is a run of consecutive rows of one band: at most kBandRows rows and kBandEdges edges (a single row may
-// have more).  Its record is two int4: (first row, rows, first edge, edges) and the rows' edge offsets relative
-// to the first edge, one byte each (entries 0 .. rows; unused for a one-row chunk, whose offsets are 0 and edges).
-static_assert(kBandEdges <= 255 && kBandRows <= 11, "row offsets of a chunk are stored as bytes, twelve per record");
-constexpr int kBandKeyRounds = (kBandEdges + kBandPad + 63) / 64;  // staging loads per lane: four pairs per load, >= 16 lanes
+// A chunk is a run of consecutive rows of one band: at most rows_cap rows and edge_cap edges (a single row may
+// have more).  Its record is four int4: (first row, rows, first edge, edges), then 24 16-bit edge offsets
+// relative to the first edge: entry i belongs to row i of the chunk, entries from `rows` on hold the number of
+// edges (a one-row chunk may have more than 65535 edges: its two offsets are taken from the header instead).
+constexpr int kBandOffsets = 24;
+static_assert(kBandEdges <= 65535 && kBandRows < kBandOffsets && kBandRows <= 16, "row offsets of a chunk are 16-bit, 24 per record");
 
 // One lane group per chunk.  A group is
 // G = slice_pad / 4 lanes (any value from 16 to 64, not only powers of two), one float4 of the restaged slice
@@ -468,13 +477,15 @@ constexpr int kBandKeyRounds = (kBandEdges + kBandPad + 63) / 64;  // staging lo
 //      gathers would stall every gather behind it;
 //   3. the tile rows that received edges are written back.
 // A tile column belongs to one lane and a group to one wavefront: the kernel has no workgroup barrier.
-template <bool EVEN, bool OFF32>
-__global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
+template <bool EVEN, bool OFF32, bool WEIGHTED>
+__global__ __launch_bounds__(kBandBlock) __attribute__((amdgpu_waves_per_eu(2))) void spmm_band_kernel(
     const int32_t *__restrict__ col_bm, const float *__restrict__ val_bm, const float *__restrict__ xs, int64_t K,
     float *__restrict__ out, const int4 *__restrict__ chunks, int n_chunks, int F, int64_t ldo, int slice_floats,
-    int slice_pad, int n_slices, int G) {
+    int slice_pad, int n_slices, int G, int rows_cap, int edge_cap) {
     extern __shared__ float band_lds[];
     constexpr int U = kBandWindow;
+    constexpr int kRows = WEIGHTED ? kBandRowsWeighted : kBandRows;
+    constexpr int kKeyRounds = ((WEIGHTED ? kBandEdgesWeighted : kBandEdges) + kBandPad + 63) / 64;
     const int tile_stride = G * 4;
     const int gpw = 64 / G;                       // groups per wavefront
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -487,30 +498,28 @@ __global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
     const int f_lo = slice * slice_floats;        // first feature column of this slice
     const int vpr = slice_pad / 4;                // float4 per restaged row
     const bool valid = gsub < gpw && ci < n_chunks && f_lo < F;
-    float *tile = band_lds + (size_t)(gsub < gpw ? gid : 0) * band_group_floats(tile_stride);
-    int *lkey = reinterpret_cast<int *>(tile + kBandRows * tile_stride);
-    float *lval = reinterpret_cast<float *>(lkey + kBandEdges + kBandPad);
+    float *tile = band_lds + (size_t)(gsub < gpw ? gid : 0) * band_group_floats(tile_stride, rows_cap, edge_cap, WEIGHTED);
+    int *lkey = reinterpret_cast<int *>(tile + rows_cap * tile_stride);
+    float *lval = reinterpret_cast<float *>(lkey + edge_cap + kBandPad);   // only there (and only used) for a weighted matrix
     const float *xslice = xs + (int64_t)slice * K * slice_pad;
 
-    int4 ch = make_int4(0, 0, 0, 0), ch1 = make_int4(0, 0, 0, 0);
+    int4 ch = make_int4(0, 0, 0, 0);
+    int rel16 = 0;
     if (valid) {
-        ch = chunks[2 * (int64_t)ci];
-        ch1 = chunks[2 * (int64_t)ci + 1];
+        const int4 *rec = chunks + 4 * (int64_t)ci;
+        ch = rec[0];
+        rel16 = reinterpret_cast<const uint16_t *>(rec + 1)[lig < kBandOffsets - 1 ? lig : kBandOffsets - 1];
     }
     const int rb = ch.x, nr = ch.y, E = ch.w;  // rows rb .. rb+nr-1 (first and last non-empty in this band), E edges
     const int64_t B = ch.z;
     const int32_t *colp = col_bm + B;
-    const float *valp = val_bm ? val_bm + B : nullptr;
+    const float *valp = WEIGHTED ? val_bm + B : nullptr;
     // Lane i of the group holds the offset of row rb+i relative to the chunk's first edge (lanes >= nr hold the end).
     int rel = 0;
-    if (valid) {
-        const int idx = lig < nr ? lig : nr;
-        const uint32_t word = (uint32_t)(idx < 4 ? ch1.x : idx < 8 ? ch1.y : ch1.z);
-        rel = nr == 1 ? (idx == 0 ? 0 : E) : (int)((word >> (8 * (idx & 3))) & 255u);
-    }
+    if (valid) rel = nr == 1 ? (lig == 0 ? 0 : E) : rel16;
     const int rel_next = __shfl(rel, lane + 1 < 64 ? lane + 1 : 63);
     const unsigned long long bal = __ballot(valid && lig < nr && rel_next > rel);
-    const uint32_t mask = (uint32_t)(bal >> gbase) & ((1u << kBandRows) - 1u);  // bit i: row rb+i has edges in this band
+    const uint32_t mask = (uint32_t)(bal >> gbase) & ((1u << rows_cap) - 1u);  // bit i: row rb+i has edges in this band
 
     for (int t0 = 0; t0 < vpr; t0 += G) {             // slices wider than 64 float4 are walked in tiles
         const int vi = t0 + lig;                      // this lane's float4 of the slice
@@ -521,13 +530,13 @@ __global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
         // This lane's column of the tile.  Lanes that own nothing point at column 0 and never write (a write
         // through "their" offset would land in the next row or in the staged pairs).
         float *tcol = tile + (act ? lig * 4 : 0);
-        // ---- phase 1: one batch of loads: old out values of the chunk's rows, the first kBandEdges pairs ----------
-        const int se0 = E < kBandEdges ? E : kBandEdges;
+        // ---- phase 1: one batch of loads: old out values of the chunk's rows, the first edge_cap pairs -------------
+        const int se0 = E < edge_cap ? E : edge_cap;
         {
-            float old[kBandRows][4];
+            float old[kRows][4];
             if (act) {
 #pragma unroll
-                for (int k = 0; k < kBandRows; ++k) {
+                for (int k = 0; k < kRows; ++k) {
                     const int r = k < nr ? k : nr - 1;
                     out_load<EVEN>(old[k], out + (int64_t)(rb + r) * ldo + off, nf);
                 }
@@ -535,11 +544,11 @@ __global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
             // Four pairs per lane and load.  The window below gathers up to U pairs past the chunk's last one (never
             // consumed): those are the next edges of the band-major arrays, valid columns all, and the arrays end
             // in kBandPad + 4 zero entries.
-            int c[kBandKeyRounds][4];
-            float w[kBandKeyRounds][4];
+            int c[kKeyRounds][4];
+            float w[kKeyRounds][4];
             if (valid) {
 #pragma unroll
-                for (int q = 0; q < kBandKeyRounds; ++q) {
+                for (int q = 0; q < kKeyRounds; ++q) {
                     const int i = 4 * lig + 4 * G * q;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) { c[q][e] = 0; w[q][e] = 1.0f; }
@@ -548,7 +557,7 @@ __global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
                         typedef float f4 __attribute__((ext_vector_type(4), aligned(4)));
                         const i4 cv = __builtin_nontemporal_load(reinterpret_cast<const i4 *>(colp + i));
                         c[q][0] = cv.x; c[q][1] = cv.y; c[q][2] = cv.z; c[q][3] = cv.w;
-                        if (valp) {
+                        if constexpr (WEIGHTED) {
                             const f4 wv4 = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(valp + i));
                             w[q][0] = wv4.x; w[q][1] = wv4.y; w[q][2] = wv4.z; w[q][3] = wv4.w;
                         }
@@ -558,19 +567,19 @@ __global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // the previous tile's LDS reads are done
             if (act) {
 #pragma unroll
-                for (int k = 0; k < kBandRows; ++k) {
+                for (int k = 0; k < kRows; ++k) {
                     if (k < nr) *reinterpret_cast<float4 *>(tcol + k * tile_stride) = make_float4(old[k][0], old[k][1], old[k][2], old[k][3]);
                 }
             }
             if (valid) {
 #pragma unroll
-                for (int q = 0; q < kBandKeyRounds; ++q) {
+                for (int q = 0; q < kKeyRounds; ++q) {
                     const int i = 4 * lig + 4 * G * q;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         if (i + e < se0 + U) {
                             lkey[i + e] = OFF32 ? (int)((uint32_t)c[q][e] * (uint32_t)slice_pad * 4u) : c[q][e];
-                            lval[i + e] = w[q][e];
+                            if constexpr (WEIGHTED) lval[i + e] = w[q][e];
                         }
                     }
                 }
@@ -584,12 +593,12 @@ __global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
             int cur = __builtin_ctz(mask);
             int cur_end = __shfl(rel, gbase + cur + 1);
             float4 acc = *reinterpret_cast<const float4 *>(tcol + cur * tile_stride);
-            // The chunk's (row offset, val) pairs are staged in LDS, kBandEdges at a time (more than one round only
+            // The chunk's (row offset, val) pairs are staged in LDS, edge_cap at a time (more than one round only
             // for a row longer than that).  A group lives inside one wavefront, whose LDS operations execute in
             // order: a wavefront-level fence is all the staging needs.
-            for (int seg = 0; seg < E; seg += kBandEdges) {
-                const int se = E - seg < kBandEdges ? E - seg : kBandEdges;
-                if (seg > 0) {   // a later round of a row longer than kBandEdges: stage its pairs now
+            for (int seg = 0; seg < E; seg += edge_cap) {
+                const int se = E - seg < edge_cap ? E - seg : edge_cap;
+                if (seg > 0) {   // a later round of a row longer than edge_cap: stage its pairs now
                     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                     for (int i = 4 * lig; i < se + U; i += 4 * G) {
 #pragma unroll
@@ -597,7 +606,7 @@ __global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
                             if (i + e < se + U) {
                                 const int cc = __builtin_nontemporal_load(colp + seg + i + e);
                                 lkey[i + e] = OFF32 ? (int)((uint32_t)cc * (uint32_t)slice_pad * 4u) : cc;
-                                lval[i + e] = valp ? __builtin_nontemporal_load(valp + seg + i + e) : 1.0f;
+                                if constexpr (WEIGHTED) lval[i + e] = __builtin_nontemporal_load(valp + seg + i + e);
                             }
                         }
                     }
@@ -621,14 +630,15 @@ __global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
                         cur_end = __shfl(rel, gbase + cur + 1);
                         acc = *reinterpret_cast<const float4 *>(tcol + cur * tile_stride);
                     }
-                    acc.x = fmaf(wv[u], xv[u].x, acc.x);
-                    acc.y = fmaf(wv[u], xv[u].y, acc.y);
-                    acc.z = fmaf(wv[u], xv[u].z, acc.z);
-                    acc.w = fmaf(wv[u], xv[u].w, acc.w);
+                    const float wu = WEIGHTED ? wv[u] : 1.0f;   // fma(1, x, acc) is the chain the reference computes with unit weights
+                    acc.x = fmaf(wu, xv[u].x, acc.x);
+                    acc.y = fmaf(wu, xv[u].y, acc.y);
+                    acc.z = fmaf(wu, xv[u].z, acc.z);
+                    acc.w = fmaf(wu, xv[u].w, acc.w);
                 };
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    wv[u] = lval[u];
+                    if constexpr (WEIGHTED) wv[u] = lval[u];
                     gather(u, lkey[u]);
                 }
                 int base = 0;
@@ -642,12 +652,12 @@ __global__ __launch_bounds__(kBandBlock) void spmm_band_kernel(
 #pragma unroll
                     for (int u = 0; u < U; ++u) {  // the next round's pairs, read from LDS ahead of their use
                         kn[u] = lk[u];
-                        wn[u] = lv[u];
+                        if constexpr (WEIGHTED) wn[u] = lv[u];
                     }
 #pragma unroll
                     for (int u = 0; u < U; ++u) {
                         consume(seg + base + u, u);
-                        wv[u] = wn[u];
+                        if constexpr (WEIGHTED) wv[u] = wn[u];
                         gather(u, kn[u]);
                     }
                 }
@@ -1154,11 +1164,18 @@ struct BandSchedule {
     float *val_bm = nullptr;           // [nnz] edge values in band-major order
     uint64_t val_gen = 0;              // plan bind generation val_bm was filled under (0 = not from a bound array)
     int64_t M = 0, K = 0;
-    int4 *chunks = nullptr;            // all bands' chunk records (two int4 each, see spmm_band_kernel), band after band
-    std::vector<int64_t> chunk_off;    // [n_bands + 1] each band's range of chunks
+    std::vector<int32_t> h_rowptr_bm;  // host: [n_bands * (M+1)] where each (band, row) starts in the band-major arrays
+    // The bands cut into chunks, for one pair of limits (rows, edges per chunk); a launch picks the limits from
+    // its lane-group shape and from whether edge values are staged, so a schedule may hold more than one list.
+    struct ChunkList {
+        int rows_cap = 0, edge_cap = 0;
+        int4 *chunks = nullptr;            // all bands' chunk records (four int4 each, see spmm_band_kernel), band after band
+        std::vector<int64_t> chunk_off;    // [n_bands + 1] each band's range of chunks
+    };
+    std::vector<ChunkList> lists;
     ~BandSchedule() {
         (void)hipFree(col_bm); (void)hipFree(eperm_bm); (void)hipFree(val_bm);
-        (void)hipFree(chunks);
+        for (ChunkList &l : lists) (void)hipFree(l.chunks);
     }
 };
 
@@ -1538,47 +1555,52 @@ static int band_rows_sorted(sgnn_spmm_plan *p, hipStream_t st, bool *sorted) {
     return SGNN_OK;
 }
 
-// The chunk list of every band: consecutive rows, at most kBandRows rows and kBandEdges edges (one row may have
-// more), first and last row non-empty in the band.
-static int band_build_chunks(BandSchedule *bs, const std::vector<int32_t> &h_rowptr_bm, hipStream_t st) {
-    // a chunk's (col, val) pairs should fit the kernel's staging area; only a single row longer than that spills
-    int cap = env_int("SGNN_SPMM_BAND_CHUNK_EDGES", 0);
-    if (cap <= 0 || cap > kBandEdges) cap = kBandEdges;
+// The chunk list of every band for the given limits: consecutive rows, at most rows_cap rows and edge_cap edges
+// (one row may have more), first and last row non-empty in the band.
+static int band_build_chunks(BandSchedule *bs, int rows_cap, int edge_cap, hipStream_t st, const BandSchedule::ChunkList **res) {
     const int64_t M = bs->M;
-    std::vector<int4> out;
-    bs->chunk_off.assign((size_t)bs->n_bands + 1, 0);
+    std::vector<int4> out;   // four per chunk
+    BandSchedule::ChunkList list;
+    list.rows_cap = rows_cap;
+    list.edge_cap = edge_cap;
+    list.chunk_off.assign((size_t)bs->n_bands + 1, 0);
     for (int b = 0; b < bs->n_bands; ++b) {
-        const int32_t *rp = h_rowptr_bm.data() + (size_t)b * (size_t)(M + 1);
+        const int32_t *rp = bs->h_rowptr_bm.data() + (size_t)b * (size_t)(M + 1);
         int64_t m = 0;
         while (m < M) {
             if (rp[m + 1] == rp[m]) { ++m; continue; }
             const int64_t start = m;
             int64_t last = m, edges = 0;
-            while (m < M && m - start < kBandRows) {
+            while (m < M && m - start < rows_cap) {
                 const int64_t d = rp[m + 1] - rp[m];
-                if (m > start && edges + d > cap) break;
+                if (m > start && edges + d > edge_cap) break;
                 if (d > 0) last = m;
                 edges += d;
                 ++m;
             }
             const int nr = (int)(last - start + 1);
-            uint32_t w[3] = {0, 0, 0};   // offsets of rows start .. start + nr relative to the first edge, one byte each
-            if (nr > 1) {
-                for (int i = 0; i <= nr; ++i) {
-                    const uint32_t rel = (uint32_t)(rp[start + i] - rp[start]);   // <= cap <= 255
-                    w[i >> 2] |= rel << (8 * (i & 3));
-                }
+            const int64_t E = rp[last + 1] - rp[start];
+            uint32_t w[kBandOffsets / 2] = {};   // 16-bit offsets of the chunk's rows, entries >= nr hold the edge count
+            for (int i = 0; i < kBandOffsets; ++i) {
+                const int64_t rel = i < nr ? rp[start + i] - rp[start] : E;
+                w[i >> 1] |= (uint32_t)(rel & 0xffff) << (16 * (i & 1));   // (more than 65535 only in a one-row chunk)
             }
-            out.push_back(make_int4((int)start, nr, rp[start], rp[last + 1] - rp[start]));
-            out.push_back(make_int4((int)w[0], (int)w[1], (int)w[2], 0));
+            out.push_back(make_int4((int)start, nr, rp[start], (int)E));
+            for (int q = 0; q < 3; ++q) out.push_back(make_int4((int)w[4 * q], (int)w[4 * q + 1], (int)w[4 * q + 2], (int)w[4 * q + 3]));
         }
-        bs->chunk_off[(size_t)b + 1] = (int64_t)(out.size() / 2);
+        list.chunk_off[(size_t)b + 1] = (int64_t)(out.size() / 4);
     }
     if (!out.empty()) {
-        SGNN_HIP_CHECK(hipMalloc(&bs->chunks, sizeof(int4) * out.size()));
-        SGNN_HIP_CHECK(hipMemcpyAsync(bs->chunks, out.data(), sizeof(int4) * out.size(), hipMemcpyHostToDevice, st));
-        SGNN_HIP_CHECK(hipStreamSynchronize(st));
+        SGNN_HIP_CHECK(hipMalloc(&list.chunks, sizeof(int4) * out.size()));
+        const hipError_t e = hipMemcpyAsync(list.chunks, out.data(), sizeof(int4) * out.size(), hipMemcpyHostToDevice, st);
+        const hipError_t e2 = e == hipSuccess ? hipStreamSynchronize(st) : e;
+        if (e2 != hipSuccess) {
+            (void)hipFree(list.chunks);
+            SGNN_HIP_CHECK(e2);
+        }
     }
+    bs->lists.push_back(std::move(list));
+    *res = &bs->lists.back();
     return SGNN_OK;
 }
 
@@ -1629,26 +1651,50 @@ static int band_build(sgnn_spmm_plan *p, int band_cols, int n_bands, hipStream_t
                        band_cols, lo.p, rowptr_bm.p, bs->col_bm, bs->eperm_bm);
     SGNN_HIP_CHECK(hipGetLastError());
     SGNN_HIP_CHECK(hipStreamSynchronize(st));
-    const int rc = band_build_chunks(bs.get(), rp, st);
-    if (rc != SGNN_OK) return rc;
+    bs->h_rowptr_bm = std::move(rp);
     *out = bs.release();
     return SGNN_OK;
 }
 
-template <bool EVEN>
-static int launch_band(const BandSchedule *bs, const BandShape &sh, int b, const float *val_bm, const float *xs, float *out,
-                       int F, int64_t ldo, hipStream_t st, int device) {
-    const int64_t c0 = bs->chunk_off[(size_t)b], c1 = bs->chunk_off[(size_t)b + 1];
+// Limits of a chunk for one launch shape.  Two workgroups per CU is what the kernel's registers allow, so a lane
+// group may use 80 KB / (groups per workgroup) of LDS: its output tile (rows_cap rows of the slice) and the staged
+// edges (4 bytes each, 8 with values).  Large chunks matter: every chunk costs a fixed set-up, measured on the
+// 233 k-node / 114 M-edge graph at F = 602 as time = 14.7 ms + 590 ms / (edges per chunk).  The rows are sized so
+// that a chunk of average rows fills the edge budget.
+struct BandCaps { int rows, edges; };
+static BandCaps band_chunk_caps(const sgnn_spmm_plan *p, const BandShape &sh, bool weighted) {
+    const int gpb = (kBandBlock / 64) * (64 / sh.G);
+    const int64_t budget = (int64_t)80 * 1024 / gpb, row_bytes = (int64_t)sh.G * 16, bpe = weighted ? 8 : 4;
+    const int64_t avg = std::max<int64_t>(1, p->nnz / std::max<int64_t>(1, p->M) / std::max(1, sh.n_bands));
+    const int rows_lim = weighted ? kBandRowsWeighted : kBandRows, edges_lim = weighted ? kBandEdgesWeighted : kBandEdges;
+    const int rows_max = std::min(rows_lim, sh.G - 1);   // lane i of a group holds row i's offset, lane `rows` the end
+    int rows = (int)std::max<int64_t>(1, std::min<int64_t>(rows_max, (budget - kBandPad * bpe) / (row_bytes + bpe * avg)));
+    int edges = 0;
+    for (;; --rows) {
+        edges = (int)std::min<int64_t>(edges_lim, ((budget - rows * row_bytes) / bpe - kBandPad) / 16 * 16);
+        if (edges >= 64 || rows == 1) break;
+    }
+    edges = std::max(edges, 16);
+    const int er = env_int("SGNN_SPMM_BAND_CHUNK_ROWS", 0), ee = env_int("SGNN_SPMM_BAND_CHUNK_EDGES", 0);
+    if (er > 0) rows = std::min(er, rows_max);
+    if (ee > 0) edges = std::min(ee, edges_lim);
+    return BandCaps{rows, edges};
+}
+
+template <bool EVEN, bool WEIGHTED>
+static int launch_band(const BandSchedule *bs, const BandSchedule::ChunkList *cl, const BandShape &sh, int b, const float *val_bm,
+                       const float *xs, float *out, int F, int64_t ldo, hipStream_t st, int device) {
+    const int64_t c0 = cl->chunk_off[(size_t)b], c1 = cl->chunk_off[(size_t)b + 1];
     if (c1 == c0) return SGNN_OK;
     const int gpb = (kBandBlock / 64) * (64 / sh.G);  // lane groups per workgroup
     const int n_rg = kNumXCD / sh.n_slices;
     const int64_t wgs = (c1 - c0 + gpb - 1) / gpb;
     const uint32_t nb = (uint32_t)((wgs + n_rg - 1) / n_rg) * kNumXCD;
-    const size_t lds = sizeof(float) * (size_t)gpb * (size_t)band_group_floats(sh.G * 4);
+    const size_t lds = sizeof(float) * (size_t)gpb * (size_t)band_group_floats(sh.G * 4, cl->rows_cap, cl->edge_cap, WEIGHTED);
     // every restaged row of a slice within 4 GB of the slice's start: 32-bit gather offsets
     // (SGNN_SPMM_BAND_OFF64=1 forces the 64-bit variant so that tests reach it at small sizes)
     const bool off32 = (uint64_t)bs->K * (uint64_t)sh.slice_pad * 4u < ((uint64_t)1 << 32) && env_int("SGNN_SPMM_BAND_OFF64", 0) == 0;
-    auto kernel = off32 ? spmm_band_kernel<EVEN, true> : spmm_band_kernel<EVEN, false>;
+    auto kernel = off32 ? spmm_band_kernel<EVEN, true, WEIGHTED> : spmm_band_kernel<EVEN, false, WEIGHTED>;
     // the dynamic-LDS limit of a kernel is a per-device setting: remember what each device has been told
     static std::mutex mu;
     static size_t lds_allowed[64][2];
@@ -1660,8 +1706,8 @@ static int launch_band(const BandSchedule *bs, const BandShape &sh, int b, const
             allowed = lds;
         }
     }
-    hipLaunchKernelGGL(kernel, dim3(nb), dim3(kBandBlock), lds, st, bs->col_bm, val_bm, xs, bs->K, out, bs->chunks + 2 * c0,
-                       (int)(c1 - c0), F, ldo, sh.slice_floats, sh.slice_pad, sh.n_slices, sh.G);
+    hipLaunchKernelGGL(kernel, dim3(nb), dim3(kBandBlock), lds, st, bs->col_bm, val_bm, xs, bs->K, out, cl->chunks + 4 * c0,
+                       (int)(c1 - c0), F, ldo, sh.slice_floats, sh.slice_pad, sh.n_slices, sh.G, cl->rows_cap, cl->edge_cap);
     return SGNN_OK;
 }
 
@@ -1701,6 +1747,15 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
             p->band_xs_floats = xs_floats;
         }
     }
+    const BandCaps caps = band_chunk_caps(p, sh, val != nullptr);
+    const BandSchedule::ChunkList *cl = nullptr;
+    for (const BandSchedule::ChunkList &l : bs->lists)
+        if (l.rows_cap == caps.rows && l.edge_cap == caps.edges) cl = &l;
+    if (cl == nullptr) {
+        if (!may_build) return SGNN_OK;
+        const int rc = band_build_chunks(bs, caps.rows, caps.edges, st, &cl);
+        if (rc != SGNN_OK) return rc;
+    }
     const float *val_bm = nullptr;
     if (val != nullptr) {
         const bool bound = val == p->bound_val;
@@ -1726,8 +1781,11 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
     {
         ProfScope prof(K_SPMM_BAND, st);
         for (int b = 0; b < bs->n_bands; ++b) {
-            const int rc = sh.even ? launch_band<true>(bs, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device)
-                                   : launch_band<false>(bs, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device);
+            int rc;
+            if (val_bm) rc = sh.even ? launch_band<true, true>(bs, cl, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device)
+                                     : launch_band<false, true>(bs, cl, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device);
+            else rc = sh.even ? launch_band<true, false>(bs, cl, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device)
+                              : launch_band<false, false>(bs, cl, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device);
             if (rc != SGNN_OK) return rc;
         }
     }
