@@ -94,6 +94,30 @@ def test_band_schedule_with_64_bit_gather_offsets(F, monkeypatch):
     assert np.array_equal(out.cpu().numpy(), want)
 
 
+def test_band_schedule_row_with_more_than_65535_edges_in_one_band(monkeypatch):
+    # a chunk's row offsets are 16-bit; a row that long is a chunk of its own and takes its bounds from the header
+    ops = _ops()
+    _force(monkeypatch, 150000)
+    M, K, F = 40, 200000, 16
+    rng = np.random.default_rng(7)
+    deg = rng.integers(0, 30, size=M)
+    deg[17] = 120000
+    deg[18] = 70000
+    rowptr = np.zeros(M + 1, np.int64); np.cumsum(deg, out=rowptr[1:])
+    col = np.concatenate([np.sort(rng.choice(K, size=d, replace=False)) for d in deg]).astype(np.int64)
+    val = rng.random(col.size, dtype=np.float32)
+    x = rng.standard_normal((K, F), dtype=np.float32)
+    init = rng.standard_normal((M, F), dtype=np.float32)
+    dev = torch.device("cuda:0")
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    assert plan.schedule(F)["n_bands"] == 2
+    for v in (val, None):
+        want = init.copy(); orc.spmm_accumulate(rowptr, col, v if v is not None else np.ones_like(val), x, want)
+        out = torch.from_numpy(init.copy()).to(dev)
+        plan.run(torch.from_numpy(v).to(dev) if v is not None else None, torch.from_numpy(x).to(dev), out, accumulate=True)
+        assert np.array_equal(out.cpu().numpy(), want), "weighted" if v is not None else "unit weights"
+
+
 def test_band_schedule_equals_row_class_schedule_and_honours_rebinding(monkeypatch):
     ops = _ops()
     dev = torch.device("cuda:0")
