@@ -131,8 +131,9 @@ int sgnn_spmm_csr_f32(sgnn_spmm_plan *plan, const float *val, const float *x, fl
  *     (different streams, different host threads) race on it.  Calls queued on one stream are safe.
  *     Nothing in the scratch has to start at zero: each call writes every partial it later reads;
  *   - a matrix that sgnn_spmm_plan_schedule reports as band-scheduled runs that schedule here only if an
- *     earlier sgnn_spmm_csr_f32 call has already built it for a width >= F (building allocates); otherwise
- *     the row-class kernels run, whose long rows are summed per piece instead of in one chain. */
+ *     earlier sgnn_spmm_csr_f32 call has already built it for a width >= F and the same kind of weights
+ *     (val given or NULL: the two cut the bands into different chunks); building allocates.  Otherwise the
+ *     row-class kernels run, whose long rows are summed per piece instead of in one chain. */
 int sgnn_spmm_csr_f32_noalloc(sgnn_spmm_plan *plan, const float *val, const float *x, float *out,
                               int64_t F, int64_t ldx, int64_t ldo, int accumulate,
                               const float *row_div, sgnn_stream_t stream);
