@@ -34,12 +34,13 @@ __device__ __forceinline__ float dpp_f(float v) {
 struct OpMinF { __device__ static float f(float a, float b) { return fminf(a, b); } };
 struct OpMaxF { __device__ static float f(float a, float b) { return fmaxf(a, b); } };
 
-// All-reduce over a group of G consecutive lanes (G in {16, 32, 64}); every lane gets the result.
+// All-reduce over a group of G consecutive lanes (G in {8, 16, 32, 64}); every lane gets the result.
 template <int G, typename Op>
 __device__ __forceinline__ float group_allreduce_f(float v) {
     v = Op::f(v, dpp_f<0xB1>(v));
     v = Op::f(v, dpp_f<0x4E>(v));
     v = Op::f(v, dpp_f<0x141>(v));
+    if constexpr (G == 8) return v;
     v = Op::f(v, dpp_f<0x140>(v));
     if constexpr (G == 16) {
         return v;
@@ -63,6 +64,7 @@ __device__ __forceinline__ int group_allmin_i(int v) {
     v = min(v, dpp_i<0xB1>(v));
     v = min(v, dpp_i<0x4E>(v));
     v = min(v, dpp_i<0x141>(v));
+    if constexpr (G == 8) return v;
     v = min(v, dpp_i<0x140>(v));
     if constexpr (G == 16) {
         return v;
@@ -293,25 +295,28 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
-// Fused quantize + pack, row-group layout, one fp32 row per 16 lanes (float4 lanes, F <= 1024).
+// Fused quantize + pack, row-group layout, one fp32 row per L = 16 lanes (float4 lanes, F <= 1024) or,
+// for rows of up to 128 floats, per L = 8 lanes.
 //
-// A 16-lane DPP row owns one fp32 row (NV float4 per lane), so the per-row min/max reductions are
-// four DPP butterfly steps with no cross-row traffic, and the per-row scalars (zero_point, scale,
-// reciprocal) are computed once per lane instead of once per row per lane.  A wavefront handles
-// 4*RL consecutive rows (RL rows per lane, chosen so that every lane keeps >= 4 loads in flight);
-// the four DPP rows hold four consecutive fp32 rows, i.e. exactly the rows that share a packed byte
-// at int2 (two DPP rows at int4), so packing is a shift in each lane followed by an OR across DPP
-// rows.
+// L lanes inside one 16-lane DPP row own one fp32 row (NV float4 per lane), so the per-row min/max
+// reductions are four (three) DPP butterfly steps with no cross-row traffic, and the per-row scalars
+// (zero_point, scale, reciprocal) are computed once per lane instead of once per row per lane.  A wavefront
+// handles 64/L * RL consecutive rows (RL rows per lane, chosen so that every lane keeps >= 4 loads in
+// flight); neighbouring lane groups hold consecutive fp32 rows, i.e. exactly the rows that share a packed
+// byte (four at int2, two at int4), so packing is a shift in each lane followed by an OR across lane
+// groups.  Narrow rows take L = 8: the work per row (reductions, scale, reciprocal, parameter store) is
+// then spread over twice as many elements per lane, which is what limits rows of 64 and 128 floats.
 // ------------------------------------------------------------------------------------------------
-// FULL: F == 64 * NV, every lane's every vector lies inside the row (no per-load lane predicates).
-template <int BITS, int NV, int RL, bool kForceExactDivision, bool FULL = false>
+// FULL: F == 4 * L * NV, every lane's every vector lies inside the row (no per-load lane predicates).
+template <int BITS, int NV, int RL, bool kForceExactDivision, bool FULL = false, int L = 16>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
     const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F,
     int n_units) {
     constexpr int EPB = 8 / BITS;
     constexpr int VEC = 4;
-    const int lane = threadIdx.x & 63, d = lane >> 4, l16 = lane & 15;
+    constexpr int RW = 64 / L;  // fp32 rows of a wavefront per round
+    const int lane = threadIdx.x & 63, d = lane / L, l16 = lane % L;  // lane group (= row) inside the wavefront, lane inside the group
     const int unit = blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
     if (unit >= n_units) return;  // wave-uniform
 
@@ -320,7 +325,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
     int gp[RL];
 #pragma unroll
     for (int rl = 0; rl < RL; ++rl) {
-        const int pr = (unit * RL + rl) * 4 + d;  // row index in the padded (EPB rows per packed row) space
+        const int pr = (unit * RL + rl) * RW + d;  // row index in the padded (EPB rows per packed row) space
         const int g = pr / EPB, k = pr % EPB;
         gp[rl] = g;
         valid[rl] = false;
@@ -336,7 +341,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
     bool act[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        off[v] = (v * 16 + l16) * VEC;
+        off[v] = (v * L + l16) * VEC;
         act[v] = FULL ? true : off[v] < F;
     }
     float xv[RL][NV][VEC];
@@ -367,8 +372,8 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
                 mx = fmaxf(mx, xv[rl][v][k]);
             }
         }
-        mn = group_allreduce_f<16, OpMinF>(mn);
-        mx = group_allreduce_f<16, OpMaxF>(mx);
+        mn = group_allreduce_f<L, OpMinF>(mn);
+        mx = group_allreduce_f<L, OpMaxF>(mx);
         if (mn == 0.0f || mx == 0.0f) {
             // first-occurrence rule for compare-equal zeros (quantization_arm.cpp:98-101)
             int key = INT_MAX;
@@ -379,14 +384,14 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
                 for (int k = VEC - 1; k >= 0; --k)
                     if (xv[rl][v][k] == 0.0f) key = ((off[v] + k) << 1) | (int)(__float_as_uint(xv[rl][v][k]) >> 31);
             }
-            key = group_allmin_i<16>(key);
+            key = group_allmin_i<L>(key);
             const float z = (key & 1) ? -0.0f : 0.0f;
             if (mn == 0.0f) mn = z;
             if (mx == 0.0f) mx = z;
         }
-        // a NaN is sticky only as element 0, which lane 0 of the DPP row holds
+        // a NaN is sticky only as element 0, which lane 0 of the lane group holds
         const unsigned long long nanmask = __ballot(l16 == 0 && xv[rl][0][0] != xv[rl][0][0]);
-        if ((nanmask >> (lane & 48)) & 1ull) {
+        if ((nanmask >> (lane & ~(L - 1))) & 1ull) {
             mn = __int_as_float(0x7fc00000);
             mx = mn;
         }
@@ -451,9 +456,14 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             uint32_t w = words[rl][v] << shift;
-            if constexpr (EPB >= 2) w |= (uint32_t)__shfl_xor((int)w, 16, 64);
-            if constexpr (EPB == 4) w |= (uint32_t)__shfl_xor((int)w, 32, 64);
-            const bool mine = EPB == 1 ? true : EPB == 2 ? ((d & 1) == (v & 1)) : (d == (v & 3));
+            if constexpr (L == 16) {
+                if constexpr (EPB >= 2) w |= (uint32_t)__shfl_xor((int)w, 16, 64);
+                if constexpr (EPB == 4) w |= (uint32_t)__shfl_xor((int)w, 32, 64);
+            } else {  // L == 8: the neighbouring row sits in the other half of the DPP row (row_ror:8 swaps the halves)
+                if constexpr (EPB >= 2) w |= (uint32_t)dpp_i<0x128>((int)w);
+                if constexpr (EPB == 4) w |= (uint32_t)__shfl_xor((int)w, 16, 64);
+            }
+            const bool mine = EPB == 1 ? true : EPB == 2 ? ((d & 1) == (v & 1)) : ((d & 3) == (v & 3));
             if (mine && act[v] && gp[rl] < n_packed)
                 __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(q + (int64_t)gp[rl] * F + off[v]));
         }
@@ -958,22 +968,23 @@ static void launch_rows(const RowsArgs &a, hipStream_t st) {
                            a.x_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
-template <int BITS, int NV>
+template <int BITS, int NV, int L = 16>
 static void launch_quant16(const RowsArgs &a, hipStream_t st) {
     constexpr int RL = NV >= 4 ? 1 : 4 / NV;
     constexpr int EPB = 8 / BITS;
+    constexpr int RW = 64 / L;
     const int64_t padded = (int64_t)a.n_packed * EPB;
-    const int n_units = (int)((padded + 4 * RL - 1) / (4 * RL));
+    const int n_units = (int)((padded + RW * RL - 1) / (RW * RL));
     const int nb = (n_units + kQBlock / 64 - 1) / (kQBlock / 64);
     ProfScope prof(K_QUANT_PACK_ROWS, st);
     if (a.exact_division)
-        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
+        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, true, false, L>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
                            a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
-    else if (a.F == 64 * NV)
-        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
+    else if (a.F == 4 * L * NV)
+        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, true, L>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
                            a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
     else
-        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
+        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
                            a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
@@ -1025,6 +1036,13 @@ template <int BITS, int VEC>
 static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
     if constexpr (VEC == 4) {
         if (a.quantize && a.layout16) {
+            // rows of up to 128 floats: eight lanes per row (SGNN_QUANT_LAYOUT8=0: sixteen, for comparison)
+            static const bool layout8 = [] { const char *e = getenv("SGNN_QUANT_LAYOUT8"); return !(e && e[0] == '0'); }();
+            if (layout8 && (a.F % 32 == 0 || nvec <= 16)) {   // (a ragged 17..31-vector row gains nothing from it)
+                if (nvec <= 8) return launch_quant16<BITS, 1, 8>(a, st);
+                if (nvec <= 16) return launch_quant16<BITS, 2, 8>(a, st);
+                if (nvec <= 32) return launch_quant16<BITS, 4, 8>(a, st);
+            }
             if (nvec <= 16) return launch_quant16<BITS, 1>(a, st);
             if (nvec <= 32) return launch_quant16<BITS, 2>(a, st);
             if (nvec <= 64) return launch_quant16<BITS, 4>(a, st);

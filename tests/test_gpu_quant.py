@@ -229,13 +229,14 @@ def test_facades_and_errors():
                         torch.zeros(0, 2, device="cuda"), 2)
 
 
+@pytest.mark.parametrize("n,F", [(1_000_000, 256), (2_000_000, 128), (4_000_000, 64)])
 @pytest.mark.parametrize("bits", [8, 4, 2])
-def test_full_size_properties(bits):
-    # the sweep's full shape (1M x 256, 10% outlier rows): size-independent properties plus an
-    # exact comparison with the oracle on a strided sample of row groups
+def test_full_size_properties(bits, n, F):
+    # the sweep's full shape (1M x 256, 10% outlier rows) and the same bytes as rows of 128 and 64 floats (the
+    # widths the layers exchange; they take the eight-lanes-per-row kernel): size-independent properties plus an
+    # exact comparison of every row with the oracle
     from super_gnn_amd import synth
     ops = _ops()
-    n, F = 1_000_000, 256
     x = synth.boundary_features(n, F, seed=5, device="cuda")
     epb = 8 // bits
     seg = torch.tensor([0, n], dtype=torch.int32)
