@@ -850,6 +850,110 @@ __global__ __launch_bounds__(kQBlock) void quant_v1_vec_kernel(const float *__re
     }
 }
 
+// The quantizer once more with L = 16 or 8 lanes per row instead of a whole wavefront (F <= 4 * L * NV): the
+// min/max/zero-sign reductions stay inside a DPP row (four or three butterfly steps, no readlane round trips), a
+// wavefront carries 64/L rows side by side and R such rounds, and rows of different bit widths simply take
+// different store paths.  Same arithmetic and same bytes as quant_v1_vec_kernel.
+template <int NV, int R, int L>
+__global__ __launch_bounds__(kQBlock) void quant_v1_group_kernel(const float *__restrict__ x, uint8_t *__restrict__ q,
+                                                                 const int64_t *__restrict__ range,
+                                                                 float *__restrict__ params, int64_t n, int F) {
+    constexpr int RW = 64 / L;
+    const int lane = threadIdx.x & 63, d = lane / L, ll = lane % L;
+    const int64_t unit = (int64_t)blockIdx.x * (kQBlock / 64) + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int64_t i0 = unit * (RW * R);
+    if (i0 >= n) return;  // wave-uniform
+    float bits_f[R];
+    int64_t r0[R];
+    float xv[R][NV][4];
+    int off[NV];
+    bool act[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        off[v] = (v * L + ll) * 4;
+        act[v] = off[v] < F;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t i = i0 + r * RW + d < n ? i0 + r * RW + d : n - 1;  // rows past the end repeat the last row's loads
+        bits_f[r] = params[i * 3];
+        r0[r] = range[i];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) vec_load_nt<4>(xv[r][v], x + i * F + (act[v] ? off[v] : 0));  // unconditional
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t i = i0 + r * RW + d;
+        const int b = (int)bits_f[r];
+        float mn = INFINITY, mx = -INFINITY;
+        int key = INT_MAX;
+#pragma unroll
+        for (int v = NV - 1; v >= 0; --v) {
+            if (!act[v]) continue;
+#pragma unroll
+            for (int k = 3; k >= 0; --k) {
+                mn = fminf(mn, xv[r][v][k]);
+                mx = fmaxf(mx, xv[r][v][k]);
+                if (xv[r][v][k] == 0.0f) key = ((off[v] + k) << 1) | (int)(__float_as_uint(xv[r][v][k]) >> 31);
+            }
+        }
+        mn = group_allreduce_f<L, OpMinF>(mn);
+        mx = group_allreduce_f<L, OpMaxF>(mx);
+        key = group_allmin_i<L>(key);
+        const float first = __shfl(xv[r][0][0], lane & ~(L - 1));  // element 0 of the row
+        // everything from here on is private to a row's lanes
+        if (i >= n || (b != 8 && b != 4 && b != 2)) continue;  // the reference prints an error and leaves the row (quantization_x86.cpp:244-245)
+        const float z = (key & 1) ? -0.0f : 0.0f;
+        if (mn == 0.0f) mn = z;
+        if (mx == 0.0f) mx = z;
+        if (first != first) { mn = first; mx = first; }
+        float s = (mx - mn) / (float)((1 << b) - 1);
+        if (s == 0.0f) s = 1.0f;
+        if (ll == 0) { params[i * 3 + 1] = mn; params[i * 3 + 2] = s; }
+        const float rinv = __builtin_amdgcn_rcpf(s);
+        uint8_t *qo = q + r0[r];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            if (!act[v]) continue;
+            // product with the hardware reciprocal first, IEEE division only for a lane that sees an
+            // element within 2^-13 of a rounding tie (same argument as in quant_pack_rows16_kernel)
+            uint32_t c[4];
+            bool redo = !(s >= 0x1p-100f && s <= 0x1p100f);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const float qf = (xv[r][v][k] - mn) * rinv;
+                const float ri = rintf(qf);
+                if (!(fabsf(qf - ri) < 0.5f - 0x1p-13f)) redo = true;
+                c[k] = (uint32_t)ri;
+            }
+            if (redo) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) c[k] = quant_code(xv[r][v][k], mn, s);
+            }
+            if (b == 8) {
+                uint8_t *dst = qo + off[v];
+                if ((r0[r] & 3) == 0) {
+                    __builtin_nontemporal_store(c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24), reinterpret_cast<uint32_t *>(dst));
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) dst[k] = (uint8_t)c[k];
+                }
+            } else if (b == 4) {
+                uint8_t *dst = qo + off[v] / 2;
+                const uint32_t b0 = (c[0] << 4) | c[1], b1 = (c[2] << 4) | c[3];
+                if ((r0[r] & 1) == 0) {
+                    __builtin_nontemporal_store((uint16_t)(b0 | (b1 << 8)), reinterpret_cast<uint16_t *>(dst));
+                } else {
+                    dst[0] = (uint8_t)b0;
+                    dst[1] = (uint8_t)b1;
+                }
+            } else {
+                qo[off[v] / 4] = (uint8_t)((c[0] << 6) | (c[1] << 4) | (c[2] << 2) | c[3]);
+            }
+        }
+    }
+}
+
 template <int NV, int R>
 __global__ __launch_bounds__(kQBlock) void dequant_v1_vec_kernel(const uint8_t *__restrict__ q, float *__restrict__ x,
                                                                  const int64_t *__restrict__ range,
@@ -1204,7 +1308,20 @@ extern "C" int sgnn_quant_v1_f32(const float *x, uint8_t *q, const int64_t *rang
     const dim3 grid((uint32_t)nb), block(kQBlock);
     const auto grid_r = [&](int rows) { return dim3((uint32_t)((nb + rows - 1) / rows)); };
     hipStream_t st = (hipStream_t)stream;
-    if (F % 4 == 0 && F <= 1024 && aligned(x, 16)) {
+    static const bool group_layout = [] { const char *e = getenv("SGNN_QUANT_V1_GROUPS"); return !(e && e[0] == '0'); }();
+    if (group_layout && F % 4 == 0 && F <= 512 && aligned(x, 16)) {   // (wider rows: a wavefront per row is faster)
+        const auto grid_g = [&](int rows_per_wave) {
+            const int64_t waves = (n + rows_per_wave - 1) / rows_per_wave;
+            return dim3((uint32_t)((waves + kQBlock / 64 - 1) / (kQBlock / 64)));
+        };
+#define SGNN_V1G(NV, R, L) hipLaunchKernelGGL((quant_v1_group_kernel<NV, R, L>), grid_g((64 / L) * R), block, 0, st, x, q, range, params, n, (int)F)
+        if (F <= 32) SGNN_V1G(1, 4, 8);
+        else if (F <= 64) SGNN_V1G(2, 2, 8);
+        else if (F <= 128) SGNN_V1G(4, 1, 8);
+        else if (F <= 256) SGNN_V1G(4, 1, 16);
+        else SGNN_V1G(8, 1, 16);
+#undef SGNN_V1G
+    } else if (F % 4 == 0 && F <= 1024 && aligned(x, 16)) {
         if (F <= 256) hipLaunchKernelGGL((quant_v1_vec_kernel<1, 4>), grid_r(4), block, 0, st, x, q, range, params, n, (int)F);
         else if (F <= 512) hipLaunchKernelGGL((quant_v1_vec_kernel<2, 2>), grid_r(2), block, 0, st, x, q, range, params, n, (int)F);
         else hipLaunchKernelGGL((quant_v1_vec_kernel<4, 1>), grid, block, 0, st, x, q, range, params, n, (int)F);
