@@ -215,3 +215,18 @@ def test_full_size_community_graph_takes_the_band_schedule_and_matches_oracle():
     want = np.zeros((n, F), np.float32)
     orc.spmm_accumulate(rp, cl, np.ones(cl.shape[0], np.float32), x.cpu().numpy(), want)
     assert np.array_equal(out.cpu().numpy(), want), "band schedule: the reference's fma chain, bit for bit"
+
+
+def test_schedule_is_chosen_from_the_matrix_shape():
+    # the plan-time rule: a dense-degree matrix whose operand overflows the caches takes the band schedule, a
+    # power-law graph of the same size (few edges per row and band) and a small matrix keep the row-class kernels
+    from super_gnn_amd import synth
+    ops = _ops()
+    dev = torch.device("cuda:0")
+    rp, cl = synth.sbm_graph(60000, 10, 0.02, 0.001, seed=3, device=dev)              # ~170 edges per row
+    dense = ops.SpmmPlan(rp, cl, 60000)
+    assert dense.schedule(602)["band"] == 1 and dense.schedule(602)["n_slices"] == 8
+    assert dense.schedule(64)["band"] == 0                                             # 15 MB of X: cache-resident
+    rp, cl = synth.rmat_graph(200000, 2500000, seed=1, device=dev)                     # 25 edges per row
+    power = ops.SpmmPlan(rp, cl, 200000)
+    assert power.schedule(602)["band"] == 0 and power.schedule(128)["band"] == 0
