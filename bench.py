@@ -531,10 +531,10 @@ def wl_sbm(args, ctx):
     """Dense-degree community graph, wide odd feature rows (the band schedule)."""
     import torch
     from super_gnn_amd import synth, supergnn_ops as ops
-    dev, F = ctx["dev"], 602
-    n = args.sbm_nodes // 50 * 50
+    dev, F = ctx["dev"], args.sbm_feat
+    n = args.sbm_nodes // args.sbm_blocks * args.sbm_blocks
     t0 = time.perf_counter()
-    rowptr, col = synth.sbm_graph(n, 50, 0.03048, 0.001524, seed=3, device=dev)
+    rowptr, col = synth.sbm_graph(n, args.sbm_blocks, args.sbm_pin, args.sbm_pin / 20, seed=3, device=dev)
     g = torch.Generator(device=dev); g.manual_seed(4)
     x = torch.rand(n, F, generator=g, device=dev) * 2 - 1
     torch.cuda.synchronize()
@@ -558,7 +558,7 @@ def wl_sbm(args, ctx):
              "compulsory_bytes": int(spmm_compulsory_bytes(nnz, n, n, F, False)), "step_roofline": step_roofline(wl, per_kernel)}
     log(f"[bench] sbm sum: {ms:.3f} ms/step, {nnz / ms / 1e6:.2f} GEdges/s, schedule {sched}, kernels (ms per step) "
         f"{ {k: round(v, 4) for k, v in per_kernel.items()} }")
-    return {"metric": "SpMM GEdges/s (dense-degree community graph, F=602 fp32)", "value": round(nnz / ms / 1e6, 4),
+    return {"metric": f"SpMM GEdges/s (dense-degree community graph, F={F} fp32)", "value": round(nnz / ms / 1e6, 4),
             "unit": "GEdges/s", "config": {"workload": wl, "F": F}, "ms_per_step": ms, "dtype": "f32",
             "roofline": roofline(wl, dom, per_kernel[dom], dom_bytes, launches[dom]), "cpu_baseline": None, "extra": extra}
 
@@ -664,6 +664,9 @@ def main():
     ap.add_argument("--local-und-edges", type=int, default=160_000_000)
     ap.add_argument("--remote-edges", type=int, default=80_000_000)
     ap.add_argument("--sbm-nodes", type=int, default=233_000)
+    ap.add_argument("--sbm-blocks", type=int, default=50)
+    ap.add_argument("--sbm-pin", type=float, default=0.03048, help="sbm: edge probability inside a block (20x the one between blocks)")
+    ap.add_argument("--sbm-feat", type=int, default=602)
     ap.add_argument("--hidden", type=int, default=256, help="sage: hidden width")
     ap.add_argument("--classes", type=int, default=47, help="sage: output classes")
     ap.add_argument("--parts", type=int, default=8, help="aggregate: number of vertex partitions simulated in this process")
