@@ -230,3 +230,38 @@ def test_schedule_is_chosen_from_the_matrix_shape():
     rp, cl = synth.rmat_graph(200000, 2500000, seed=1, device=dev)                     # 25 edges per row
     power = ops.SpmmPlan(rp, cl, 200000)
     assert power.schedule(602)["band"] == 0 and power.schedule(128)["band"] == 0
+
+
+def test_band_schedule_replays_from_a_captured_graph(monkeypatch):
+    # steady-state products of the band schedule (restage + one launch per band, more than 48 KB of LDS per
+    # workgroup) only launch kernels: capture once, replay with eager work in between, compare bits
+    ops = _ops()
+    _force(monkeypatch, 256)
+    dev = torch.device("cuda:0")
+    M, K, F = 900, 1500, 602
+    rowptr, col, val = random_csr(M, K, 40, seed=21, empty_frac=0.1, hubs=2, hub_deg=900)
+    x = torch.randn(K, F, generator=torch.Generator().manual_seed(3)).to(dev)
+    w = torch.from_numpy(val).to(dev)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    out, out1 = torch.zeros(M, F, device=dev), torch.zeros(M, F, device=dev)
+
+    def step():
+        out.zero_(); out1.zero_()
+        plan.run(w, x, out, accumulate=True)
+        plan.run(None, x, out1, accumulate=True)
+
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    want, want1 = out.clone(), out1.clone()
+    ref = np.zeros((M, F), np.float32); orc.spmm_accumulate(rowptr, col, val, x.cpu().numpy(), ref)
+    assert np.array_equal(want.cpu().numpy(), ref)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for i in range(3):
+        out.fill_(float(i)); out1.fill_(-2.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want) and torch.equal(out1, want1), f"replay {i}"
