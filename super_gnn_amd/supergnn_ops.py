@@ -179,6 +179,21 @@ class SpmmPlan:
             self._bound = (value, value._version)
         self._seen = (value, value._version)
 
+    def bind_values(self, value):
+        """Bind (or re-bind) an edge-value tensor by hand.  run() does this by itself for a tensor that comes
+        back unchanged, and notices edits that move the tensor's version counter; call this after changing the
+        values in a way the counter does not see (a write through ``.data``, a kernel given the raw pointer)."""
+        _want(value, torch.float32, "value")
+        if not (value.is_cuda and value.is_contiguous() and value.numel() == self.nnz):
+            raise ValueError("value must be a contiguous GPU tensor with one entry per edge")
+        check(lib.sgnn_spmm_plan_bind_values(self._h, _ptr(value), _stream()))
+        self._bound = self._seen = (value, value._version)
+
+    def unbind_values(self):
+        """Forget the bound edge values: every later product reads the tensor it is given."""
+        check(lib.sgnn_spmm_plan_bind_values(self._h, None, _stream()))
+        self._bound = self._seen = None
+
     def run_quantized(self, value, data_int8, params, segs, bits, out, accumulate=True, row_div=None):
         """out (+)= A @ dequantize(data_int8): the dense operand stays packed (row-group layout,
         ``segs`` from quant_segments()) and is decoded inside the gather."""

@@ -365,6 +365,30 @@ def test_steady_state_calls_replay_from_a_captured_graph():
         assert torch.equal(out, want) and torch.equal(out_q, want_q), f"replay {i}"
 
 
+def test_explicit_rebinding_after_an_edit_the_version_counter_does_not_see():
+    ops = _gpu()
+    dev = torch.device("cuda:0")
+    rowptr, col, val = random_csr(600, 500, 8, seed=13, hubs=3, hub_deg=400)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), 500)
+    x = torch.randn(500, 32, generator=torch.Generator().manual_seed(2)).to(dev)
+    w = torch.from_numpy(val).to(dev)
+    out = torch.zeros(600, 32, device=dev)
+    for _ in range(3):                                   # bound from the second call on
+        out.zero_(); plan.run(w, x, out, accumulate=True)
+    first = out.clone()
+    w.data.mul_(3.0)                                     # the version counter stays where it was
+    plan.bind_values(w)
+    out.zero_(); plan.run(w, x, out, accumulate=True)
+    want = np.zeros((600, 32), np.float32)
+    orc.spmm_accumulate(rowptr, col, w.cpu().numpy(), x.cpu().numpy(), want)
+    _assert_close(out.cpu().numpy(), want, orc.spmm_f64(rowptr, col, w.cpu().numpy(), x.cpu().numpy(), None),
+                      _abs_sum64(rowptr, col, w.cpu().numpy(), x.cpu().numpy(), None), np.diff(rowptr), what="rebound")
+    assert not torch.equal(out, first)
+    plan.unbind_values()
+    out2 = torch.zeros(600, 32, device=dev); plan.run(w, x, out2, accumulate=True)
+    assert torch.equal(out2, out)                        # same floats with and without the bound copy
+
+
 def test_plan_finalised_during_a_capture_does_not_invalidate_it():
     """Python may run a dead plan's finaliser at any time, also inside someone's graph capture; freeing device
     memory there would invalidate the capture, so the wrapper parks the handle until later."""
