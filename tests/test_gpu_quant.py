@@ -409,7 +409,7 @@ def test_cpu_runnable_configuration_int8_boundary_rows():
     assert np.all(np.abs(back.cpu().numpy() - x.numpy()) <= p_ref[:, 1:2] * 0.5 * (1 + 1e-6) + 4 * tol)
 
 
-@pytest.mark.parametrize("F", [4, 12, 100, 128, 256, 600, 1024, 1028, 37])
+@pytest.mark.parametrize("F", [4, 12, 32, 36, 64, 100, 128, 132, 256, 260, 512, 600, 1024, 1028, 37])
 def test_v1_mixed_bits_all_widths(F):
     """Feature-packed mixed-bit rows (2/4/8 bits chosen per row, so row byte offsets fall on every
     alignment): bytes and params bit-exact vs the oracle, floats within one rounding; widths on both
