@@ -365,6 +365,31 @@ def test_steady_state_calls_replay_from_a_captured_graph():
         assert torch.equal(out, want) and torch.equal(out_q, want_q), f"replay {i}"
 
 
+def test_workgroup_per_hub_row_alternative(monkeypatch):
+    # the scheduling kept for comparison (one workgroup per long row, partial sums reduced in LDS): same bar
+    ops = _gpu()
+    dev = torch.device("cuda:0")
+    monkeypatch.setenv("SGNN_SPMM_HUB_LDS", "1")
+    for F in (128, 100, 602, 7):
+        rowptr, col, val = random_csr(1200, 900, 10, seed=F, empty_frac=0.2, hubs=6, hub_deg=2000, dup=True)
+        x = np.random.default_rng(F).standard_normal((900, F)).astype(np.float32)
+        init = np.random.default_rng(F + 1).standard_normal((1200, F)).astype(np.float32)
+        div = np.maximum(np.diff(rowptr), 1).astype(np.float32)
+        plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), 900)
+        for accumulate, mean in ((True, False), (False, True)):
+            out = torch.from_numpy(init.copy()).to(dev)
+            plan.run(torch.from_numpy(val).to(dev), torch.from_numpy(x).to(dev), out, accumulate=accumulate,
+                     row_div=torch.from_numpy(div).to(dev) if mean else None)
+            base = init if accumulate else None
+            want = init.copy() if accumulate else np.zeros_like(init)
+            orc.spmm_accumulate(rowptr, col, val, x, want)
+            f64, asum = orc.spmm_f64(rowptr, col, val, x, base), _abs_sum64(rowptr, col, val, x, base)
+            if mean:
+                orc.row_divide(want, div)
+                f64, asum = f64 / div[:, None].astype(np.float64), asum / div[:, None].astype(np.float64)
+            _assert_close(out.cpu().numpy(), want, f64, asum, np.diff(rowptr), what=f"hub rows in LDS, F={F}")
+
+
 def test_explicit_rebinding_after_an_edit_the_version_counter_does_not_see():
     ops = _gpu()
     dev = torch.device("cuda:0")
