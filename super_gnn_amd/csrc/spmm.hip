@@ -803,7 +803,7 @@ __global__ __launch_bounds__(kBlock) void spmm_piece_kernel(
                                              off_ld, act_ld, lig);
 #pragma unroll
         for (int v = 0; v < NV; ++v)
-            if (act[v]) vec_store<VEC>(partial + (int64_t)item * F + off[v], acc[v]);
+            if (act[v]) vec_store_nt<VEC>(partial + (int64_t)item * F + off[v], acc[v]);
     }
 }
 
@@ -898,7 +898,7 @@ __global__ __launch_bounds__(kBlock) void spmm_long_final_kernel(
 #pragma unroll
                 for (int u = 0; u < UP; ++u) {
                     const int si = s + u < s1 ? s + u : s1 - 1;
-                    vec_load<VEC>(p[u], partial + (int64_t)si * F + off);
+                    vec_load_nt<VEC>(p[u], partial + (int64_t)si * F + off);
                 }
 #pragma unroll
                 for (int u = 0; u < UP; ++u) {
