@@ -146,6 +146,19 @@ __device__ __forceinline__ void vec_load_nt(float (&r)[VEC], const float *p) {
     }
 }
 
+// A 16-byte non-temporal load from an address that is only 4-byte aligned (rows whose width is not a
+// multiple of four floats).  Global memory on gfx950 serves such a vector access in one instruction.
+__device__ __forceinline__ void vec4_load_nt_unaligned(float (&r)[4], const float *p) {
+    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+    const f4u v = __builtin_nontemporal_load(reinterpret_cast<const f4u *>(p));
+    r[0] = v.x; r[1] = v.y; r[2] = v.z; r[3] = v.w;
+}
+// A 4-byte non-temporal store to an address of any alignment.
+__device__ __forceinline__ void u32_store_nt_unaligned(uint8_t *p, uint32_t w) {
+    typedef uint32_t u32u __attribute__((aligned(1)));
+    __builtin_nontemporal_store(w, reinterpret_cast<u32u *>(p));
+}
+
 template <int VEC>
 __device__ __forceinline__ void vec_store_nt(float *p, const float (&r)[VEC]) {
     if constexpr (VEC == 4) {

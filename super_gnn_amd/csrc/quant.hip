@@ -308,7 +308,11 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
 // then spread over twice as many elements per lane, which is what limits rows of 64 and 128 floats.
 // ------------------------------------------------------------------------------------------------
 // FULL: F == 4 * L * NV, every lane's every vector lies inside the row (no per-load lane predicates).
-template <int BITS, int NV, int RL, bool kForceExactDivision, bool FULL = false, int L = 16>
+// RAGGED: any F and any 4-byte aligned row start (F = 602, F = 123, a window with an odd leading dimension):
+// the float4 loads and the 4-byte code stores are issued at their natural (unaligned) addresses, and the one
+// vector per row that reaches past the end of the row is loaded and stored element by element, its missing
+// elements filled with copies of its first one (copies change neither min nor max nor the first-zero rule).
+template <int BITS, int NV, int RL, bool kForceExactDivision, bool FULL = false, int L = 16, bool RAGGED = false>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
     const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F,
@@ -350,8 +354,20 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
         if (!valid[rl]) continue;
         const float *xr = row_ptr(xs, row[rl]);
 #pragma unroll
-        for (int v = 0; v < NV; ++v)
-            if (act[v]) vec_load_nt<VEC>(xv[rl][v], xr + off[v]);
+        for (int v = 0; v < NV; ++v) {
+            if (!act[v]) continue;
+            if constexpr (RAGGED) {
+                if (off[v] + VEC <= F) {
+                    vec4_load_nt_unaligned(xv[rl][v], xr + off[v]);
+                } else {
+                    xv[rl][v][0] = xr[off[v]];
+#pragma unroll
+                    for (int k = 1; k < VEC; ++k) xv[rl][v][k] = off[v] + k < F ? xr[off[v] + k] : xv[rl][v][0];
+                }
+            } else {
+                vec_load_nt<VEC>(xv[rl][v], xr + off[v]);
+            }
+        }
     }
 
     float zp[RL], sc[RL], rinv[RL];
@@ -464,8 +480,18 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
                 if constexpr (EPB == 4) w |= (uint32_t)__shfl_xor((int)w, 16, 64);
             }
             const bool mine = EPB == 1 ? true : EPB == 2 ? ((d & 1) == (v & 1)) : ((d & 3) == (v & 3));
-            if (mine && act[v] && gp[rl] < n_packed)
-                __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(q + (int64_t)gp[rl] * F + off[v]));
+            if (mine && act[v] && gp[rl] < n_packed) {
+                uint8_t *dst = q + (int64_t)gp[rl] * F + off[v];
+                if constexpr (RAGGED) {
+                    if (off[v] + VEC <= F) {
+                        u32_store_nt_unaligned(dst, w);
+                    } else {
+                        for (int k = 0; off[v] + k < F; ++k) dst[k] = (uint8_t)(w >> (8 * k));
+                    }
+                } else {
+                    __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(dst));
+                }
+            }
         }
     }
 }
@@ -609,6 +635,99 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
+// The same flat decomposition for widths that are not a multiple of four (F = 602, F = 123 ...): the
+// output is still written as 16-byte vectors over the flat array, but a vector may now straddle a row
+// boundary, so it is made of 4 / VEC pieces of VEC floats (VEC = 2 for even F, 1 for odd F), each with
+// its own (row, column), its own VEC code bytes and its own params.  The last vector of the array may be
+// partial and is written element by element.  x must be 16-byte aligned (the row-tiled kernels take
+// other cases).
+// ------------------------------------------------------------------------------------------------
+template <int BITS, int VEC, int R, bool SEGMENTED>
+__global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_ragged_kernel(
+    const uint8_t *__restrict__ q, float *__restrict__ x, const ParamBuf pb, const int32_t *__restrict__ seg,
+    const int32_t *__restrict__ pseg, int P, int F, int64_t n_elem) {
+    constexpr int EPB = 8 / BITS;
+    constexpr int NP = 4 / VEC;
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
+    const int64_t base = wave * (R * 64) + lane;
+    const int64_t n_vec = (n_elem + 3) >> 2;
+    uint32_t word[R][NP];
+    float2 ps[R][NP];
+    int shift[R][NP];
+    int w_p = 0, w_s0 = 0, w_s1 = 0, w_ps0 = 0;
+    if constexpr (SEGMENTED) {  // the segment of the wave's first row, found on wave-uniform values
+        const int64_t i0 = ((int64_t)blockIdx.x * (kQBlock / 64) + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))) * (R * 64);
+        const int row_w = (int)((i0 * 4) / F);
+        int lo = 0, hi = P - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (seg[mid + 1] > row_w) hi = mid; else lo = mid + 1;
+        }
+        w_p = lo;
+        w_s0 = seg[lo];
+        w_s1 = seg[lo + 1];
+        w_ps0 = pseg[lo];
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const int64_t i = base + u * 64;
+        int row = 0, c = 0;
+        if (i < n_vec) {
+            const int64_t e0 = i * 4;
+            row = (int)(e0 / F);
+            c = (int)(e0 - (int64_t)row * F);
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            word[u][p] = 0;
+            ps[u][p] = make_float2(0.0f, 0.0f);
+            shift[u][p] = 0;
+            if (i < n_vec && i * 4 + p * VEC < n_elem) {
+                int slot = row;
+                if constexpr (SEGMENTED) {
+                    if (row < w_s1) {
+                        slot = w_ps0 * EPB + (row - w_s0);
+                    } else {
+                        int lo = w_p, hi = P - 1;
+                        while (lo < hi) {
+                            const int mid = (lo + hi) >> 1;
+                            if (seg[mid + 1] > row) hi = mid; else lo = mid + 1;
+                        }
+                        slot = pseg[lo] * EPB + (row - seg[lo]);
+                    }
+                }
+                ps[u][p] = load_params(pb, row);
+                shift[u][p] = (EPB - 1 - (slot % EPB)) * BITS;
+                const uint8_t *src = q + (int64_t)(slot / EPB) * F + c;  // cacheable: rows that share a byte hit in cache
+                if constexpr (VEC == 2) word[u][p] = *reinterpret_cast<const uint16_t *>(src);
+                else word[u][p] = *src;
+            }
+            c += VEC;
+            if (c >= F) { c = 0; ++row; }  // F % VEC == 0: a piece never straddles a row boundary
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const int64_t i = base + u * 64;
+        if (i >= n_vec) continue;
+        float o[4];
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                o[p * VEC + e] = fmaf((float)((word[u][p] >> (8 * e + shift[u][p])) & MASK), ps[u][p].y, ps[u][p].x);
+        if (i * 4 + 4 <= n_elem) {
+            vec_store_nt<4>(x + i * 4, o);
+        } else {
+            for (int e = 0; e < 4; ++e)
+                if (i * 4 + e < n_elem) x[i * 4 + e] = o[e];
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Any-F fallbacks (F wider than a register tile): one wavefront per packed row, two passes.
 // ------------------------------------------------------------------------------------------------
 template <int BITS>
@@ -621,20 +740,42 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_wide_kernel(
     if (gp >= n_packed) return;
     int64_t row0, rend;
     locate_packed_row(seg, pseg, P, single_rows, gp, __builtin_amdgcn_readfirstlane(gp), EPB, row0, rend);
-    float zp[EPB], sc[EPB];
+    // Both passes walk a row in 16-byte vectors at their natural (4-byte aligned) addresses; the one
+    // vector that reaches past the end of the row is read element by element.  The second pass finds
+    // the rows in cache.
+    const int nvr = (F + 3) >> 2;
+    constexpr float kGuard = BITS == 8 ? 0x1p-13f : BITS == 4 ? 0x1p-17f : 0x1p-19f;
+    float zp[EPB], sc[EPB], rinv[EPB];
+    const float *xr[EPB];
 #pragma unroll
     for (int k = 0; k < EPB; ++k) {
         zp[k] = 0.0f;
         sc[k] = 1.0f;
+        rinv[k] = 1.0f;
+        xr[k] = nullptr;
         if (row0 + k >= rend) continue;
-        const float *xr = row_ptr(xs, row0 + k);
+        xr[k] = row_ptr(xs, row0 + k);
         float mn = INFINITY, mx = -INFINITY;
         int key = INT_MAX;
-        for (int j = lane; j < F; j += 64) {
-            const float v = xr[j];
-            mn = fminf(mn, v);
-            mx = fmaxf(mx, v);
-            if (v == 0.0f && key == INT_MAX) key = (j << 1) | (int)(__float_as_uint(v) >> 31);
+        for (int j = lane; j < nvr; j += 64) {
+            const int c = 4 * j;
+            float v[4];
+            if (c + 4 <= F) {
+                vec4_load_nt_unaligned(v, xr[k] + c);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) v[t] = c + t < F ? xr[k][c + t] : xr[k][c];
+            }
+#pragma unroll
+            for (int t = 3; t >= 0; --t) {
+                mn = fminf(mn, v[t]);
+                mx = fmaxf(mx, v[t]);
+            }
+            if (key == INT_MAX) {
+#pragma unroll
+                for (int t = 3; t >= 0; --t)
+                    if (v[t] == 0.0f) key = ((c + t) << 1) | (int)(__float_as_uint(v[t]) >> 31);
+            }
         }
         mn = group_allreduce_f<64, OpMinF>(mn);
         mx = group_allreduce_f<64, OpMaxF>(mx);
@@ -642,21 +783,53 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_wide_kernel(
         const float z = (key & 1) ? -0.0f : 0.0f;
         if (mn == 0.0f) mn = z;
         if (mx == 0.0f) mx = z;
-        const float first = xr[0];
+        const float first = xr[k][0];
         if (first != first) { mn = first; mx = first; }
         float s = (mx - mn) / (float)((1 << BITS) - 1);
         if (s == 0.0f) s = 1.0f;
         zp[k] = mn;
         sc[k] = s;
+        rinv[k] = __builtin_amdgcn_rcpf(s);
         if (lane == 0) store_params(pb, row0 + k, mn, s);
     }
     uint8_t *qr = q + (int64_t)gp * F;
-    for (int j = lane; j < F; j += 64) {
-        uint32_t byte = 0;
+    for (int j = lane; j < nvr; j += 64) {
+        const int c = 4 * j;
+        const int nval = F - c < 4 ? F - c : 4;
+        uint32_t word = 0;
 #pragma unroll
-        for (int k = 0; k < EPB; ++k)
-            if (row0 + k < rend) byte |= quant_code(row_ptr(xs, row0 + k)[j], zp[k], sc[k]) << ((EPB - 1 - k) * BITS);
-        qr[j] = (uint8_t)byte;
+        for (int k = 0; k < EPB; ++k) {
+            if (row0 + k >= rend) continue;
+            float v[4];
+            if (nval == 4) {
+                vec4_load_nt_unaligned(v, xr[k] + c);
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) v[t] = t < nval ? xr[k][c + t] : xr[k][c];
+            }
+            // product with the hardware reciprocal first, IEEE division only when an element lies inside the
+            // guard band around a rounding tie (same argument and bands as in quant_pack_rows16_kernel)
+            uint32_t w = 0;
+            bool redo = !(sc[k] >= 0x1p-100f && sc[k] <= 0x1p100f);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const float qf = (v[t] - zp[k]) * rinv[k];
+                const float ri = rintf(qf);
+                if (!(fabsf(qf - ri) < 0.5f - kGuard)) redo = true;
+                w = __builtin_amdgcn_cvt_pk_u8_f32(ri, t, w);
+            }
+            if (redo) {
+                w = 0;
+#pragma unroll
+                for (int t = 0; t < 4; ++t) w |= quant_code(v[t], zp[k], sc[k]) << (8 * t);
+            }
+            word |= w << ((EPB - 1 - k) * BITS);
+        }
+        if (nval == 4) {
+            u32_store_nt_unaligned(qr + c, word);
+        } else {
+            for (int t = 0; t < nval; ++t) qr[c + t] = (uint8_t)(word >> (8 * t));
+        }
     }
 }
 
@@ -1072,6 +1245,32 @@ static void launch_rows(const RowsArgs &a, hipStream_t st) {
                            a.x_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
+template <int BITS, int NV, int L>
+static void launch_quant16_ragged(const RowsArgs &a, hipStream_t st) {
+    constexpr int RL = NV >= 4 ? 1 : 4 / NV;
+    constexpr int EPB = 8 / BITS;
+    constexpr int RW = 64 / L;
+    const int64_t padded = (int64_t)a.n_packed * EPB;
+    const int n_units = (int)((padded + RW * RL - 1) / (RW * RL));
+    const int nb = (n_units + kQBlock / 64 - 1) / (kQBlock / 64);
+    ProfScope prof(K_QUANT_PACK_ROWS, st);
+    hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
+                       a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
+}
+
+// Widths or row starts that are not a multiple of four floats, up to 1024 floats per row.
+template <int BITS>
+static void dispatch_quant16_ragged(const RowsArgs &a, hipStream_t st) {
+    const int nvec = (a.F + 3) / 4;
+    if (nvec <= 8) return launch_quant16_ragged<BITS, 1, 8>(a, st);
+    if (nvec <= 16) return launch_quant16_ragged<BITS, 2, 8>(a, st);
+    if (nvec <= 32) return launch_quant16_ragged<BITS, 2, 16>(a, st);
+    if (nvec <= 64) return launch_quant16_ragged<BITS, 4, 16>(a, st);
+    if (nvec <= 128) return launch_quant16_ragged<BITS, 8, 16>(a, st);
+    if (nvec <= 160) return launch_quant16_ragged<BITS, 10, 16>(a, st);
+    return launch_quant16_ragged<BITS, 16, 16>(a, st);
+}
+
 template <int BITS, int NV, int L = 16>
 static void launch_quant16(const RowsArgs &a, hipStream_t st) {
     constexpr int RL = NV >= 4 ? 1 : 4 / NV;
@@ -1124,6 +1323,22 @@ static void launch_dequant_flat(const RowsArgs &a, int64_t n_rows, hipStream_t s
     else launch_dequant_flat_r<BITS, 2>(a, n_rows, st);
 }
 
+template <int BITS, int VEC>
+static void launch_dequant_flat_ragged(const RowsArgs &a, int64_t n_rows, hipStream_t st) {
+    constexpr int R = 2;
+    const int64_t n_elem = n_rows * (int64_t)a.F;
+    const int64_t n_vec = (n_elem + 3) / 4;
+    const int64_t n_waves = (n_vec + R * 64 - 1) / (R * 64);
+    const unsigned nb = (unsigned)((n_waves + kQBlock / 64 - 1) / (kQBlock / 64));
+    ProfScope prof(K_UNPACK_DEQUANT_ROWS, st);
+    if (BITS != 8 && a.P > 1)
+        hipLaunchKernelGGL((unpack_dequant_flat_ragged_kernel<BITS, VEC, R, true>), dim3(nb), dim3(kQBlock), 0, st, a.q_in,
+                           a.x_out, a.params, a.seg, a.pseg, a.P, a.F, n_elem);
+    else
+        hipLaunchKernelGGL((unpack_dequant_flat_ragged_kernel<BITS, VEC, R, false>), dim3(nb), dim3(kQBlock), 0, st, a.q_in,
+                           a.x_out, a.params, a.seg, a.pseg, a.P, a.F, n_elem);
+}
+
 template <int BITS>
 static void launch_rows_wide(const RowsArgs &a, hipStream_t st) {
     const int nb = (a.n_packed + kQBlock / 64 - 1) / (kQBlock / 64);
@@ -1151,6 +1366,7 @@ static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
             if (nvec <= 32) return launch_quant16<BITS, 2>(a, st);
             if (nvec <= 64) return launch_quant16<BITS, 4>(a, st);
             if (nvec <= 128) return launch_quant16<BITS, 8>(a, st);
+            if (nvec <= 160) return launch_quant16<BITS, 10>(a, st);
             if (nvec <= 256) return launch_quant16<BITS, 16>(a, st);
         }
     }
@@ -1199,6 +1415,16 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
         if (bits == 8) launch_dequant_flat<8>(a, n_rows, st);
         else if (bits == 4) launch_dequant_flat<4>(a, n_rows, st);
         else launch_dequant_flat<2>(a, n_rows, st);
+    } else if (!a.quantize && a.flat && a.F % 4 != 0 && aligned(fp32_ptr, 16) && (a.F % 2 != 0 || aligned(u8_ptr, 2))) {
+        // widths that are not a multiple of four: flat 16-byte stores made of float2 / float pieces
+        const bool even = a.F % 2 == 0;
+        if (bits == 8) even ? launch_dequant_flat_ragged<8, 2>(a, n_rows, st) : launch_dequant_flat_ragged<8, 1>(a, n_rows, st);
+        else if (bits == 4) even ? launch_dequant_flat_ragged<4, 2>(a, n_rows, st) : launch_dequant_flat_ragged<4, 1>(a, n_rows, st);
+        else even ? launch_dequant_flat_ragged<2, 2>(a, n_rows, st) : launch_dequant_flat_ragged<2, 1>(a, n_rows, st);
+    } else if (a.quantize && vec != 4 && a.layout16 && !a.exact_division && a.F <= 1024) {
+        if (bits == 8) dispatch_quant16_ragged<8>(a, st);
+        else if (bits == 4) dispatch_quant16_ragged<4>(a, st);
+        else dispatch_quant16_ragged<2>(a, st);
     } else if (bits == 8) dispatch_rows<8>(vec, a, st);
     else if (bits == 4) dispatch_rows<4>(vec, a, st);
     else dispatch_rows<2>(vec, a, st);

@@ -68,7 +68,7 @@ def test_rows_bit_exact_vs_oracle(bits, n, F):
 
 
 @pytest.mark.parametrize("bits", [8, 4, 2])
-@pytest.mark.parametrize("F", [128, 123])
+@pytest.mark.parametrize("F", [128, 123, 602])
 def test_many_segments_bit_exact(bits, F):
     # the reference script's layout check: 256 random segments (tests/test_quantization_ops.py:130-148)
     rng = np.random.default_rng(bits + F)
@@ -267,7 +267,7 @@ def test_full_size_properties(bits, n, F):
     assert np.all(np.abs(d.cpu().numpy() - d_ref) <= dequant_atol(p_ref[:, 0], p_ref[:, 1], bits)[:, None])
 
 
-@pytest.mark.parametrize("F", [256, 128, 64])
+@pytest.mark.parametrize("F", [256, 128, 64, 602, 123, 100])
 @pytest.mark.parametrize("bits", [8, 4, 2])
 def test_fast_quotient_equals_ieee_division(bits, F):
     """The kernel forms (x-zp)*RN(1/scale) and falls back to the IEEE division near half-integers;
@@ -278,7 +278,9 @@ def test_fast_quotient_equals_ieee_division(bits, F):
     ops = _ops()
     qmax = (1 << bits) - 1
     g = torch.Generator(device="cuda"); g.manual_seed(bits)
-    n = 256_000_000 // F
+    # (F = 602 / 123: the rows start on 8- / 4-byte boundaries and the default kernel reads them with unaligned
+    # 16-byte loads, while the all-IEEE variant is the lane-group kernel with float2 / scalar lanes)
+    n = (256_000_000 if F % 4 == 0 else 64_000_000) // F
     x = synth.boundary_features(n, F, seed=5, device="cuda")
     # adversarial block: min 0, max qmax*s, values at (k + 0.5 +- tiny) * s for assorted scales s
     na = 4096
@@ -317,7 +319,7 @@ def test_fast_quotient_equals_ieee_division(bits, F):
 # wire-side variants: gathered input rows, bf16 (zero_point, scale)
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("bits", [8, 4, 2])
-@pytest.mark.parametrize("F", [128, 256, 100, 37, 1200])
+@pytest.mark.parametrize("F", [128, 256, 100, 37, 1200, 602])
 def test_gathering_quantizer_equals_index_select_then_quantize(bits, F):
     from super_gnn_amd import supergnn_ops as ops
     gen = torch.Generator().manual_seed(bits * 1000 + F)
@@ -334,6 +336,12 @@ def test_gathering_quantizer_equals_index_select_then_quantize(bits, F):
     wide = torch.randn(5000, F + 8, generator=gen).cuda()
     view = wide[:, 4:4 + F]
     q_c = torch.zeros_like(q_a); p_c = torch.zeros_like(p_a)
+    ops.quantize_tensor_for_all_procs(view, q_c, p_c, wr, 4, bits, row_index=idx)
+    ops.quantize_tensor_for_all_procs(view[idx].contiguous(), q_a, p_a, wr, 4, bits)
+    assert torch.equal(q_a, q_c) and torch.equal(p_a, p_c)
+    # a window whose rows start on odd 4-byte boundaries (odd leading dimension, odd column offset)
+    wide = torch.randn(5000, F + 7, generator=gen).cuda()
+    view = wide[:, 3:3 + F]
     ops.quantize_tensor_for_all_procs(view, q_c, p_c, wr, 4, bits, row_index=idx)
     ops.quantize_tensor_for_all_procs(view[idx].contiguous(), q_a, p_a, wr, 4, bits)
     assert torch.equal(q_a, q_c) and torch.equal(p_a, p_c)
@@ -368,7 +376,7 @@ def test_bf16_params_equal_torch_casts(bits, F):
 
 
 @pytest.mark.parametrize("bits", [8, 4, 2])
-@pytest.mark.parametrize("F", [4, 64, 100, 128, 256, 600, 1028, 2052])
+@pytest.mark.parametrize("F", [4, 64, 100, 128, 256, 600, 1028, 2052, 602, 123, 6, 3, 1, 2050])
 def test_flat_and_row_tiled_dequantizers_agree(bits, F, monkeypatch):
     """The flat-output kernel (default) and the row-tiled kernels are two decompositions of the same
     arithmetic: same bits out, ragged multi-segment tables included."""
