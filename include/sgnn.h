@@ -208,7 +208,8 @@ int sgnn_quant_row_slots(const int32_t *seg, const int32_t *pseg, int P, int bit
  * Replaces the pair "dequantize into recv_buf, then SPMM_forward(remote graph, recv_buf, out)" of
  * super_gnn/aggregator.py:72-93 (forward) and :159-171 (backward); no fp32 recv_buf is written or
  * re-read.  The result is bit-identical to running sgnn_unpack_dequant_rows_f32 followed by
- * sgnn_spmm_csr_f32 with the same plan.  F % 4 == 0 required; other arguments as in
+ * sgnn_spmm_csr_f32 with the same plan.  F must be even (F % 4 == 0 takes four-code lanes, other even widths such
+ * as 602 two-code lanes; an odd F is refused: dequantize, then multiply); other arguments as in
  * sgnn_spmm_csr_f32.  row_slot: see sgnn_quant_row_slots (NULL = identity). */
 int sgnn_spmm_csr_dq_f32(sgnn_spmm_plan *plan, const float *val, const uint8_t *q, const float *params,
                          const int32_t *row_slot, int bits, float *out, int64_t F, int64_t ldo,

@@ -156,7 +156,7 @@ def _world_forward(world, feats, bits, out_all=None):
     F = feats[0].shape[-1]
     arena = world.arena(F, feats[0].device, bits)
     qz = Quantizer_for_all_procs(len(graphs), bits) if quantized else None
-    fused = quantized and F % 4 == 0
+    fused = quantized and F % 2 == 0
     feats = [x.contiguous() for x in feats]
     main = torch.cuda.current_stream()
     side = world.side_stream(feats[0].device)
@@ -209,7 +209,7 @@ def _world_backward(world, grads, bits, out_all=None):
     F = grads[0].shape[-1]
     arena = world.arena(F, grads[0].device, bits)
     qz = Quantizer_for_all_procs(len(graphs), bits) if quantized else None
-    fused = quantized and F % 4 == 0
+    fused = quantized and F % 2 == 0
     grads = [go.contiguous() for go in grads]
     main = torch.cuda.current_stream()
     side = world.side_stream(grads[0].device)

@@ -484,7 +484,16 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
                 uint8_t *dst = q + (int64_t)gp[rl] * F + off[v];
                 if constexpr (RAGGED) {
                     if (off[v] + VEC <= F) {
-                        u32_store_nt_unaligned(dst, w);
+                        // a 4-byte store that is not 4-byte aligned is slower than two aligned 2-byte stores
+                        const uintptr_t al = reinterpret_cast<uintptr_t>(dst) & 3;
+                        if (al == 0) {
+                            __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(dst));
+                        } else if (al == 2) {
+                            __builtin_nontemporal_store((uint16_t)w, reinterpret_cast<uint16_t *>(dst));
+                            __builtin_nontemporal_store((uint16_t)(w >> 16), reinterpret_cast<uint16_t *>(dst) + 1);
+                        } else {
+                            for (int k = 0; k < 4; ++k) dst[k] = (uint8_t)(w >> (8 * k));
+                        }
                     } else {
                         for (int k = 0; off[v] + k < F; ++k) dst[k] = (uint8_t)(w >> (8 * k));
                     }

@@ -1171,9 +1171,20 @@ static int dispatch_shape(int nvec, const ShortArgs &a, const PieceArgs &s, cons
     return SGNN_OK;
 }
 
-// Quantized dense operand: float4-wide lanes only (F % 4 == 0), one packed word per lane and vector.
+// Quantized dense operand: one packed word of VEC codes per lane and vector.  VEC = 4 when F % 4 == 0,
+// VEC = 2 for the other even widths (F = 602: 301 two-float lanes slots, five per lane).
 template <int BITS>
-static int dispatch_shape_dq(int nvec, const ShortArgs &a, const PieceArgs &s, const FinalArgs &f, hipStream_t st) {
+static int dispatch_shape_dq(int vec, int nvec, const ShortArgs &a, const PieceArgs &s, const FinalArgs &f, hipStream_t st) {
+    if (vec == 2) {
+        if (nvec <= 8) launch_all<2, 8, 1, BITS>(a, s, f, st);
+        else if (nvec <= 16) launch_all<2, 16, 1, BITS>(a, s, f, st);
+        else if (nvec <= 32) launch_all<2, 32, 1, BITS>(a, s, f, st);
+        else if (nvec <= 64) launch_all<2, 64, 1, BITS>(a, s, f, st);
+        else if (nvec <= 128) launch_all<2, 64, 2, BITS>(a, s, f, st);
+        else if (nvec <= 320) launch_all<2, 64, 5, BITS>(a, s, f, st);
+        else launch_all<2, 64, 8, BITS>(a, s, f, st);
+        return SGNN_OK;
+    }
     if (nvec <= 8) launch_all<4, 8, 1, BITS>(a, s, f, st);
     else if (nvec <= 16) launch_all<4, 16, 1, BITS>(a, s, f, st);
     else if (nvec <= 32) launch_all<4, 32, 1, BITS>(a, s, f, st);
@@ -1909,8 +1920,9 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     }
     int vec = 1;
     if (bits != 0) {
-        vec = 4;  // checked by the caller: F % 4 == 0 and 4-byte aligned packed rows
-        SGNN_REQUIRE(ldo % 4 == 0 && aligned(out, 16), "out must be 16-byte aligned with ldo %% 4 == 0 for the fused path");
+        vec = F % 4 == 0 ? 4 : 2;  // checked by the caller: F even, 4-byte aligned packed buffer
+        SGNN_REQUIRE(ldo % vec == 0 && aligned(out, 4 * vec),
+                     "the fused path at F=%lld needs out %d-byte aligned with ldo %% %d == 0", (long long)F, 4 * vec, vec);
     } else if (F % 4 == 0 && dense.ldx % 4 == 0 && ldo % 4 == 0 && aligned(dense.x, 16) && aligned(out, 16)) {
         vec = 4;
     } else if (F % 2 == 0 && dense.ldx % 2 == 0 && ldo % 2 == 0 && aligned(dense.x, 8) && aligned(out, 8)) {
@@ -1945,7 +1957,7 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     if (bits != 0) {
         const int fmt = bits + (dense.params.bf16 ? kBf16Params : 0) + (dense.eslot_csr ? kEdgeSlots : 0);
         switch (fmt) {
-#define SGNN_DQ(FMT) case FMT: dispatch_shape_dq<FMT>(nvec, a, s, f, st); break
+#define SGNN_DQ(FMT) case FMT: dispatch_shape_dq<FMT>(vec, nvec, a, s, f, st); break
             SGNN_DQ(8); SGNN_DQ(4); SGNN_DQ(2);
             SGNN_DQ(8 + kBf16Params); SGNN_DQ(4 + kBf16Params); SGNN_DQ(2 + kBf16Params);
             SGNN_DQ(8 + kEdgeSlots); SGNN_DQ(4 + kEdgeSlots); SGNN_DQ(2 + kEdgeSlots);
@@ -2026,7 +2038,7 @@ static int spmm_dq_impl(sgnn_spmm_plan *p, const float *val, const uint8_t *q, c
     SGNN_REQUIRE(p != nullptr, "plan is null");
     SGNN_REQUIRE(bits == 8 || bits == 4 || bits == 2, "bits=%d, expected 8, 4 or 2", bits);
     SGNN_REQUIRE(params_bf16 == 0 || params_bf16 == 1, "params_bf16=%d, expected 0 or 1", params_bf16);
-    SGNN_REQUIRE(F % 4 == 0, "the fused path needs F %% 4 == 0 (F=%lld): dequantize, then call sgnn_spmm_csr_f32", (long long)F);
+    SGNN_REQUIRE(F % 2 == 0, "the fused path needs an even feature width (F=%lld): dequantize, then call sgnn_spmm_csr_f32", (long long)F);
     SGNN_REQUIRE((q != nullptr && params != nullptr) || p->nnz == 0 || p->M == 0, "q / params is null");
     SGNN_REQUIRE(aligned(q, 4) && aligned(params, params_bf16 ? 4 : 8), "q must be 4-byte and params %d-byte aligned",
                  params_bf16 ? 4 : 8);

@@ -208,8 +208,8 @@ class SpmmPlan:
         if out.dim() != 2 or out.shape[0] != self.M:
             raise ValueError(f"out must be [{self.M}, F]")
         F = out.shape[1]
-        if F % 4:
-            raise ValueError("the fused path needs a feature width divisible by 4")
+        if F % 2:
+            raise ValueError("the fused path needs an even feature width")
         if segs.n_rows != self.K:
             raise ValueError(f"the segment table covers {segs.n_rows} rows, the sparse matrix has {self.K} columns")
         if data_int8.numel() < segs.n_packed * F or params.numel() < self.K * 2:

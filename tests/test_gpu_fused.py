@@ -41,6 +41,10 @@ def _setup(M, K, F, deg, bits, seg, seed, hubs=0):
     (200, 180, 1024, 4, [0, 180], 0),                 # 4 words per lane
     (150, 120, 100, 5, [0, 61, 120], 0),              # partly idle group
     (120, 90, 8, 5, [0, 90], 0),
+    (400, 350, 602, 8, [0, 350], 3),                  # even width that is not a multiple of four: two-code lanes, five per lane
+    (300, 256, 130, 6, [0, 100, 256], 2),             # two-code lanes, two per lane, ragged segments
+    (200, 180, 6, 5, [0, 61, 180], 1),                # three two-code lanes
+    (100, 90, 1030, 4, [0, 90], 0),                   # two-code lanes walking the feature axis in two tiles
 ])
 def test_fused_equals_separate_and_oracle(bits, M, K, F, deg, seg, hubs):
     ops, plan, rowptr, col, val, x, seg_t, P, q, params = _setup(M, K, F, deg, bits, seg, seed=M + F + bits, hubs=hubs)
@@ -133,7 +137,7 @@ def test_fused_errors():
     with pytest.raises(ValueError):
         ops.spmm_dequantized(None, None, None, q, params, torch.tensor([0, 39], dtype=torch.int32), 1, 2, out, plan=plan)
     with pytest.raises(ValueError):
-        ops.spmm_dequantized(None, None, None, q, params, seg_t, P, 2, torch.zeros(50, 62, device="cuda"), plan=plan)
+        ops.spmm_dequantized(None, None, None, q, params, seg_t, P, 2, torch.zeros(50, 63, device="cuda"), plan=plan)  # odd width
 
 
 @pytest.mark.parametrize("bits", [8, 2])

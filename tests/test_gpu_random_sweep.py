@@ -99,7 +99,7 @@ def test_fused_random_shapes(case):
     from super_gnn_amd import supergnn_ops as ops
     rng = np.random.default_rng(3000 + case)
     bits = int(rng.choice([8, 4, 2]))
-    F = int(rng.choice([4, 8, 12, 36, 64, 100, 128, 256, 260, 512, 1028]))
+    F = int(rng.choice([4, 8, 12, 36, 64, 100, 128, 256, 260, 512, 1028, 2, 6, 130, 602, 1030]))
     M, K = int(rng.integers(1, 1500)), int(rng.integers(8, 1500))
     deg = int(rng.choice([1, 3, 9, 40]))
     hubs = int(rng.choice([0, 0, 3]))
