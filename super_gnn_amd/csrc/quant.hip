@@ -312,7 +312,14 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
 // the float4 loads and the 4-byte code stores are issued at their natural (unaligned) addresses, and the one
 // vector per row that reaches past the end of the row is loaded and stored element by element, its missing
 // elements filled with copies of its first one (copies change neither min nor max nor the first-zero rule).
-template <int BITS, int NV, int RL, bool kForceExactDivision, bool FULL = false, int L = 16, bool RAGGED = false>
+// STAGED: the packed bytes of a wavefront (RL * 64 / L consecutive fp32 rows = consecutive packed rows, one
+// contiguous run of the output) first go to a wave-private piece of LDS and are then written with 4-byte stores
+// over that run, 256 consecutive bytes per store instruction, instead of one 64-byte piece per lane group and
+// vector.  For rows that do not start on cache lines the many short, oddly aligned pieces are what limits the
+// kernel (F = 602 int2: 5.2 -> 6.4 TB/s with the output redirected into a cache-resident window).
+constexpr int kStageBytes = 4096 + 16;  // per wavefront: at most 4 packed rows of 1024 bytes (int8, F = 1024)
+template <int BITS, int NV, int RL, bool kForceExactDivision, bool FULL = false, int L = 16, bool RAGGED = false,
+          bool STAGED = false>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
     const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F,
@@ -467,6 +474,11 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
         }
     }
     // Pack: shift to the row's bit position, OR across the DPP rows that share a packed row, store.
+    __shared__ __align__(16) uint8_t stage_all[STAGED ? kQBlock / 64 : 1][STAGED ? kStageBytes : 16];
+    uint8_t *stage = stage_all[STAGED ? (threadIdx.x >> 6) : 0];
+    const int gp_first = (unit * RL * RW) / EPB;                       // the wavefront's first packed row
+    const int64_t run_lo = (int64_t)gp_first * F;                      // byte offset of its output run
+    const int mis = (int)((reinterpret_cast<uintptr_t>(q) + (uint64_t)run_lo) & 3);  // the LDS copy keeps the run's alignment modulo 4
 #pragma unroll
     for (int rl = 0; rl < RL; ++rl) {
 #pragma unroll
@@ -480,6 +492,22 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
                 if constexpr (EPB == 4) w |= (uint32_t)__shfl_xor((int)w, 16, 64);
             }
             const bool mine = EPB == 1 ? true : EPB == 2 ? ((d & 1) == (v & 1)) : ((d & 3) == (v & 3));
+            if constexpr (STAGED) {
+                if (mine && act[v] && gp[rl] < n_packed) {
+                    uint8_t *dst = stage + mis + (gp[rl] - gp_first) * F + off[v];
+                    const int nb = RAGGED ? (F - off[v] < VEC ? F - off[v] : VEC) : VEC;
+                    const uintptr_t al = reinterpret_cast<uintptr_t>(dst) & 3;
+                    if (nb == VEC && al == 0) {
+                        *reinterpret_cast<uint32_t *>(dst) = w;
+                    } else if (nb == VEC && al == 2) {
+                        reinterpret_cast<uint16_t *>(dst)[0] = (uint16_t)w;
+                        reinterpret_cast<uint16_t *>(dst)[1] = (uint16_t)(w >> 16);
+                    } else {
+                        for (int k = 0; k < nb; ++k) dst[k] = (uint8_t)(w >> (8 * k));
+                    }
+                }
+                continue;
+            }
             if (mine && act[v] && gp[rl] < n_packed) {
                 uint8_t *dst = q + (int64_t)gp[rl] * F + off[v];
                 if constexpr (RAGGED) {
@@ -502,6 +530,25 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
                 }
             }
         }
+    }
+    if constexpr (STAGED) {
+        // LDS operations of one wavefront complete in program order; the fence keeps the compiler from moving
+        // the reads below above the writes of other lanes.
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        int gp_end = gp_first + RL * RW / EPB;
+        if (gp_end > n_packed) gp_end = n_packed;
+        const int nbytes = (gp_end - gp_first) * F;                    // the run [run_lo, run_lo + nbytes)
+        uint8_t *qo = q + run_lo;
+        int head = (4 - mis) & 3;
+        if (head > nbytes) head = nbytes;
+        const int ndw = (nbytes - head) >> 2;
+        const int tail_bytes = nbytes - head - 4 * ndw;
+        if (lane < head) qo[lane] = stage[mis + lane];
+        const uint32_t *s32 = reinterpret_cast<const uint32_t *>(stage + mis + head);   // (mis + head) % 4 == 0 whenever ndw > 0
+        uint32_t *q32 = reinterpret_cast<uint32_t *>(qo + head);
+        for (int i = lane; i < ndw; i += 64) __builtin_nontemporal_store(s32[i], q32 + i);
+        if (lane < tail_bytes) qo[head + 4 * ndw + lane] = stage[mis + head + 4 * ndw + lane];
     }
 }
 
@@ -1254,6 +1301,15 @@ static void launch_rows(const RowsArgs &a, hipStream_t st) {
                            a.x_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
+// Rows that are not a whole number of lane-group passes (every width but 4 * L * NV floats) write their packed
+// bytes through the wave-private LDS stage (SGNN_QUANT_STAGED=0: straight from the lanes, for comparison).  Measured
+// on MI355X at 256 M elements: F = 300 / 600 / 1000 5.2-5.9 -> 6.0-6.2 TB/s, F = 602 4.7-5.2 -> 5.6-5.9 TB/s; rows that
+// are whole passes (F = 64 ... 1024 in steps of the lane-group width) gain nothing from it and keep the direct stores.
+static bool quant_staged_output() {
+    static const bool on = [] { const char *e = getenv("SGNN_QUANT_STAGED"); return !(e && e[0] == '0'); }();
+    return on;
+}
+
 template <int BITS, int NV, int L>
 static void launch_quant16_ragged(const RowsArgs &a, hipStream_t st) {
     constexpr int RL = NV >= 4 ? 1 : 4 / NV;
@@ -1263,8 +1319,12 @@ static void launch_quant16_ragged(const RowsArgs &a, hipStream_t st) {
     const int n_units = (int)((padded + RW * RL - 1) / (RW * RL));
     const int nb = (n_units + kQBlock / 64 - 1) / (kQBlock / 64);
     ProfScope prof(K_QUANT_PACK_ROWS, st);
-    hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
-                       a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
+    if (quant_staged_output())
+        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L, true, true>), dim3(nb), dim3(kQBlock), 0, st,
+                           a.x_in, a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
+    else
+        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
+                           a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
 // Widths or row starts that are not a multiple of four floats, up to 1024 floats per row.
@@ -1295,6 +1355,9 @@ static void launch_quant16(const RowsArgs &a, hipStream_t st) {
     else if (a.F == 4 * L * NV)
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, true, L>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
                            a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
+    else if (quant_staged_output())
+        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L, false, true>), dim3(nb), dim3(kQBlock), 0, st,
+                           a.x_in, a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
     else
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
                            a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
