@@ -709,11 +709,13 @@ def main():
             cpu_saved = args.no_cpu
             args.no_cpu = args.no_cpu or name in ("sbm", "prepost")
             others[name] = brief(WORKLOADS[name](args, ctx))
-            if name == "quant":   # the narrow rows the live path exchanges (F = 128, 64): more rows for the same bytes
+            if name == "quant":   # the narrow rows the live path exchanges (F = 128, 64): more rows for the same bytes;
                 torch.cuda.empty_cache()
                 others["quant_F128"] = brief(wl_quant(args, ctx, rows=2 * args.quant_rows, feat=128, headline=False))
                 torch.cuda.empty_cache()
                 others["quant_F64"] = brief(wl_quant(args, ctx, rows=4 * args.quant_rows, feat=64, headline=False))
+                torch.cuda.empty_cache()  # rows that do not start on cache lines: the dense-degree graph's feature width
+                others["quant_F602"] = brief(wl_quant(args, ctx, rows=425_000 * args.quant_rows // 1_000_000, feat=602, headline=False))
             args.no_cpu = cpu_saved
             log(f"[bench] extra workload {name}: {time.perf_counter() - t0:.1f}s")
         args.steps, args.warmup = saved
