@@ -68,6 +68,13 @@ __device__ __forceinline__ uint32_t xcd_contiguous_block(uint32_t bid, uint32_t 
     return xcd * per + (xcd < rem ? xcd : rem) + idx;
 }
 
+// The first active lane's 64-bit value, as a wave-uniform (scalar) value.
+__device__ __forceinline__ int64_t uniform64(int64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 template <int VEC>
 __device__ __forceinline__ void vec_load(float (&r)[VEC], const float *p) {
     if constexpr (VEC == 4) {

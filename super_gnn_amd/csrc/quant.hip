@@ -1079,6 +1079,58 @@ __global__ __launch_bounds__(kQBlock) void quant_v1_vec_kernel(const float *__re
     }
 }
 
+// SGNN_V1_STAGED=0 at build time restores the direct stores of the v1 quantizer (for comparison).
+#ifndef SGNN_V1_STAGED
+#define SGNN_V1_STAGED 1
+#endif
+constexpr bool kV1Staged = SGNN_V1_STAGED;
+
+// True when the byte ranges [r0, r1) of a wavefront's rows (row index = round * RW + lane group) follow one another
+// without gaps: each row ends where the next begins.  Wave-uniform.
+template <int R>
+__device__ __forceinline__ bool contiguous_rows(const int64_t (&r0)[R], const int64_t (&r1)[R], int L) {
+    const int lane = threadIdx.x & 63;
+    bool ok = true;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        // the next row sits L lanes further on, or in lane group 0 of the next round
+        const int64_t nxt_same = __shfl_down(r0[r], L, 64);
+        const int64_t nxt_round = __shfl(r0[r + 1 < R ? r + 1 : r], lane % L, 64);
+        if (lane + L < 64) ok = ok && r1[r] == nxt_same;
+        else if (r + 1 < R) ok = ok && r1[r] == nxt_round;
+    }
+    return __ballot(!ok) == 0ull;
+}
+
+// The four codes of one lane of a v1 row, packed and stored at the row's byte position for columns off .. off+3:
+// 4 / 2 / 1 bytes at 8 / 4 / 2 bits, in one store when the address allows it.  NT: non-temporal (global memory).
+template <bool NT>
+__device__ __forceinline__ void store_v1_codes(uint8_t *row_bytes, int off, int b, const uint32_t (&c)[4]) {
+    if (b == 8) {
+        uint8_t *dst = row_bytes + off;
+        const uint32_t w = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+        if ((reinterpret_cast<uintptr_t>(dst) & 3) == 0) {
+            if constexpr (NT) __builtin_nontemporal_store(w, reinterpret_cast<uint32_t *>(dst));
+            else *reinterpret_cast<uint32_t *>(dst) = w;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) dst[k] = (uint8_t)c[k];
+        }
+    } else if (b == 4) {
+        uint8_t *dst = row_bytes + off / 2;
+        const uint32_t b0 = (c[0] << 4) | c[1], b1 = (c[2] << 4) | c[3];
+        if ((reinterpret_cast<uintptr_t>(dst) & 1) == 0) {
+            if constexpr (NT) __builtin_nontemporal_store((uint16_t)(b0 | (b1 << 8)), reinterpret_cast<uint16_t *>(dst));
+            else *reinterpret_cast<uint16_t *>(dst) = (uint16_t)(b0 | (b1 << 8));
+        } else {
+            dst[0] = (uint8_t)b0;
+            dst[1] = (uint8_t)b1;
+        }
+    } else {
+        row_bytes[off / 4] = (uint8_t)((c[0] << 6) | (c[1] << 4) | (c[2] << 2) | c[3]);
+    }
+}
+
 // The quantizer once more with L = 16 or 8 lanes per row instead of a whole wavefront (F <= 4 * L * NV): the
 // min/max/zero-sign reductions stay inside a DPP row (four or three butterfly steps, no readlane round trips), a
 // wavefront carries 64/L rows side by side and R such rounds, and rows of different bit widths simply take
@@ -1093,7 +1145,7 @@ __global__ __launch_bounds__(kQBlock) void quant_v1_group_kernel(const float *__
     const int64_t i0 = unit * (RW * R);
     if (i0 >= n) return;  // wave-uniform
     float bits_f[R];
-    int64_t r0[R];
+    int64_t r0[R], r1[R];
     float xv[R][NV][4];
     int off[NV];
     bool act[NV];
@@ -1107,9 +1159,31 @@ __global__ __launch_bounds__(kQBlock) void quant_v1_group_kernel(const float *__
         const int64_t i = i0 + r * RW + d < n ? i0 + r * RW + d : n - 1;  // rows past the end repeat the last row's loads
         bits_f[r] = params[i * 3];
         r0[r] = range[i];
+        r1[r] = range[i + 1];
 #pragma unroll
         for (int v = 0; v < NV; ++v) vec_load_nt<4>(xv[r][v], x + i * F + (act[v] ? off[v] : 0));  // unconditional
     }
+    // The wavefront's rows are consecutive, and so -- in the layout the reference builds (row i's bytes end where
+    // row i + 1's begin) -- are their packed bytes: one run of the output.  When every row of the wavefront exists,
+    // has a legal bit width and lies where that layout puts it, the codes go to a wave-private piece of LDS first
+    // and then out as 4-byte stores over the run (256 consecutive bytes per instruction instead of one 8- to
+    // 64-byte piece per lane group and vector: F = 128 at 8 bits 3.9 -> 6.2 TB/s, mixed widths 4.4 -> 6.3);
+    // otherwise the lanes store their pieces themselves.
+    constexpr int kStage = RW * R * L * NV * 4;   // bytes of the wavefront's rows at 8 bits
+    __shared__ __align__(16) uint8_t stage_all[kQBlock / 64][kStage + 16];
+    uint8_t *stage = stage_all[threadIdx.x >> 6];
+    bool lane_ok = true;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int b = (int)bits_f[r];
+        const bool legal = b == 8 || b == 4 || b == 2;
+        lane_ok = lane_ok && i0 + r * RW + d < n && legal && r1[r] - r0[r] == (int64_t)((F * (legal ? b : 8) + 7) / 8);
+    }
+    const int64_t run_lo = uniform64(r0[0]);                                             // lane 0 holds the wavefront's first row
+    const int64_t run_hi = range[i0 + RW * R < n ? i0 + RW * R : n];
+    const bool rows_ok = __ballot(!lane_ok) == 0ull;
+    const bool staged = kV1Staged && contiguous_rows<R>(r0, r1, L) && rows_ok && run_hi - run_lo <= (int64_t)kStage;
+    const int mis = (int)((reinterpret_cast<uintptr_t>(q) + (uint64_t)run_lo) & 3);     // the LDS copy keeps the run's alignment modulo 4
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int64_t i = i0 + r * RW + d;
@@ -1159,27 +1233,24 @@ __global__ __launch_bounds__(kQBlock) void quant_v1_group_kernel(const float *__
 #pragma unroll
                 for (int k = 0; k < 4; ++k) c[k] = quant_code(xv[r][v][k], mn, s);
             }
-            if (b == 8) {
-                uint8_t *dst = qo + off[v];
-                if ((r0[r] & 3) == 0) {
-                    __builtin_nontemporal_store(c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24), reinterpret_cast<uint32_t *>(dst));
-                } else {
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) dst[k] = (uint8_t)c[k];
-                }
-            } else if (b == 4) {
-                uint8_t *dst = qo + off[v] / 2;
-                const uint32_t b0 = (c[0] << 4) | c[1], b1 = (c[2] << 4) | c[3];
-                if ((r0[r] & 1) == 0) {
-                    __builtin_nontemporal_store((uint16_t)(b0 | (b1 << 8)), reinterpret_cast<uint16_t *>(dst));
-                } else {
-                    dst[0] = (uint8_t)b0;
-                    dst[1] = (uint8_t)b1;
-                }
-            } else {
-                qo[off[v] / 4] = (uint8_t)((c[0] << 6) | (c[1] << 4) | (c[2] << 2) | c[3]);
-            }
+            if (staged) store_v1_codes<false>(stage + mis + (int)(r0[r] - run_lo), off[v], b, c);
+            else store_v1_codes<true>(qo, off[v], b, c);
         }
+    }
+    if (staged) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // LDS operations of one wavefront complete in program order
+        __builtin_amdgcn_wave_barrier();
+        const int nbytes = (int)(run_hi - run_lo);
+        uint8_t *qrun = q + run_lo;
+        int head = (4 - mis) & 3;
+        if (head > nbytes) head = nbytes;
+        const int ndw = (nbytes - head) >> 2;
+        const int tail_bytes = nbytes - head - 4 * ndw;
+        if (lane < head) qrun[lane] = stage[mis + lane];
+        const uint32_t *s32 = reinterpret_cast<const uint32_t *>(stage + mis + head);
+        uint32_t *q32 = reinterpret_cast<uint32_t *>(qrun + head);
+        for (int i = lane; i < ndw; i += 64) __builtin_nontemporal_store(s32[i], q32 + i);
+        if (lane < tail_bytes) qrun[head + 4 * ndw + lane] = stage[mis + head + 4 * ndw + lane];
     }
 }
 
@@ -1250,6 +1321,67 @@ __global__ __launch_bounds__(kQBlock) void dequant_v1_vec_kernel(const uint8_t *
             for (int k = 0; k < 4; ++k) o[k] = fmaf((float)c[k], sc[r], zp[r]);
             vec_store_nt<4>(xo + off, o);
         }
+    }
+}
+
+// The v1 dequantizer over the flat output (F % 4 == 0): as in unpack_dequant_flat_kernel every wavefront store
+// covers 1 KB of consecutive output whatever the row width, and a lane looks up what it needs for its four
+// elements -- its row's bit width, params and byte offset, then one to four code bytes -- with cacheable
+// loads.  Narrow rows no longer leave most of a wavefront idle (F = 64: a wavefront-per-row kernel has 16 of
+// 64 lanes at work).
+template <int R>
+__global__ __launch_bounds__(kQBlock) void dequant_v1_flat_kernel(const uint8_t *__restrict__ q, float *__restrict__ x,
+                                                                  const int64_t *__restrict__ range,
+                                                                  const float *__restrict__ params, int64_t n_vec, int G) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
+    const int64_t base = wave * (R * 64) + lane;
+    uint32_t w[R];
+    float zp[R], sc[R];
+    int b[R];
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const int64_t i = base + u * 64;
+        w[u] = 0; zp[u] = 0.0f; sc[u] = 0.0f; b[u] = 0;
+        if (i >= n_vec) continue;
+        const int64_t row = i / G;
+        const int col = (int)(i - row * G) * 4;
+        b[u] = (int)params[row * 3];
+        zp[u] = params[row * 3 + 1];
+        sc[u] = params[row * 3 + 2];
+        const int64_t r0 = range[row];
+        const uint8_t *qi = q + r0;
+        if (b[u] == 8) {
+            const uint8_t *src = qi + col;
+            if ((r0 & 3) == 0) w[u] = *reinterpret_cast<const uint32_t *>(src);
+            else w[u] = src[0] | (src[1] << 8) | (src[2] << 16) | ((uint32_t)src[3] << 24);
+        } else if (b[u] == 4) {
+            const uint8_t *src = qi + col / 2;
+            if ((r0 & 1) == 0) w[u] = *reinterpret_cast<const uint16_t *>(src);
+            else w[u] = src[0] | (src[1] << 8);
+        } else if (b[u] == 2) {
+            w[u] = qi[col / 4];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const int64_t i = base + u * 64;
+        if (i >= n_vec || (b[u] != 8 && b[u] != 4 && b[u] != 2)) continue;  // other widths: the row is left alone
+        const uint32_t ww = w[u];
+        uint32_t c[4];
+        if (b[u] == 8) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) c[k] = (ww >> (8 * k)) & 255u;
+        } else if (b[u] == 4) {
+            c[0] = (ww >> 4) & 15u; c[1] = ww & 15u; c[2] = (ww >> 12) & 15u; c[3] = (ww >> 8) & 15u;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) c[k] = (ww >> (6 - 2 * k)) & 3u;
+        }
+        float o[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) o[k] = fmaf((float)c[k], sc[u], zp[u]);
+        vec_store_nt<4>(x + i * 4, o);
     }
 }
 
@@ -1641,7 +1773,16 @@ extern "C" int sgnn_dequant_v1_f32(const uint8_t *q, float *x, const int64_t *ra
     const dim3 grid((uint32_t)nb), block(kQBlock);
     const auto grid_r = [&](int rows) { return dim3((uint32_t)((nb + rows - 1) / rows)); };
     hipStream_t st = (hipStream_t)stream;
-    if (F % 4 == 0 && F <= 1024 && aligned(x, 16)) {
+    // narrow rows (a wavefront per row leaves lanes idle) and rows beyond the vector kernel's width: flat output
+    // (SGNN_DEQUANT_V1_FLAT=0 / 1: never / at every width, for comparison)
+    static const int flat_mode = [] { const char *e = getenv("SGNN_DEQUANT_V1_FLAT"); return e ? atoi(e) : -1; }();
+    if (F % 4 == 0 && aligned(x, 16) && (flat_mode == 1 || (flat_mode != 0 && (F <= 128 || F > 1024)))) {
+        constexpr int R = 2;
+        const int64_t n_vec = n * (F / 4);
+        const int64_t n_waves = (n_vec + R * 64 - 1) / (R * 64);
+        hipLaunchKernelGGL((dequant_v1_flat_kernel<R>), dim3((uint32_t)((n_waves + kQBlock / 64 - 1) / (kQBlock / 64))), block, 0, st,
+                           q, x, range, params, n_vec, (int)(F / 4));
+    } else if (F % 4 == 0 && F <= 1024 && aligned(x, 16)) {
         if (F <= 256) hipLaunchKernelGGL((dequant_v1_vec_kernel<1, 4>), grid_r(4), block, 0, st, q, x, range, params, n, (int)F);
         else if (F <= 512) hipLaunchKernelGGL((dequant_v1_vec_kernel<2, 2>), grid_r(2), block, 0, st, q, x, range, params, n, (int)F);
         else hipLaunchKernelGGL((dequant_v1_vec_kernel<4, 1>), grid, block, 0, st, q, x, range, params, n, (int)F);

@@ -54,12 +54,6 @@ __device__ __forceinline__ float group_bcast_f(float v, int src) {
     return __int_as_float(group_bcast_i<G>(__float_as_int(v), src));
 }
 
-__device__ __forceinline__ int64_t uniform64(int64_t v) {
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
-    return (int64_t)(((uint64_t)hi << 32) | lo);
-}
-
 // The dense operand of the product: fp32 rows (BITS == 0), or rows that arrive quantized and
 // bit-packed in the row-group layout (see quant.hip) and are decoded on the fly.  For those the
 // template parameter BITS is a format code: the low four bits are the code width (8, 4 or 2) and

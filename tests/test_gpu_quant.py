@@ -453,6 +453,50 @@ def test_v1_mixed_bits_all_widths(F):
     assert np.all(np.abs(back.cpu().numpy() - want) <= tol)
 
 
+@pytest.mark.parametrize("F", [32, 64, 128, 256, 512])
+def test_v1_rows_with_gaps_and_illegal_widths(F):
+    """The v1 quantizer gathers a wavefront's rows into one run of stores when the rows' byte ranges follow one
+    another; ranges with gaps between rows, rows of an illegal bit width (left untouched, as the reference leaves
+    them, quantization_x86.cpp:244-245) and the last, partly filled wavefront must take the per-row stores and
+    leave every byte outside the rows' ranges alone."""
+    from super_gnn_amd import supergnn_ops as ops, _lib
+    rng_ = np.random.default_rng(100 + F)
+    n = 1003
+    x = rng_.standard_normal((n, F)).astype(np.float32)
+    bits = rng_.choice([2, 4, 8], size=n)
+    q_ref, r_ref, p_ref = orc.quant_v1(x, bits)
+    length = np.diff(r_ref)
+    for gaps, bad in ((True, []), (False, [17, 500, 501, 1002]), (True, [0, 64])):
+        start = r_ref[:-1] + (3 * np.arange(n) if gaps else 0)
+        rng_dev = np.concatenate([start, [start[-1] + length[-1] + (3 if gaps else 0)]]).astype(np.int64)
+        total = int(rng_dev[-1]) + 8
+        q = torch.full((total,), 0xAB, dtype=torch.uint8, device="cuda")
+        prm = torch.full((n, 3), -7.0, device="cuda")
+        b_dev = bits.astype(np.float32).copy()
+        b_dev[bad] = 3.0
+        prm[:, 0] = torch.from_numpy(b_dev).cuda()
+        xd, rd = torch.from_numpy(x).cuda(), torch.from_numpy(rng_dev).cuda()
+        # through the C ABI: the Python wrapper refuses illegal widths before the library sees them
+        _lib.check(_lib.lib.sgnn_quant_v1_f32(xd.data_ptr(), q.data_ptr(), rd.data_ptr(), prm.data_ptr(), n, F, ops._stream()))
+        got, gp = q.cpu().numpy(), prm.cpu().numpy()
+        want = np.full(total, 0xAB, dtype=np.uint8)
+        for i in range(n):
+            if i in bad:
+                assert gp[i, 1] == -7.0 and gp[i, 2] == -7.0
+                continue
+            want[start[i]:start[i] + length[i]] = q_ref[r_ref[i]:r_ref[i + 1]]
+            assert gp[i, 1] == p_ref[i, 1] and gp[i, 2] == p_ref[i, 2]
+        assert np.array_equal(got, want), f"gaps={gaps} bad={bad}"
+        # and back: rows of an illegal width keep what the output held
+        back = torch.full((n, F), 9.0, device="cuda")
+        _lib.check(_lib.lib.sgnn_dequant_v1_f32(q.data_ptr(), back.data_ptr(), rd.data_ptr(), prm.data_ptr(), n, F, ops._stream()))
+        wantx = orc.dequant_v1(q_ref, r_ref, p_ref, F)
+        wantx[bad] = 9.0
+        tol = dequant_atol(p_ref[:, 1], p_ref[:, 2], bits)[:, None]
+        tol[bad] = 0.0
+        assert np.all(np.abs(back.cpu().numpy() - wantx) <= tol)
+
+
 def test_offsets_beyond_four_gigabytes():
     # 9 M x 128 fp32 = 4.6 GB: byte offsets of the last rows do not fit 32 bits.  Params against torch's
     # min/max, the round-trip bound everywhere, and the last rows of every segment bit-exact against the oracle.
