@@ -57,8 +57,11 @@ int sgnn_version(void);
 typedef struct sgnn_spmm_plan sgnn_spmm_plan;
 
 /* rowptr: int64[M+1] (device). col: int64[nnz] if col_is_i64 else int32[nnz] (device).
- * K = number of sparse columns = rows of the dense operand.  M, K and nnz must be below 2^31 (the
+ * K = number of sparse columns = rows of the dense operand.  M and K must be below 2^31 (the
  * reference's kernel computes its offsets in 32-bit int as well, super_gnn/ops/csrc/spmm.cpp:30,94).
+ * nnz may be larger: a matrix of 2^31 edges or more is held as consecutive row blocks of fewer edges,
+ * each scheduled on its own, and every call on the plan runs the blocks one after the other on the
+ * caller's stream (same results; a single row must still have fewer than 2^31 edges).
  * Every col must lie in [0, K) and rowptr must be non-decreasing with rowptr[0] == 0: both are
  * checked (SGNN_ERR_RANGE).
  * long_row_threshold: rows with more edges take the long-row path (<= 0: default 128).

@@ -1283,6 +1283,10 @@ struct sgnn_spmm_plan {
     std::vector<BandSchedule *> bands;
     float *band_xs = nullptr;       // the dense operand restaged slice by slice (see band_restage_kernel), grown on demand
     size_t band_xs_floats = 0;
+    // A matrix with 2^31 edges or more is held as consecutive row blocks, each a plan of its own with fewer
+    // edges than that (the kernels' edge offsets are 32-bit); every call on the whole runs the blocks in turn.
+    std::vector<sgnn_spmm_plan *> parts;
+    std::vector<int64_t> part_row0, part_edge0;
     // Short-row chunks, one list per chunk row limit (7, 15, 31).
     std::vector<int64_t> h_rowptr;
     int4 *chunks[3] = {nullptr, nullptr, nullptr};
@@ -1330,6 +1334,7 @@ static int build_chunks(sgnn_spmm_plan *p, int which, hipStream_t st) {
 
 extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     if (!p) return SGNN_OK;
+    for (sgnn_spmm_plan *part : p->parts) (void)sgnn_spmm_plan_destroy(part);
     (void)hipFree(p->rowptr);
     (void)hipFree(p->col);
     (void)hipFree(p->long_rows);
@@ -1527,6 +1532,56 @@ static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void
     return SGNN_OK;
 }
 
+// Most edges one plan holds (the kernels address edges with 32-bit offsets).  SGNN_SPMM_PART_EDGES lowers it so
+// that the row-block path can be exercised on small matrices.
+static int64_t part_edge_cap() {
+    const int64_t dflt = (int64_t)INT32_MAX - ((int64_t)1 << 20);
+    const char *e = getenv("SGNN_SPMM_PART_EDGES");
+    const int64_t v = e ? atoll(e) : 0;
+    return v > 0 && v < dflt ? v : dflt;
+}
+
+// A matrix with more edges than one plan holds: consecutive row blocks of at most `cap` edges, each a plan of its
+// own over a rebased copy of its slice of rowptr.  A single row longer than the cap is refused.
+static int plan_create_parts(sgnn_spmm_plan *p, const int64_t *rowptr, const void *col, int col_is_i64, int64_t cap,
+                             hipStream_t st) {
+    const int64_t M = p->M;
+    SGNN_HIP_CHECK(hipGetDevice(&p->device));
+    std::vector<int64_t> h((size_t)M + 1);
+    SGNN_HIP_CHECK(hipMemcpyAsync(h.data(), rowptr, sizeof(int64_t) * h.size(), hipMemcpyDeviceToHost, st));
+    SGNN_HIP_CHECK(hipStreamSynchronize(st));
+    if (h[0] != 0) return fail(SGNN_ERR_RANGE, "rowptr[0] = %lld, expected 0", (long long)h[0]);
+    for (int64_t m = 0; m < M; ++m)
+        if (h[m + 1] < h[m]) return fail(SGNN_ERR_RANGE, "rowptr decreases at row %lld", (long long)m);
+    if (h[M] != p->nnz) return fail(SGNN_ERR_RANGE, "rowptr[M] = %lld but nnz = %lld", (long long)h[M], (long long)p->nnz);
+    const size_t col_bytes = col_is_i64 ? sizeof(int64_t) : sizeof(int32_t);
+    int64_t r0 = 0;
+    while (r0 < M) {
+        // the longest run of rows from r0 on with at most `cap` edges
+        int64_t r1 = std::upper_bound(h.begin() + r0, h.end(), h[r0] + cap) - h.begin() - 1;
+        if (r1 <= r0)
+            return fail(SGNN_ERR_ARG, "row %lld has %lld edges, more than one plan holds (%lld)", (long long)r0,
+                        (long long)(h[r0 + 1] - h[r0]), (long long)cap);
+        if (r1 > M) r1 = M;
+        std::vector<int64_t> rebased((size_t)(r1 - r0) + 1);
+        for (int64_t i = r0; i <= r1; ++i) rebased[(size_t)(i - r0)] = h[i] - h[r0];
+        DevTmp<int64_t> d_rp;
+        int rc = upload(&d_rp.p, rebased, st);
+        if (rc != SGNN_OK) return rc;
+        sgnn_spmm_plan *part = new sgnn_spmm_plan();
+        p->parts.push_back(part);  // owned from here on: destroyed with the whole
+        p->part_row0.push_back(r0);
+        p->part_edge0.push_back(h[r0]);
+        part->M = r1 - r0; part->K = p->K; part->nnz = h[r1] - h[r0];
+        part->long_thresh = p->long_thresh; part->piece_edges = p->piece_edges;
+        rc = plan_create_impl(part, d_rp.p, (const char *)col + (size_t)h[r0] * col_bytes, col_is_i64, st);
+        if (rc != SGNN_OK) return rc;
+        SGNN_HIP_CHECK(hipStreamSynchronize(st));  // the rebased row pointers die at the end of the iteration
+        r0 = r1;
+    }
+    return SGNN_OK;
+}
+
 extern "C" int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int col_is_i64, int64_t M, int64_t K,
                                      int64_t nnz, int long_row_threshold, int piece_edges,
                                      sgnn_stream_t stream, sgnn_spmm_plan **plan_out) {
@@ -1534,14 +1589,15 @@ extern "C" int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int
     *plan_out = nullptr;
     SGNN_REQUIRE(rowptr != nullptr, "rowptr is null");
     SGNN_REQUIRE(M >= 0 && K >= 0 && nnz >= 0, "negative size (M=%lld K=%lld nnz=%lld)", (long long)M, (long long)K, (long long)nnz);
-    SGNN_REQUIRE(M < INT32_MAX && K < INT32_MAX && nnz < INT32_MAX,
-                 "M, K and nnz must fit 31 bits (M=%lld K=%lld nnz=%lld)", (long long)M, (long long)K, (long long)nnz);
+    SGNN_REQUIRE(M < INT32_MAX && K < INT32_MAX, "M and K must fit 31 bits (M=%lld K=%lld)", (long long)M, (long long)K);
     SGNN_REQUIRE(nnz == 0 || col != nullptr, "col is null with nnz=%lld", (long long)nnz);
     sgnn_spmm_plan *p = new sgnn_spmm_plan();
     p->M = M; p->K = K; p->nnz = nnz;
     p->long_thresh = long_row_threshold > 0 ? long_row_threshold : env_int("SGNN_SPMM_LONG_THRESHOLD", kDefaultLongThreshold);
     p->piece_edges = piece_edges > 0 ? piece_edges : env_int("SGNN_SPMM_PIECE_EDGES", kDefaultPieceEdges);
-    const int rc = plan_create_impl(p, rowptr, col, col_is_i64, (hipStream_t)stream);
+    const int64_t part_cap = part_edge_cap();
+    const int rc = nnz <= part_cap ? plan_create_impl(p, rowptr, col, col_is_i64, (hipStream_t)stream)
+                                   : plan_create_parts(p, rowptr, col, col_is_i64, part_cap, (hipStream_t)stream);
     if (rc != SGNN_OK) {
         sgnn_spmm_plan_destroy(p);
         return rc;
@@ -1555,6 +1611,11 @@ extern "C" int sgnn_spmm_plan_info(const sgnn_spmm_plan *p, int64_t info[10]) {
     info[0] = p->M; info[1] = p->K; info[2] = p->nnz; info[3] = p->n_long; info[4] = p->n_items;
     info[5] = p->long_edges; info[6] = p->long_thresh; info[7] = p->piece_edges;
     info[8] = p->partitioned ? 1 : 0; info[9] = (int64_t)(p->top_share * 1e6);
+    for (const sgnn_spmm_plan *part : p->parts) {  // row blocks: counts add up, the flags are those of any block
+        info[3] += part->n_long; info[4] += part->n_items; info[5] += part->long_edges;
+        info[8] |= part->partitioned ? 1 : 0;
+        info[9] = std::max<int64_t>(info[9], (int64_t)(part->top_share * 1e6));
+    }
     return SGNN_OK;
 }
 
@@ -1871,6 +1932,7 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
 extern "C" int sgnn_spmm_plan_schedule(const sgnn_spmm_plan *p, int64_t F, int64_t info[4]) {
     SGNN_REQUIRE(p != nullptr && info != nullptr, "null argument");
     SGNN_REQUIRE(F > 0 && F < (1 << 24), "feature width F=%lld out of range", (long long)F);
+    if (!p->parts.empty()) p = p->parts[0];  // row blocks decide one by one; the first one's answer is reported
     const BandShape sh = band_shape(p, F, true);
     info[0] = (band_wanted(p, F, sh) && p->cols_sorted != 0) ? 1 : 0;
     info[1] = sh.band_cols; info[2] = sh.n_bands; info[3] = sh.n_slices;
@@ -1887,6 +1949,20 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     SGNN_REQUIRE(ldo >= F, "leading dimension smaller than F (ldo=%lld F=%lld)", (long long)ldo, (long long)F);
     if (p->M == 0) return SGNN_OK;
     SGNN_REQUIRE(out != nullptr, "out is null");
+    if (!p->parts.empty()) {  // row blocks, one after the other on the caller's stream
+        for (size_t i = 0; i < p->parts.size(); ++i) {
+            sgnn_spmm_plan *part = p->parts[i];
+            DenseSrc d = dense;
+            if (d.eslot_csr != nullptr) {  // per-edge slot streams belong to the block
+                d.eslot_csr = part->eslot_csr;
+                d.eslot_long = part->eslot_long ? part->eslot_long : part->eslot_csr;
+            }
+            const int rc = spmm_run(part, val ? val + p->part_edge0[i] : nullptr, d, bits, out + p->part_row0[i] * ldo, F, ldo,
+                                    accumulate, row_div ? row_div + p->part_row0[i] : nullptr, st, scratch, scratch_floats);
+            if (rc != SGNN_OK) return rc;
+        }
+        return SGNN_OK;
+    }
     int dev = 0;
     SGNN_HIP_CHECK(hipGetDevice(&dev));
     SGNN_REQUIRE(dev == p->device, "plan was created on device %d, current device is %d", p->device, dev);
@@ -1969,6 +2045,11 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
 
 extern "C" int sgnn_spmm_plan_bind_values(sgnn_spmm_plan *p, const float *val, sgnn_stream_t stream) {
     SGNN_REQUIRE(p != nullptr, "plan is null");
+    for (size_t i = 0; i < p->parts.size(); ++i) {
+        const int rc = sgnn_spmm_plan_bind_values(p->parts[i], val ? val + p->part_edge0[i] : nullptr, stream);
+        if (rc != SGNN_OK) return rc;
+    }
+    if (!p->parts.empty()) return SGNN_OK;
     p->bound_val = nullptr;
     ++p->bind_gen;  // band schedules refill their value copies on their next use
     if (val == nullptr) return SGNN_OK;
@@ -1988,6 +2069,14 @@ extern "C" int sgnn_spmm_plan_bind_values(sgnn_spmm_plan *p, const float *val, s
 extern "C" int sgnn_spmm_plan_bind_row_slots(sgnn_spmm_plan *p, const int32_t *row_slot, sgnn_stream_t stream) {
     SGNN_REQUIRE(p != nullptr, "plan is null");
     p->bound_slots = nullptr;
+    for (sgnn_spmm_plan *part : p->parts) {
+        const int rc = sgnn_spmm_plan_bind_row_slots(part, row_slot, stream);
+        if (rc != SGNN_OK) return rc;
+    }
+    if (!p->parts.empty()) {
+        p->bound_slots = row_slot;
+        return SGNN_OK;
+    }
     if (row_slot == nullptr || p->nnz == 0) return SGNN_OK;
     hipStream_t st = (hipStream_t)stream;
     if (p->eslot_csr == nullptr) SGNN_HIP_CHECK(hipMalloc(&p->eslot_csr, sizeof(int32_t) * (size_t)p->nnz));
@@ -2045,8 +2134,14 @@ static int spmm_dq_impl(sgnn_spmm_plan *p, const float *val, const uint8_t *q, c
             const int rc = sgnn_spmm_plan_bind_row_slots(p, row_slot, stream);
             if (rc != SGNN_OK) return rc;
         }
-        d.eslot_csr = p->eslot_csr;
-        d.eslot_long = p->eslot_long ? p->eslot_long : p->eslot_csr;  // unregrouped long rows index the CSR arrays
+        if (!p->parts.empty()) {
+            // "slots are bound": spmm_run takes each row block's own streams
+            for (const sgnn_spmm_plan *part : p->parts)
+                if (part->eslot_csr != nullptr) { d.eslot_csr = d.eslot_long = part->eslot_csr; break; }
+        } else {
+            d.eslot_csr = p->eslot_csr;
+            d.eslot_long = p->eslot_long ? p->eslot_long : p->eslot_csr;  // unregrouped long rows index the CSR arrays
+        }
     }
     return spmm_run(p, val, d, bits, out, F, ldo, accumulate, row_div, (hipStream_t)stream);
 }
