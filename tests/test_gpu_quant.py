@@ -497,6 +497,39 @@ def test_v1_rows_with_gaps_and_illegal_widths(F):
         assert np.all(np.abs(back.cpu().numpy() - wantx) <= tol)
 
 
+@pytest.mark.parametrize("bits", [8, 4, 2])
+@pytest.mark.parametrize("F", [602, 123, 100, 128])
+def test_buffers_at_odd_addresses(bits, F):
+    """fp32 rows that start 4 bytes into an allocation and packed bytes that start 1 or 2 bytes into theirs (views
+    of larger buffers): every kernel choice must still write exactly the oracle's bytes, and only those."""
+    ops = _ops()
+    n = 1237
+    rng_ = np.random.default_rng(bits * 10 + F)
+    x = rng_.standard_normal((n, F)).astype(np.float32)
+    seg = [0, 400, 401, n]
+    q_ref, p_ref = orc.quant_rows(x, seg, bits)
+    npk = q_ref.shape[0]
+    for xoff, qoff in ((1, 1), (2, 2), (0, 3), (3, 0)):
+        xb = torch.zeros(n * F + 8, device="cuda")
+        xv = xb[xoff:xoff + n * F].view(n, F)
+        xv.copy_(torch.from_numpy(x))
+        qb = torch.full((npk * F + 8,), 0xCD, dtype=torch.uint8, device="cuda")
+        qv = qb[qoff:qoff + npk * F].view(npk, F)
+        prm = torch.zeros(n, 2, device="cuda")
+        ops.quantize_tensor_for_all_procs(xv, qv, prm, torch.tensor(seg, dtype=torch.int32), 3, bits)
+        got = qb.cpu().numpy()
+        assert np.array_equal(got[qoff:qoff + npk * F].reshape(npk, F), q_ref), (xoff, qoff)
+        assert (got[:qoff] == 0xCD).all() and (got[qoff + npk * F:] == 0xCD).all(), "bytes outside the packed rows were written"
+        assert np.array_equal(prm.cpu().numpy().view(np.uint32), p_ref.view(np.uint32))
+        ob = torch.full((n * F + 8,), 7.0, device="cuda")
+        ov = ob[xoff:xoff + n * F].view(n, F)
+        ops.dequantize_tensor_for_all_procs(qv, ov, prm, torch.tensor(seg, dtype=torch.int32), 3, bits)
+        d_ref = orc.dequant_rows(q_ref, p_ref, seg, bits, F)
+        o = ob.cpu().numpy()
+        assert np.all(np.abs(o[xoff:xoff + n * F].reshape(n, F) - d_ref) <= dequant_atol(p_ref[:, 0], p_ref[:, 1], bits)[:, None])
+        assert (o[:xoff] == 7.0).all() and (o[xoff + n * F:] == 7.0).all(), "floats outside the rows were written"
+
+
 def test_offsets_beyond_four_gigabytes():
     # 9 M x 128 fp32 = 4.6 GB: byte offsets of the last rows do not fit 32 bits.  Params against torch's
     # min/max, the round-trip bound everywhere, and the last rows of every segment bit-exact against the oracle.
