@@ -116,14 +116,17 @@ template <int VEC, int NV, int BITS>
 __device__ __forceinline__ void fma_row(float (&acc)[NV][VEC], float w, const Fetched<VEC, NV, BITS> &r) {
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
+        // all codes of the word moved to the bottom of their bytes with one shift and one mask; each then
+        // converts with a single byte-to-float instruction
+        uint32_t wm = 0;
+        if constexpr (BITS != 0) wm = (r.w[v] >> r.shift) & (((1u << (BITS & 15)) - 1u) * 0x01010101u);
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
             float xv;
             if constexpr (BITS == 0) {
                 xv = r.f[v][k];
             } else {
-                const uint32_t code = (r.w[v] >> (8 * k + r.shift)) & ((1u << (BITS & 15)) - 1u);
-                xv = fmaf((float)code, r.sc, r.zp);
+                xv = fmaf((float)((wm >> (8 * k)) & 0xffu), r.sc, r.zp);
             }
             acc[v][k] = fmaf(w, xv, acc[v][k]);
         }
