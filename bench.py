@@ -527,6 +527,35 @@ def wl_prepost(args, ctx):
             "roofline": roofline(wl, dom, k_fused[dom], dom_bytes, launches[dom]), "cpu_baseline": None, "extra": extra}
 
 
+def wl_quant_widths(args, ctx):
+    """Quantize+pack and unpack+dequantize over row widths (256 M floats each), all three code widths: kernel
+    times from the library's HIP-event profiler, rates by the algorithmic bytes.  A diagnostic sweep, not part
+    of the default run."""
+    import torch
+    from super_gnn_amd import synth, supergnn_ops as ops
+    widths = [int(w) for w in args.widths.split(",")]
+    table = {}
+    for F in widths:
+        n = 256_000_000 // F
+        x = synth.boundary_features(n, F, seed=5, device=ctx["dev"])
+        row = {}
+        for bits in (8, 4, 2):
+            c = quant_case(ops, x, bits, max(args.steps, 5), max(args.warmup, 2))
+            row[f"int{bits}"] = {"quant_us": round(c["quant_roofline"]["kernel_ms_per_step"] * 1e3, 1),
+                                 "quant_GBps": c["quant_roofline"]["gather_model"]["GBps"],
+                                 "dequant_us": round(c["dequant_roofline"]["kernel_ms_per_step"] * 1e3, 1),
+                                 "dequant_GBps": c["dequant_roofline"]["gather_model"]["GBps"]}
+        table[str(F)] = row
+        log(f"[bench] F={F:5d} rows={n:9d}  quantize+pack GB/s int8/4/2: " + " / ".join(f"{row[f'int{b}']['quant_GBps']:6.0f}" for b in (8, 4, 2)) +
+            "   unpack+dequantize GB/s: " + " / ".join(f"{row[f'int{b}']['dequant_GBps']:6.0f}" for b in (8, 4, 2)))
+        del x
+        torch.cuda.empty_cache()
+    worst = min(r["int2"]["quant_GBps"] for r in table.values())
+    return {"metric": "quantize-pack GB/s at int2, slowest row width of the sweep", "value": worst, "unit": "GB/s",
+            "config": {"workload": "quant_widths_256M_floats", "widths": widths}, "ms_per_step": 0.0, "dtype": "u8",
+            "roofline": None, "cpu_baseline": None, "extra": {"kernel_rates_by_width": table}}
+
+
 def wl_sbm(args, ctx):
     """Dense-degree community graph, wide odd feature rows (the band schedule)."""
     import torch
@@ -636,7 +665,7 @@ def wl_sage(args, ctx):
             "ms_per_step": ms, "dtype": "f32", "roofline": None, "cpu_baseline": None, "extra": {}}
 
 
-WORKLOADS = {"rmat": wl_rmat, "quant": wl_quant, "copy": wl_copy, "prepost": wl_prepost, "sbm": wl_sbm,
+WORKLOADS = {"rmat": wl_rmat, "quant": wl_quant, "quant_widths": wl_quant_widths, "copy": wl_copy, "prepost": wl_prepost, "sbm": wl_sbm,
              "aggregate": wl_aggregate, "sage": wl_sage, "small": wl_small}
 
 
@@ -678,6 +707,8 @@ def main():
     ap.add_argument("--quant-rows", type=int, default=1_000_000)
     ap.add_argument("--quant-feat", type=int, default=256)
     ap.add_argument("--bits", type=int, default=2)
+    ap.add_argument("--widths", default="32,64,100,123,128,200,256,300,500,600,602,640,1000,1024,1200,2050",
+                    help="quant_widths: row widths of the sweep")
     ap.add_argument("--long-threshold", type=int, default=0, help="SpMM plan: rows longer than this are split (0 = default)")
     ap.add_argument("--piece-edges", type=int, default=0, help="SpMM plan: minimum edges per long-row piece (0 = default)")
     ap.add_argument("--no-extras", action="store_true", help="only the chosen workload (used under rocprofv3)")
