@@ -125,7 +125,9 @@ __device__ __forceinline__ uint32_t quant_code(float x, float zp, float sc) {
 // Fused quantize + pack, row-group layout.  One group of G lanes handles kRowsPerGroup fp32 rows
 // (= 1 packed row at int2, 2 at int4, 4 at int8); G*VEC*NV >= F so a row lives in registers.
 // ------------------------------------------------------------------------------------------------
-template <int BITS, int VEC, int G, int NV, bool kForceExactDivision>
+// RAGGED (VEC == 4 only): any F and any 4-byte aligned row start -- 16-byte loads at their natural addresses, the
+// vector that reaches past the end of the row read and written element by element (see quant_pack_rows16_kernel).
+template <int BITS, int VEC, int G, int NV, bool kForceExactDivision, bool RAGGED = false>
 __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
     const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F,
@@ -168,8 +170,20 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
         if (!valid[r]) continue;
         const float *xr = row_ptr(xs, row[r]);
 #pragma unroll
-        for (int v = 0; v < NV; ++v)
-            if (act[v]) vec_load_nt<VEC>(xv[r][v], xr + off[v]);
+        for (int v = 0; v < NV; ++v) {
+            if (!act[v]) continue;
+            if constexpr (RAGGED) {
+                if (off[v] + VEC <= F) {
+                    vec4_load_nt_unaligned(xv[r][v], xr + off[v]);
+                } else {  // missing elements: copies of the first one (they change neither min nor max nor the first zero)
+                    xv[r][v][0] = xr[off[v]];
+#pragma unroll
+                    for (int k = 1; k < VEC; ++k) xv[r][v][k] = off[v] + k < F ? xr[off[v] + k] : xv[r][v][0];
+                }
+            } else {
+                vec_load_nt<VEC>(xv[r][v], xr + off[v]);
+            }
+        }
     }
 
     float zp[R], sc[R];
@@ -287,7 +301,18 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
         for (int v = 0; v < NV; ++v) {
             if (!act[v]) continue;
             const uint32_t word = words[pi][v];
-            if constexpr (VEC == 4) __builtin_nontemporal_store(word, reinterpret_cast<uint32_t *>(qr + off[v]));
+            if constexpr (RAGGED) {
+                uint8_t *dst = qr + off[v];
+                const uintptr_t al = reinterpret_cast<uintptr_t>(dst) & 3;
+                if (off[v] + VEC <= F && al == 0) {
+                    __builtin_nontemporal_store(word, reinterpret_cast<uint32_t *>(dst));
+                } else if (off[v] + VEC <= F && al == 2) {
+                    __builtin_nontemporal_store((uint16_t)word, reinterpret_cast<uint16_t *>(dst));
+                    __builtin_nontemporal_store((uint16_t)(word >> 16), reinterpret_cast<uint16_t *>(dst) + 1);
+                } else {
+                    for (int k = 0; k < VEC && off[v] + k < F; ++k) dst[k] = (uint8_t)(word >> (8 * k));
+                }
+            } else if constexpr (VEC == 4) __builtin_nontemporal_store(word, reinterpret_cast<uint32_t *>(qr + off[v]));
             else if constexpr (VEC == 2) __builtin_nontemporal_store((uint16_t)word, reinterpret_cast<uint16_t *>(qr + off[v]));
             else qr[off[v]] = (uint8_t)word;
         }
@@ -1459,6 +1484,26 @@ static void launch_quant16_ragged(const RowsArgs &a, hipStream_t st) {
                            a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
+// The same for rows of 1025 ... 2560 floats: a wavefront holds four rows in registers, NV vectors per lane each.
+template <int BITS, int NV>
+static void launch_rows_ragged(const RowsArgs &a, hipStream_t st) {
+    constexpr int NPR = kRowsPerGroup / (8 / BITS);
+    constexpr int GPB = kQBlock / 64;
+    const int n_units = (a.n_packed + NPR - 1) / NPR;
+    const int nb = (n_units + GPB - 1) / GPB;
+    ProfScope prof(K_QUANT_PACK_ROWS, st);
+    hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, 4, 64, NV, false, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
+                       a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
+}
+template <int BITS>
+static void dispatch_rows_ragged_wide(const RowsArgs &a, hipStream_t st) {
+    const int nvec = (a.F + 3) / 4;
+    if (nvec <= 320) return launch_rows_ragged<BITS, 5>(a, st);
+    if (nvec <= 384) return launch_rows_ragged<BITS, 6>(a, st);
+    if (nvec <= 512) return launch_rows_ragged<BITS, 8>(a, st);
+    return launch_rows_ragged<BITS, 10>(a, st);
+}
+
 // Widths or row starts that are not a multiple of four floats, up to 1024 floats per row.
 template <int BITS>
 static void dispatch_quant16_ragged(const RowsArgs &a, hipStream_t st) {
@@ -1581,6 +1626,12 @@ static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
     if constexpr (VEC == 4) {
         if (nvec <= 192) return launch_rows<BITS, VEC, 64, 3>(a, st);
         if (nvec <= 256) return launch_rows<BITS, VEC, 64, 4>(a, st);
+        if (a.quantize) {  // rows of up to 2048 floats still fit a wavefront's registers (four rows, NV vectors per lane each)
+            if (nvec <= 320) return launch_rows<BITS, VEC, 64, 5>(a, st);
+            if (nvec <= 384) return launch_rows<BITS, VEC, 64, 6>(a, st);
+            if (nvec <= 512) return launch_rows<BITS, VEC, 64, 8>(a, st);
+            if (nvec <= 640) return launch_rows<BITS, VEC, 64, 10>(a, st);
+        }
     } else {
         if (nvec <= 256) return launch_rows<BITS, VEC, 64, 4>(a, st);
         if (nvec <= 512) return launch_rows<BITS, VEC, 64, 8>(a, st);
@@ -1629,6 +1680,10 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
         if (bits == 8) dispatch_quant16_ragged<8>(a, st);
         else if (bits == 4) dispatch_quant16_ragged<4>(a, st);
         else dispatch_quant16_ragged<2>(a, st);
+    } else if (a.quantize && vec != 4 && !a.exact_division && a.F <= 2560) {
+        if (bits == 8) dispatch_rows_ragged_wide<8>(a, st);
+        else if (bits == 4) dispatch_rows_ragged_wide<4>(a, st);
+        else dispatch_rows_ragged_wide<2>(a, st);
     } else if (bits == 8) dispatch_rows<8>(vec, a, st);
     else if (bits == 4) dispatch_rows<4>(vec, a, st);
     else dispatch_rows<2>(vec, a, st);
