@@ -519,7 +519,8 @@ def wl_prepost(args, ctx):
              "local_GEdges_per_s": round(nl / ms_local / 1e6, 3),
              "local_kernel_ms_per_step": {k: round(v, 5) for k, v in k_local.items()},
              "fused_kernel_ms_per_step": {k: round(v, 5) for k, v in k_fused.items()},
-             "fused_step_roofline": step_roofline(wl, k_fused)}
+             "fused_step_roofline": step_roofline(wl, k_fused),
+             "local_step_roofline": step_roofline(wl, {k + "(local)": v for k, v in k_local.items()})}
     log(f"[bench] prepost: local SpMM {ms_local:.3f} ms; remote: separate {ms_sep:.3f} ms vs fused {ms_fused:.3f} ms")
     return {"metric": "SpMM GEdges/s, pre/post-aggregation partition (local fp32 + int2-packed remote rows, fused)",
             "value": round((nl + nr) / total / 1e6, 4), "unit": "GEdges/s",

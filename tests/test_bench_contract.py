@@ -30,7 +30,9 @@ def test_measured_traffic_of_every_default_workload_is_tracked():
             ("quant_pack_int2_1000000x256", "quant_pack_rows_kernel"), ("unpack_dequant_int2_1000000x256", "unpack_dequant_rows_kernel"),
             ("quant_pack_int2_2000000x128", "quant_pack_rows_kernel"), ("quant_pack_int2_4000000x64", "quant_pack_rows_kernel"),
             ("quant_pack_int2_425000x602", "quant_pack_rows_kernel"), ("unpack_dequant_int2_425000x602", "unpack_dequant_rows_kernel"),
-            ("prepost_8000000n_160000000ue_local_2000000c_80000000e_remote_int2_F128", "spmm_piece_kernel(dq)")]
+            ("prepost_8000000n_160000000ue_local_2000000c_80000000e_remote_int2_F128", "spmm_piece_kernel(dq)"),
+            ("prepost_8000000n_160000000ue_local_2000000c_80000000e_remote_int2_F128", "spmm_piece_kernel(local)"),
+            ("prepost_8000000n_160000000ue_local_2000000c_80000000e_remote_int2_F128", "spmm_short_kernel(local)")]
     for key in want:
         t = b.TRAFFIC.get(key)
         assert t is not None, f"no traffic line for {key} under profiles/"
