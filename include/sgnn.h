@@ -243,7 +243,10 @@ int sgnn_spmm_csr_dq_wire_f32(sgnn_spmm_plan *plan, const float *val, const uint
 /* params f32[n,3] = (bits, zero_point, scale): bits is read, zero_point/scale are written.
  * range i64[n+1]: row i's bytes are q[range[i] .. range[i+1]).  The table is trusted, as in the reference:
  * range[i+1] - range[i] must be at least ceil(F * bits_i / 8), or a row's bytes spill into the next row's
- * (the Python layer checks this once per (params, range) pair).
+ * (the Python layer checks this once per (params, range) pair).  Rows may lie anywhere in q; where the ranges
+ * of consecutive rows follow one another without gaps (range[i+1] - range[i] == ceil(F * bits_i / 8), the
+ * layout the reference builds) the bytes of several rows leave the GPU as one run of stores.  A row whose bits
+ * is not 8, 4 or 2 is left untouched (the reference prints an error and skips it, quantization_x86.cpp:244-245).
  * Replaces quantize_tensor_v1 (super_gnn/ops/csrc/quantization_arm.cpp:635-702). */
 int sgnn_quant_v1_f32(const float *x, uint8_t *q, const int64_t *range, float *params, int64_t n,
                       int64_t F, sgnn_stream_t stream);
