@@ -588,6 +588,30 @@ def wl_sbm(args, ctx):
              "compulsory_bytes": int(spmm_compulsory_bytes(nnz, n, n, F, False)), "step_roofline": step_roofline(wl, per_kernel)}
     log(f"[bench] sbm sum: {ms:.3f} ms/step, {nnz / ms / 1e6:.2f} GEdges/s, schedule {sched}, kernels (ms per step) "
         f"{ {k: round(v, 4) for k, v in per_kernel.items()} }")
+    if args.sbm_packed and F % 2 == 0:
+        # the same product with every dense row arriving packed (one segment): dequantize-then-multiply against
+        # the fused unpack+dequantize+SpMM, which takes two-code lanes when F % 4 != 0
+        seg = torch.tensor([0, n], dtype=torch.int32)
+        recv = torch.empty(n, F, device=dev)
+        fused = {}
+        for bits in (8, 4, 2):
+            epb = 8 // bits
+            q = torch.empty((n + epb - 1) // epb, F, dtype=torch.uint8, device=dev)
+            prm = torch.empty(n, 2, device=dev)
+            ops.quantize_tensor_for_all_procs(x, q, prm, seg, 1, bits)
+            segs = ops.quant_segments(seg, bits)
+
+            def separate():
+                ops.dequantize_tensor_for_all_procs(q, recv, prm, seg, 1, bits)
+                plan.run(None, recv, out, accumulate=True)
+
+            ms_sep = time_steps(separate, min(args.steps, 5), 2)
+            ms_f, k_f, _ = profiled_steps(lambda: plan.run_quantized(None, q, prm, segs, bits, out, accumulate=True), min(args.steps, 5), 2)
+            fused[f"int{bits}"] = {"separate_ms": round(ms_sep, 3), "fused_ms": round(ms_f, 3),
+                                   "fused_kernel_ms_per_step": {k: round(v, 4) for k, v in k_f.items()}}
+            log(f"[bench] sbm, dense rows packed at int{bits}: dequantize + product {ms_sep:.2f} ms, fused {ms_f:.2f} ms")
+            del q, prm
+        extra["packed_operand"] = fused
     return {"metric": f"SpMM GEdges/s (dense-degree community graph, F={F} fp32)", "value": round(nnz / ms / 1e6, 4),
             "unit": "GEdges/s", "config": {"workload": wl, "F": F}, "ms_per_step": ms, "dtype": "f32",
             "roofline": roofline(wl, dom, per_kernel[dom], dom_bytes, launches[dom]), "cpu_baseline": None, "extra": extra}
@@ -697,6 +721,8 @@ def main():
     ap.add_argument("--sbm-blocks", type=int, default=50)
     ap.add_argument("--sbm-pin", type=float, default=0.03048, help="sbm: edge probability inside a block (20x the one between blocks)")
     ap.add_argument("--sbm-feat", type=int, default=602)
+    ap.add_argument("--sbm-packed", action="store_true", help="sbm: also time the product with the dense rows arriving int8/4/2-packed "
+                    "(dequantize-then-multiply against the fused kernel)")
     ap.add_argument("--hidden", type=int, default=256, help="sage: hidden width")
     ap.add_argument("--classes", type=int, default=47, help="sage: output classes")
     ap.add_argument("--parts", type=int, default=8, help="aggregate: number of vertex partitions simulated in this process")

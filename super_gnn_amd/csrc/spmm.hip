@@ -1168,6 +1168,18 @@ static int dispatch_shape(int nvec, const ShortArgs &a, const PieceArgs &s, cons
     return SGNN_OK;
 }
 
+// Lane slots (of VEC codes each) the fused kernels' lane-group shape for a row of nvec vectors holds: the shapes
+// instantiated in dispatch_shape_dq.
+static int dq_slots(int vec, int nvec) {
+    if (nvec <= 8) return 8;
+    if (nvec <= 16) return 16;
+    if (nvec <= 32) return 32;
+    if (nvec <= 64) return 64;
+    if (nvec <= 128) return 128;
+    if (vec == 2) return nvec <= 320 ? 320 : (nvec + 511) / 512 * 512;
+    return nvec <= 256 ? 256 : (nvec + 511) / 512 * 512;
+}
+
 // Quantized dense operand: one packed word of VEC codes per lane and vector.  VEC = 4 when F % 4 == 0,
 // VEC = 2 for the other even widths (F = 602: 301 two-float lanes slots, five per lane).
 template <int BITS>
@@ -1994,6 +2006,10 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     int vec = 1;
     if (bits != 0) {
         vec = F % 4 == 0 ? 4 : 2;  // checked by the caller: F even, 4-byte aligned packed buffer
+        // With a dense-degree matrix the fused kernels are bound by instruction issue (two fmas and a conversion
+        // per element), so idle lane slots cost time: F = 600 fills 150 of the 256 four-code slots of its lane-group
+        // shape but 300 of the 320 two-code slots (measured on the 114 M-edge community graph: 11.7 -> 10.5 ms).
+        if (vec == 4 && dq_slots(2, (int)(F / 2)) * 2 < dq_slots(4, (int)(F / 4)) * 4 * 0.8) vec = 2;
         SGNN_REQUIRE(ldo % vec == 0 && aligned(out, 4 * vec),
                      "the fused path at F=%lld needs out %d-byte aligned with ldo %% %d == 0", (long long)F, 4 * vec, vec);
     } else if (F % 4 == 0 && dense.ldx % 4 == 0 && ldo % 4 == 0 && aligned(dense.x, 16) && aligned(out, 16)) {
