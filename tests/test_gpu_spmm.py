@@ -327,22 +327,28 @@ def test_bound_values_follow_in_place_changes():
     assert torch.equal(o2, o)
 
 
-def test_steady_state_calls_replay_from_a_captured_graph():
+@pytest.mark.parametrize("F,row_blocks", [(128, False), (602, False), (100, True)])
+def test_steady_state_calls_replay_from_a_captured_graph(F, row_blocks, monkeypatch):
     """After warm-up a call only launches kernels (no allocation, no synchronisation), so an
     SpMM + quantize + fused-SpMM sequence can be captured once and replayed; every replay, with eager
-    work in between, must reproduce the eager result bit for bit."""
+    work in between, must reproduce the eager result bit for bit.  F = 602: rows on 8-byte boundaries (unaligned
+    vector loads, packed bytes staged through LDS, two-code lanes in the fused product); row_blocks: the plan
+    held as several row blocks."""
     ops = _gpu()
     dev = torch.device("cuda:0")
     rowptr, col, val = random_csr(4000, 3000, 9, seed=5, empty_frac=0.2, hubs=8, hub_deg=1200)
     gen = torch.Generator().manual_seed(0)
-    x = torch.randn(3000, 128, generator=gen).to(dev)
+    x = torch.randn(3000, F, generator=gen).to(dev)
+    if row_blocks:
+        monkeypatch.setenv("SGNN_SPMM_PART_EDGES", str(int(rowptr[-1]) // 3))
     plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), 3000)
+    monkeypatch.delenv("SGNN_SPMM_PART_EDGES", raising=False)
     v = torch.from_numpy(val).to(dev)
     seg = torch.tensor([0, 1001, 2003, 3000], dtype=torch.int32)
     segs = ops.quant_segments(seg, 4)
-    q = torch.zeros(segs.n_packed, 128, dtype=torch.uint8, device=dev)
+    q = torch.zeros(segs.n_packed, F, dtype=torch.uint8, device=dev)
     prm = torch.zeros(3000, 2, device=dev)
-    out, out_q = torch.zeros(4000, 128, device=dev), torch.zeros(4000, 128, device=dev)
+    out, out_q = torch.zeros(4000, F, device=dev), torch.zeros(4000, F, device=dev)
 
     def step():
         out.zero_(); out_q.zero_()
