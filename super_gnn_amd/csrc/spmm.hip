@@ -1302,6 +1302,10 @@ struct sgnn_spmm_plan {
     // edges than that (the kernels' edge offsets are 32-bit); every call on the whole runs the blocks in turn.
     std::vector<sgnn_spmm_plan *> parts;
     std::vector<int64_t> part_row0, part_edge0;
+    sgnn_spmm_plan *whole = nullptr;   // a row block: the plan it belongs to, which owns the restaged-operand workspace
+    uint64_t call_serial = 0;          // products run on this (whole) plan so far
+    uint64_t xs_serial = 0;            // the product whose dense operand band_xs holds ...
+    int xs_F = 0, xs_slice_pad = 0, xs_slices = 0;  // ... and in which slice layout
     // Short-row chunks, one list per chunk row limit (7, 15, 31).
     std::vector<int64_t> h_rowptr;
     int4 *chunks[3] = {nullptr, nullptr, nullptr};
@@ -1587,6 +1591,7 @@ static int plan_create_parts(sgnn_spmm_plan *p, const int64_t *rowptr, const voi
         p->parts.push_back(part);  // owned from here on: destroyed with the whole
         p->part_row0.push_back(r0);
         p->part_edge0.push_back(h[r0]);
+        part->whole = p;
         part->M = r1 - r0; part->K = p->K; part->nnz = h[r1] - h[r0];
         part->long_thresh = p->long_thresh; part->piece_edges = p->piece_edges;
         rc = plan_create_impl(part, d_rp.p, (const char *)col + (size_t)h[r0] * col_bytes, col_is_i64, st);
@@ -1873,8 +1878,11 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
     BandSchedule *bs = nullptr;
     for (BandSchedule *c : p->bands)
         if (c->band_cols == sh.band_cols) bs = c;
+    // The restaged operand lives in the plan the caller holds: the row blocks of a large matrix share one copy,
+    // restaged by the first block of a product that takes the band schedule.
+    sgnn_spmm_plan *root = p->whole ? p->whole : p;
     const size_t xs_floats = (size_t)sh.n_slices * (size_t)p->K * (size_t)sh.slice_pad;
-    if (bs == nullptr || xs_floats > p->band_xs_floats) {
+    if (bs == nullptr || xs_floats > root->band_xs_floats) {
         if (!may_build) return SGNN_OK;
         bool sorted = false;
         int rc = band_rows_sorted(p, st, &sorted);
@@ -1884,13 +1892,14 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
             if ((rc = band_build(p, sh.band_cols, sh.n_bands, st, &bs)) != SGNN_OK) return rc;
             p->bands.push_back(bs);
         }
-        if (xs_floats > p->band_xs_floats) {
+        if (xs_floats > root->band_xs_floats) {
             SGNN_HIP_CHECK(hipDeviceSynchronize());  // the old workspace may still be read by queued work
-            (void)hipFree(p->band_xs);
-            p->band_xs = nullptr;
-            p->band_xs_floats = 0;
-            SGNN_HIP_CHECK(hipMalloc(&p->band_xs, xs_floats * sizeof(float)));
-            p->band_xs_floats = xs_floats;
+            (void)hipFree(root->band_xs);
+            root->band_xs = nullptr;
+            root->band_xs_floats = 0;
+            root->xs_serial = 0;
+            SGNN_HIP_CHECK(hipMalloc(&root->band_xs, xs_floats * sizeof(float)));
+            root->band_xs_floats = xs_floats;
         }
     }
     const BandCaps caps = band_chunk_caps(p, sh, val != nullptr);
@@ -1913,11 +1922,14 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
         val_bm = bs->val_bm;
     }
     const int iF = (int)F;
-    {
+    if (p->whole == nullptr) ++root->call_serial;  // (a plan of row blocks counts its products in spmm_run)
+    if (!(root->xs_serial == root->call_serial && root->xs_F == iF && root->xs_slice_pad == sh.slice_pad && root->xs_slices == sh.n_slices)) {
         ProfScope prof(K_SPMM_BAND_RESTAGE, st);
         const int64_t n = (int64_t)sh.n_slices * p->K * (sh.slice_pad / 4);
         hipLaunchKernelGGL(band_restage_kernel, dim3((uint32_t)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, dense.x, dense.ldx,
-                           p->band_xs, p->K, iF, sh.slice_floats, sh.slice_pad, sh.n_slices);
+                           root->band_xs, p->K, iF, sh.slice_floats, sh.slice_pad, sh.n_slices);
+        root->xs_serial = root->call_serial;
+        root->xs_F = iF; root->xs_slice_pad = sh.slice_pad; root->xs_slices = sh.n_slices;
     }
     const int ev = sh.even ? 2 : 1;  // vector width of the fill / divide passes
     if (!accumulate) {
@@ -1928,10 +1940,10 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
         ProfScope prof(K_SPMM_BAND, st);
         for (int b = 0; b < bs->n_bands; ++b) {
             int rc;
-            if (val_bm) rc = sh.even ? launch_band<true, true>(bs, cl, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device)
-                                     : launch_band<false, true>(bs, cl, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device);
-            else rc = sh.even ? launch_band<true, false>(bs, cl, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device)
-                              : launch_band<false, false>(bs, cl, sh, b, val_bm, p->band_xs, out, iF, ldo, st, p->device);
+            if (val_bm) rc = sh.even ? launch_band<true, true>(bs, cl, sh, b, val_bm, root->band_xs, out, iF, ldo, st, p->device)
+                                     : launch_band<false, true>(bs, cl, sh, b, val_bm, root->band_xs, out, iF, ldo, st, p->device);
+            else rc = sh.even ? launch_band<true, false>(bs, cl, sh, b, val_bm, root->band_xs, out, iF, ldo, st, p->device)
+                              : launch_band<false, false>(bs, cl, sh, b, val_bm, root->band_xs, out, iF, ldo, st, p->device);
             if (rc != SGNN_OK) return rc;
         }
     }
@@ -1965,6 +1977,7 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     if (p->M == 0) return SGNN_OK;
     SGNN_REQUIRE(out != nullptr, "out is null");
     if (!p->parts.empty()) {  // row blocks, one after the other on the caller's stream
+        ++p->call_serial;     // one product: the blocks that take the band schedule share one restaged operand
         for (size_t i = 0; i < p->parts.size(); ++i) {
             sgnn_spmm_plan *part = p->parts[i];
             DenseSrc d = dense;

@@ -68,6 +68,34 @@ def test_row_blocks_equal_the_single_plan(case, monkeypatch):
         assert torch.equal(a, b)
 
 
+def test_row_blocks_share_one_restaged_operand(monkeypatch):
+    """With the band schedule every block of a plan gathers from the same restaged copy of the dense operand: it is
+    made once per product and held once, however many blocks there are (64 blocks of a 60 MB operand would
+    otherwise hold 3.8 GB)."""
+    M, K, F = 6000, 30000, 512
+    rowptr, col, val = random_csr(M, K, 40, seed=77)
+    monkeypatch.setenv("SGNN_SPMM_BAND", "1")
+    ops, whole, blocked = _plans(monkeypatch, rowptr, col, K, int(rowptr[-1]) // 64 + 1)
+    assert whole.schedule(F)["band"] == 1
+    x = torch.randn(K, F, generator=torch.Generator().manual_seed(3)).cuda()
+    init = torch.randn(M, F, generator=torch.Generator().manual_seed(4)).cuda()
+    v = torch.from_numpy(val).cuda()
+    a = init.clone()
+    whole.run(v, x, a)
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    b = init.clone()
+    blocked.run(v, x, b)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert torch.equal(a, b)
+    assert free0 - free1 < 4 * K * F * 4, f"the blocked plan took {(free0 - free1) >> 20} MB for its first product"
+    x2 = x * 2.0                              # a new operand must be restaged, not taken from the last product
+    a2, b2 = init.clone(), init.clone()
+    whole.run(v, x2, a2); blocked.run(v, x2, b2)
+    assert torch.equal(a2, b2) and not torch.equal(a2, a)
+
+
 def test_a_row_longer_than_a_block_is_refused(monkeypatch):
     from super_gnn_amd import supergnn_ops as ops
     rowptr, col, _ = random_csr(100, 400, 3, seed=1, hubs=1, hub_deg=300)
