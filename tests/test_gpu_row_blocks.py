@@ -96,6 +96,44 @@ def test_row_blocks_share_one_restaged_operand(monkeypatch):
     assert torch.equal(a2, b2) and not torch.equal(a2, a)
 
 
+def test_plans_release_their_memory(monkeypatch):
+    """Everything a plan allocates -- work lists, regrouped long rows, bound values and slot streams, the band
+    schedule and its restaged operand, the row blocks -- goes back when the plan is destroyed."""
+    import gc
+    from super_gnn_amd import supergnn_ops as ops
+    M, K, F = 5000, 20000, 256
+    rowptr, col, val = random_csr(M, K, 30, seed=5, hubs=6, hub_deg=3000)
+    rp, cl, v = torch.from_numpy(rowptr).cuda(), torch.from_numpy(col).cuda(), torch.from_numpy(val).cuda()
+    x = torch.randn(K, F, generator=torch.Generator().manual_seed(1)).cuda()
+    out = torch.zeros(M, F, device="cuda")
+    seg = torch.tensor([0, 7001, K], dtype=torch.int32)
+    segs = ops.quant_segments(seg, 2)
+    q = torch.zeros(segs.n_packed, F, dtype=torch.uint8, device="cuda"); prm = torch.zeros(K, 2, device="cuda")
+    ops.quantize_tensor_for_all_procs(x, q, prm, seg, 2, 2)
+
+    def cycle(blocks, band):
+        monkeypatch.setenv("SGNN_SPMM_BAND", "1" if band else "0")
+        if blocks:
+            monkeypatch.setenv("SGNN_SPMM_PART_EDGES", str(int(rowptr[-1]) // 5))
+        plan = ops.SpmmPlan(rp, cl, K)
+        monkeypatch.delenv("SGNN_SPMM_PART_EDGES", raising=False)
+        for _ in range(2):
+            plan.run(v, x, out)
+            plan.run_quantized(v, q, prm, segs, 2, out)
+        torch.cuda.synchronize()
+        del plan
+        gc.collect()
+
+    cycle(True, True)                       # first use of every kernel: code objects, event pools
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for i in range(12):
+        cycle(i % 2 == 0, i % 3 != 0)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free0 - free1 < 8 << 20, f"{(free0 - free1) >> 20} MB not returned after 12 plans"
+
+
 def test_a_row_longer_than_a_block_is_refused(monkeypatch):
     from super_gnn_amd import supergnn_ops as ops
     rowptr, col, _ = random_csr(100, 400, 3, seed=1, hubs=1, hub_deg=300)
