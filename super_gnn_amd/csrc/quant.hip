@@ -760,6 +760,36 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_ragged_kernel(
             row = (int)(e0 / F);
             c = (int)(e0 - (int64_t)row * F);
         }
+        // When no vector of the wavefront straddles a row boundary -- most wavefronts of a wide row -- a lane's two
+        // pieces share row, slot and params, and one 4-byte load at the bytes' natural address fetches both.
+        const bool whole = c + 4 <= F;
+        if (VEC == 2 && __ballot(i < n_vec && !whole) == 0ull) {
+            word[u][0] = word[u][NP - 1] = 0;
+            ps[u][0] = ps[u][NP - 1] = make_float2(0.0f, 0.0f);
+            shift[u][0] = shift[u][NP - 1] = 0;
+            if (i < n_vec) {
+                int slot = row;
+                if constexpr (SEGMENTED) {
+                    if (row < w_s1) {
+                        slot = w_ps0 * EPB + (row - w_s0);
+                    } else {
+                        int lo = w_p, hi = P - 1;
+                        while (lo < hi) {
+                            const int mid = (lo + hi) >> 1;
+                            if (seg[mid + 1] > row) hi = mid; else lo = mid + 1;
+                        }
+                        slot = pseg[lo] * EPB + (row - seg[lo]);
+                    }
+                }
+                typedef uint32_t u32u __attribute__((aligned(2)));
+                const uint32_t w = *reinterpret_cast<const u32u *>(q + (int64_t)(slot / EPB) * F + c);
+                word[u][0] = w & 0xffffu;
+                word[u][NP - 1] = w >> 16;
+                ps[u][0] = ps[u][NP - 1] = load_params(pb, row);
+                shift[u][0] = shift[u][NP - 1] = (EPB - 1 - (slot % EPB)) * BITS;
+            }
+            continue;
+        }
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             word[u][p] = 0;
@@ -804,6 +834,89 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_ragged_kernel(
         } else {
             for (int e = 0; e < 4; ++e)
                 if (i * 4 + e < n_elem) x[i * 4 + e] = o[e];
+        }
+    }
+}
+
+// Odd F >= 4: the four floats of a 16-byte vector lie in at most two rows, A (the first n_a of them) and the
+// row after it, so a lane looks up two rows (slot, params) instead of four and fetches its four code bytes from
+// the one or two places they sit in.
+template <int BITS, int R, bool SEGMENTED>
+__global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_odd_kernel(
+    const uint8_t *__restrict__ q, float *__restrict__ x, const ParamBuf pb, const int32_t *__restrict__ seg,
+    const int32_t *__restrict__ pseg, int P, int F, int n_rows, int64_t n_elem) {
+    constexpr int EPB = 8 / BITS;
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (kQBlock / 64) + (threadIdx.x >> 6);
+    const int64_t base = wave * (R * 64) + lane;
+    const int64_t n_vec = (n_elem + 3) >> 2;
+    auto slot_of = [&](int row) {
+        if constexpr (!SEGMENTED) return row;
+        int lo = 0, hi = P - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (seg[mid + 1] > row) hi = mid; else lo = mid + 1;
+        }
+        return pseg[lo] * EPB + (row - seg[lo]);
+    };
+    uint32_t code[R][4];
+    float2 psa[R], psb[R];
+    int na[R];
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const int64_t i = base + u * 64;
+        na[u] = 0;
+        psa[u] = psb[u] = make_float2(0.0f, 0.0f);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) code[u][k] = 0;
+        if (i >= n_vec) continue;
+        const int64_t e0 = i * 4;
+        const int row_a = (int)(e0 / F);
+        const int c_a = (int)(e0 - (int64_t)row_a * F);
+        na[u] = F - c_a < 4 ? F - c_a : 4;
+        const bool has_b = na[u] < 4 && row_a + 1 < n_rows;
+        const bool wave_whole = __ballot(na[u] != 4) == 0ull;   // every active lane's vector lies inside one row
+        const int slot_a = slot_of(row_a);
+        psa[u] = load_params(pb, row_a);
+        const uint8_t *src_a = q + (int64_t)(slot_a / EPB) * F + c_a;
+        const int shift_a = (EPB - 1 - (slot_a % EPB)) * BITS;
+        const uint8_t *src_b = src_a;
+        int shift_b = 0;
+        if (has_b) {
+            const int slot_b = slot_of(row_a + 1);
+            psb[u] = load_params(pb, row_a + 1);
+            src_b = q + (int64_t)(slot_b / EPB) * F - na[u];   // piece k of row B is its column k - n_a
+            shift_b = (EPB - 1 - (slot_b % EPB)) * BITS;
+        }
+        if (wave_whole) {   // one 4-byte load at the bytes' natural address
+            typedef uint32_t u32u __attribute__((aligned(1)));
+            const uint32_t w = *reinterpret_cast<const u32u *>(src_a);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) code[u][k] = (w >> (8 * k + shift_a)) & MASK;
+            continue;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const bool in_a = k < na[u];
+            if (in_a || has_b) code[u][k] = ((in_a ? src_a : src_b)[k] >> (in_a ? shift_a : shift_b)) & MASK;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {
+        const int64_t i = base + u * 64;
+        if (i >= n_vec) continue;
+        float o[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float2 ps = k < na[u] ? psa[u] : psb[u];
+            o[k] = fmaf((float)code[u][k], ps.y, ps.x);
+        }
+        if (i * 4 + 4 <= n_elem) {
+            vec_store_nt<4>(x + i * 4, o);
+        } else {
+            for (int k = 0; k < 4; ++k)
+                if (i * 4 + k < n_elem) x[i * 4 + k] = o[k];
         }
     }
 }
@@ -1580,6 +1693,17 @@ static void launch_dequant_flat_ragged(const RowsArgs &a, int64_t n_rows, hipStr
     const int64_t n_waves = (n_vec + R * 64 - 1) / (R * 64);
     const unsigned nb = (unsigned)((n_waves + kQBlock / 64 - 1) / (kQBlock / 64));
     ProfScope prof(K_UNPACK_DEQUANT_ROWS, st);
+    const char *odd2 = getenv("SGNN_DEQUANT_ODD2");
+    const bool two_rows = !(odd2 && odd2[0] == '0');
+    if (VEC == 1 && a.F >= 4 && two_rows) {
+        if (BITS != 8 && a.P > 1)
+            hipLaunchKernelGGL((unpack_dequant_flat_odd_kernel<BITS, R, true>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, a.x_out,
+                               a.params, a.seg, a.pseg, a.P, a.F, (int)n_rows, n_elem);
+        else
+            hipLaunchKernelGGL((unpack_dequant_flat_odd_kernel<BITS, R, false>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, a.x_out,
+                               a.params, a.seg, a.pseg, a.P, a.F, (int)n_rows, n_elem);
+        return;
+    }
     if (BITS != 8 && a.P > 1)
         hipLaunchKernelGGL((unpack_dequant_flat_ragged_kernel<BITS, VEC, R, true>), dim3(nb), dim3(kQBlock), 0, st, a.q_in,
                            a.x_out, a.params, a.seg, a.pseg, a.P, a.F, n_elem);

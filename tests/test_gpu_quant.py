@@ -376,10 +376,11 @@ def test_bf16_params_equal_torch_casts(bits, F):
 
 
 @pytest.mark.parametrize("bits", [8, 4, 2])
-@pytest.mark.parametrize("F", [4, 64, 100, 128, 256, 600, 1028, 2052, 602, 123, 6, 3, 1, 2050])
+@pytest.mark.parametrize("F", [4, 64, 100, 128, 256, 600, 1028, 2052, 602, 123, 6, 3, 1, 2050, 5, 301, 1433])
 def test_flat_and_row_tiled_dequantizers_agree(bits, F, monkeypatch):
-    """The flat-output kernel (default) and the row-tiled kernels are two decompositions of the same
-    arithmetic: same bits out, ragged multi-segment tables included."""
+    """The flat-output kernels (default; at odd widths also the general one that the two-row kernel
+    replaces) and the row-tiled kernels are decompositions of the same arithmetic: same bits out,
+    ragged multi-segment tables included."""
     from super_gnn_amd import supergnn_ops as ops
     gen = torch.Generator().manual_seed(bits * 7 + F)
     n = 3001
@@ -391,12 +392,13 @@ def test_flat_and_row_tiled_dequantizers_agree(bits, F, monkeypatch):
         q = torch.zeros((npk, F), dtype=torch.uint8, device="cuda"); prm = torch.zeros((n, 2), device="cuda")
         ops.quantize_tensor_for_all_procs(x, q, prm, wr_t, P, bits)
         outs = []
-        for flat in ("1", "0"):
+        for flat, odd2 in (("1", "1"), ("0", "1"), ("1", "0")):
             monkeypatch.setenv("SGNN_DEQUANT_FLAT", flat)
+            monkeypatch.setenv("SGNN_DEQUANT_ODD2", odd2)
             o = torch.full((n, F), 7.0, device="cuda")
             ops.dequantize_tensor_for_all_procs(q, o, prm, wr_t, P, bits)
             outs.append(o)
-        assert torch.equal(outs[0], outs[1])
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
 
 
 def test_cpu_runnable_configuration_int8_boundary_rows():
