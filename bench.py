@@ -405,6 +405,20 @@ def wl_rmat(args, ctx):
         extra["spmm_cache_flushed"] = time_reps_events(step, 20, 2, flush=lambda: scratch.fill_(1.0))
         log(f"[bench] weighted sum per repetition: warm {extra['spmm_warm']}, caches flushed before each {extra['spmm_cache_flushed']}")
         del scratch
+        if not args.uniform_rows and F == 128:
+            # the hidden width of the reference's GraphSAGE layers (examples/graphsage/sage.py: hidden 256): products
+            # from 256 columns up run as feature slices; SGNN_SPMM_SLICE=0 is the same product in one piece
+            xh = torch.randn(x.shape[0], 256, device=dev)
+            oh = torch.zeros(M, 256, device=dev)
+            run_h = lambda: plan.run(w, xh, oh, accumulate=True)  # noqa: E731
+            sliced = time_reps_events(run_h, 10, 3)
+            os.environ["SGNN_SPMM_SLICE"] = "0"
+            whole = time_reps_events(run_h, 10, 3)
+            del os.environ["SGNN_SPMM_SLICE"]
+            extra["hidden_width_F256"] = {"median_ms": sliced["median_ms"], "GEdges_per_s": round(nnz / sliced["median_ms"] / 1e6, 3),
+                                          "feature_slices": 2, "median_ms_in_one_piece": whole["median_ms"]}
+            log(f"[bench] F=256 on the same graph: {sliced['median_ms']} ms in two feature slices, {whole['median_ms']} ms in one piece")
+            del xh, oh
     # one-time preparation, like the plan itself: the unchanged weight tensor was bound during warm-up
     extra["edge_values_bound_to_plan"] = plan._bound is not None
     extra["gather_model_total"] = {"algorithmic_bytes": int(b_total), "GBps": round(b_total / ms / 1e6, 1),

@@ -1968,9 +1968,22 @@ extern "C" int sgnn_spmm_plan_schedule(const sgnn_spmm_plan *p, int64_t F, int64
 
 // scratch != null: the call must not allocate.  The piece partials then go to `scratch` (scratch_floats
 // floats) instead of the plan's own, growable buffer, and nothing is created on the way.
+// Width of the feature slices of a wide fp32 product (a multiple of 4; >= F means one slice).  Multiples of
+// 128 floats go in slices of 128 (two row chunks per wavefront, the shape of the headline width); other widths
+// from 256 floats up in equal slices of at most 192.  SGNN_SPMM_SLICE=<floats> overrides (0 = never slice).
+static int64_t slice_width(int64_t F) {
+    const int e = env_int("SGNN_SPMM_SLICE", -1);
+    if (e == 0) return F;
+    if (e > 0) return std::max<int64_t>(4, (e + 3) / 4 * 4);
+    if (F < 256) return F;
+    if (F % 128 == 0) return 128;
+    const int64_t n = (F + 191) / 192;
+    return ((F + n - 1) / n + 3) / 4 * 4;
+}
+
 static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, int bits, float *out, int64_t F,
                     int64_t ldo, int accumulate, const float *row_div, hipStream_t st, float *scratch = nullptr,
-                    size_t scratch_floats = 0) {
+                    size_t scratch_floats = 0, bool is_slice = false) {
     SGNN_REQUIRE(p != nullptr, "plan is null");
     SGNN_REQUIRE(F > 0 && F < (1 << 24), "feature width F=%lld out of range", (long long)F);
     SGNN_REQUIRE(ldo >= F, "leading dimension smaller than F (ldo=%lld F=%lld)", (long long)ldo, (long long)F);
@@ -1995,6 +2008,44 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     SGNN_HIP_CHECK(hipGetDevice(&dev));
     SGNN_REQUIRE(dev == p->device, "plan was created on device %d, current device is %d", p->device, dev);
 
+    int vec = 1;
+    if (bits != 0) {
+        vec = F % 4 == 0 ? 4 : 2;  // checked by the caller: F even, 4-byte aligned packed buffer
+        // With a dense-degree matrix the fused kernels are bound by instruction issue (two fmas and a conversion
+        // per element), so idle lane slots cost time: F = 600 fills 150 of the 256 four-code slots of its lane-group
+        // shape but 300 of the 320 two-code slots (measured on the 114 M-edge community graph: 11.7 -> 10.5 ms).
+        if (vec == 4 && dq_slots(2, (int)(F / 2)) * 2 < dq_slots(4, (int)(F / 4)) * 4 * 0.8) vec = 2;
+        SGNN_REQUIRE(ldo % vec == 0 && aligned(out, 4 * vec),
+                     "the fused path at F=%lld needs out %d-byte aligned with ldo %% %d == 0", (long long)F, 4 * vec, vec);
+    } else if (F % 4 == 0 && dense.ldx % 4 == 0 && ldo % 4 == 0 && aligned(dense.x, 16) && aligned(out, 16)) {
+        vec = 4;
+    } else if (F % 2 == 0 && dense.ldx % 2 == 0 && ldo % 2 == 0 && aligned(dense.x, 8) && aligned(out, 8)) {
+        vec = 2;
+    }
+    if (bits == 0 && !is_slice) {
+        const BandShape sh = band_shape(p, F, ldo % 2 == 0 && aligned(out, 8));
+        if (band_wanted(p, F, sh)) {
+            bool done = false;
+            const int rc = spmm_run_band(p, sh, val, dense, out, F, ldo, accumulate, row_div, st, scratch == nullptr, &done);
+            if (rc != SGNN_OK || done) return rc;
+        }
+        // Wide fp32 rows: one product per slice of the feature axis, one after the other.  The rows a gather
+        // leaves in the caches are then 512 ... 768 bytes instead of 4F, so the same cache holds more of them:
+        // on the 62 M-edge power-law graph F = 256 takes 6.3 ms in two slices against 7.3 ms in one, F = 512
+        // 13.0 against 16.7, F = 1024 27.4 against 35.2 (the edge stream is read once per slice: +8 bytes on
+        // 4 * slice bytes per edge).  A slice is the same arithmetic on its own columns: results do not change.
+        const int64_t sw = slice_width(F);
+        if (vec == 4 && sw < F) {
+            for (int64_t s0 = 0; s0 < F; s0 += sw) {
+                DenseSrc d = dense;
+                d.x = dense.x + s0;
+                const int rc = spmm_run(p, val, d, 0, out + s0, std::min(sw, F - s0), ldo, accumulate, row_div, st, scratch,
+                                        scratch_floats, true);
+                if (rc != SGNN_OK) return rc;
+            }
+            return SGNN_OK;
+        }
+    }
     float *partial = p->partial;
     if (scratch != nullptr) {
         const size_t need = (size_t)p->n_items * (size_t)F;
@@ -2015,28 +2066,6 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
             p->partial_floats = need;
         }
         partial = p->partial;
-    }
-    int vec = 1;
-    if (bits != 0) {
-        vec = F % 4 == 0 ? 4 : 2;  // checked by the caller: F even, 4-byte aligned packed buffer
-        // With a dense-degree matrix the fused kernels are bound by instruction issue (two fmas and a conversion
-        // per element), so idle lane slots cost time: F = 600 fills 150 of the 256 four-code slots of its lane-group
-        // shape but 300 of the 320 two-code slots (measured on the 114 M-edge community graph: 11.7 -> 10.5 ms).
-        if (vec == 4 && dq_slots(2, (int)(F / 2)) * 2 < dq_slots(4, (int)(F / 4)) * 4 * 0.8) vec = 2;
-        SGNN_REQUIRE(ldo % vec == 0 && aligned(out, 4 * vec),
-                     "the fused path at F=%lld needs out %d-byte aligned with ldo %% %d == 0", (long long)F, 4 * vec, vec);
-    } else if (F % 4 == 0 && dense.ldx % 4 == 0 && ldo % 4 == 0 && aligned(dense.x, 16) && aligned(out, 16)) {
-        vec = 4;
-    } else if (F % 2 == 0 && dense.ldx % 2 == 0 && ldo % 2 == 0 && aligned(dense.x, 8) && aligned(out, 8)) {
-        vec = 2;
-    }
-    if (bits == 0) {
-        const BandShape sh = band_shape(p, F, ldo % 2 == 0 && aligned(out, 8));
-        if (band_wanted(p, F, sh)) {
-            bool done = false;
-            const int rc = spmm_run_band(p, sh, val, dense, out, F, ldo, accumulate, row_div, st, scratch == nullptr, &done);
-            if (rc != SGNN_OK || done) return rc;
-        }
     }
     const int nvec = (int)(F / vec);
     const int gw = group_width(nvec);

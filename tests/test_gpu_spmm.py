@@ -600,3 +600,41 @@ def test_leading_dimensions_through_the_c_abi(F, pad_x, pad_o, off_x, off_o):
         assert torch.equal(got[:, off_o:off_o + F], want)
         keep = torch.ones(F + pad_o, dtype=torch.bool, device=dev); keep[off_o:off_o + F] = False
         assert torch.equal(got[:, keep], ow[:, keep])
+
+
+@pytest.mark.parametrize("F", [256, 320, 384, 1024, 2052])
+def test_feature_slices_of_wide_products_change_nothing(F, monkeypatch):
+    # fp32 products from 256 columns up run one feature slice after the other (cache footprint of a gathered row);
+    # same bits as the unsliced product in every mode, with long and empty rows, and inside a padded window
+    ops = _gpu()
+    from super_gnn_amd._lib import lib, check
+    dev = torch.device("cuda:0")
+    M, K = 2000, 1800
+    rowptr, col, val = random_csr(M, K, 7, seed=F, empty_frac=0.15, hubs=4, hub_deg=700)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    g = torch.Generator().manual_seed(F + 1)
+    xw = torch.randn(K, F + 8, generator=g).to(dev)
+    ow = torch.randn(M, F + 4, generator=g).to(dev)
+    w = torch.from_numpy(val).to(dev)
+    div = torch.from_numpy(np.maximum(np.diff(rowptr), 1).astype(np.float32)).to(dev)
+    st = torch.cuda.current_stream().cuda_stream
+    for accumulate, row_div, wv in ((1, None, w), (0, None, w), (1, div, None), (0, div, w)):
+        outs = []
+        for sl in ("0", "-1", "64"):
+            monkeypatch.setenv("SGNN_SPMM_SLICE", sl)
+            got = ow.clone()
+            check(lib.sgnn_spmm_csr_f32(plan._h, wv.data_ptr() if wv is not None else None, xw.data_ptr() + 16,
+                                        got.data_ptr(), F, F + 8, F + 4, accumulate,
+                                        row_div.data_ptr() if row_div is not None else None, st))
+            torch.cuda.synchronize()
+            outs.append(got)
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+        assert torch.equal(outs[1][:, F:], ow[:, F:])
+    monkeypatch.setenv("SGNN_SPMM_SLICE", "-1")
+    x = xw[:, 4:4 + F].contiguous()
+    init = np.zeros((M, F), dtype=np.float32)
+    out = torch.zeros(M, F, device=dev)
+    plan.run(w, x, out, accumulate=True)
+    ref = init.copy(); orc.spmm_accumulate(rowptr, col, val, x.cpu().numpy(), ref)
+    short = np.diff(rowptr) <= plan.info()["long_row_threshold"]
+    assert np.array_equal(out.cpu().numpy()[short], ref[short])
