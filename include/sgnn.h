@@ -117,11 +117,11 @@ int sgnn_spmm_plan_bind_values(sgnn_spmm_plan *plan, const float *val, sgnn_stre
  * Short rows are summed in CSR edge order with one fused multiply-add per edge starting from
  * the old out value, as the reference does (bit-identical results); long rows are summed per piece
  * and the piece partials are added in piece order (deterministic, no atomics).
- * When F >= 256 and x, out, ldx, ldo allow 16-byte accesses, the product runs as consecutive feature
- * slices of 128 ... 192 columns (same kernels on column windows of x and out, same results): a
- * gathered row then leaves 512 ... 768 bytes in the caches instead of 4F, and the same cache holds more
- * rows.  The reference walks the feature axis in tiles of 64 columns for its own caches
- * (spmm.cpp:502-510). */
+ * When F >= 256, the dense operand is large (K * F * 4 bytes >= 0.9 GB) and x, out, ldx, ldo allow
+ * 16-byte accesses, the product runs as consecutive feature slices of 128 ... 192 columns (same kernels
+ * on column windows of x and out, same results): a gathered row then leaves 512 ... 768 bytes in the
+ * caches instead of 4F, and the same cache holds more rows.  The reference walks the feature axis in
+ * tiles of 64 columns for its own caches (spmm.cpp:502-510). */
 int sgnn_spmm_csr_f32(sgnn_spmm_plan *plan, const float *val, const float *x, float *out,
                       int64_t F, int64_t ldx, int64_t ldo, int accumulate, const float *row_div,
                       sgnn_stream_t stream);
@@ -134,9 +134,9 @@ int sgnn_spmm_csr_f32(sgnn_spmm_plan *plan, const float *val, const float *x, fl
  * until the process ends) instead of the plan's growable buffer.
  *   - limit: (#long-row pieces of the plan) * F * 4 bytes <= 64 MiB (sgnn_spmm_plan_info, info[4]);
  *     a larger product is refused with SGNN_ERR_ARG and nothing is launched.  Matrices without long
- *     rows never touch the scratch and have no limit.  A product of 256 or more 16-byte aligned columns
- *     runs as feature slices of 128 ... 192 columns one after the other (see sgnn_spmm_csr_f32), and the
- *     limit then applies to the width of one slice;
+ *     rows never touch the scratch and have no limit.  A product that runs as feature slices (see
+ *     sgnn_spmm_csr_f32) needs the partial sums of one slice at a time, and the limit then applies to
+ *     the width of a slice;
  *   - every call on one GPU shares that GPU's scratch: two calls whose kernels may overlap in time
  *     (different streams, different host threads) race on it.  Calls queued on one stream are safe.
  *     Nothing in the scratch has to start at zero: each call writes every partial it later reads;

@@ -1968,14 +1968,18 @@ extern "C" int sgnn_spmm_plan_schedule(const sgnn_spmm_plan *p, int64_t F, int64
 
 // scratch != null: the call must not allocate.  The piece partials then go to `scratch` (scratch_floats
 // floats) instead of the plan's own, growable buffer, and nothing is created on the way.
-// Width of the feature slices of a wide fp32 product (a multiple of 4; >= F means one slice).  Multiples of
-// 128 floats go in slices of 128 (two row chunks per wavefront, the shape of the headline width); other widths
-// from 256 floats up in equal slices of at most 192.  SGNN_SPMM_SLICE=<floats> overrides (0 = never slice).
-static int64_t slice_width(int64_t F) {
+// Width of the feature slices of a wide fp32 product (a multiple of 4; >= F means one slice).  Slices pay once the
+// dense operand is too large for the caches to hold its popular rows -- measured on power-law graphs of 0.15 M to
+// 2.45 M nodes at F = 256 and 512: with K * F * 4 bytes of 1.25 GB and more two to four slices take 0.78-0.92 of
+// the time of one piece, with 0.63 GB and less 1.07-1.30 (a second pass over the edge stream and a second tail
+// for nothing).  Multiples of 128 floats go in slices of 128 (two row chunks per wavefront, the shape of the
+// headline width); other widths from 256 floats up in equal slices of at most 192.
+// SGNN_SPMM_SLICE=<floats> forces slices of that width at any size (0 = never slice).
+static int64_t slice_width(int64_t F, int64_t K) {
     const int e = env_int("SGNN_SPMM_SLICE", -1);
     if (e == 0) return F;
     if (e > 0) return std::max<int64_t>(4, (e + 3) / 4 * 4);
-    if (F < 256) return F;
+    if (F < 256 || K * F * 4 < 900000000ll) return F;
     if (F % 128 == 0) return 128;
     const int64_t n = (F + 191) / 192;
     return ((F + n - 1) / n + 3) / 4 * 4;
@@ -2029,12 +2033,12 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
             const int rc = spmm_run_band(p, sh, val, dense, out, F, ldo, accumulate, row_div, st, scratch == nullptr, &done);
             if (rc != SGNN_OK || done) return rc;
         }
-        // Wide fp32 rows: one product per slice of the feature axis, one after the other.  The rows a gather
-        // leaves in the caches are then 512 ... 768 bytes instead of 4F, so the same cache holds more of them:
+        // Wide fp32 rows of a large operand: one product per slice of the feature axis, one after the other.  The rows
+        // a gather leaves in the caches are then 512 ... 768 bytes instead of 4F, so the same cache holds more of them:
         // on the 62 M-edge power-law graph F = 256 takes 6.3 ms in two slices against 7.3 ms in one, F = 512
         // 13.0 against 16.7, F = 1024 27.4 against 35.2 (the edge stream is read once per slice: +8 bytes on
         // 4 * slice bytes per edge).  A slice is the same arithmetic on its own columns: results do not change.
-        const int64_t sw = slice_width(F);
+        const int64_t sw = slice_width(F, p->K);
         if (vec == 4 && sw < F) {
             for (int64_t s0 = 0; s0 < F; s0 += sw) {
                 DenseSrc d = dense;

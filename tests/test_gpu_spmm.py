@@ -604,8 +604,9 @@ def test_leading_dimensions_through_the_c_abi(F, pad_x, pad_o, off_x, off_o):
 
 @pytest.mark.parametrize("F", [256, 320, 384, 1024, 2052])
 def test_feature_slices_of_wide_products_change_nothing(F, monkeypatch):
-    # fp32 products from 256 columns up run one feature slice after the other (cache footprint of a gathered row);
-    # same bits as the unsliced product in every mode, with long and empty rows, and inside a padded window
+    # wide fp32 products of large operands run one feature slice after the other (cache footprint of a gathered row);
+    # forced here on a small matrix: same bits as the unsliced product in every mode, with long and empty rows, and
+    # inside a padded window
     ops = _gpu()
     from super_gnn_amd._lib import lib, check
     dev = torch.device("cuda:0")
@@ -620,7 +621,7 @@ def test_feature_slices_of_wide_products_change_nothing(F, monkeypatch):
     st = torch.cuda.current_stream().cuda_stream
     for accumulate, row_div, wv in ((1, None, w), (0, None, w), (1, div, None), (0, div, w)):
         outs = []
-        for sl in ("0", "-1", "64"):
+        for sl in ("0", "128", "172"):
             monkeypatch.setenv("SGNN_SPMM_SLICE", sl)
             got = ow.clone()
             check(lib.sgnn_spmm_csr_f32(plan._h, wv.data_ptr() if wv is not None else None, xw.data_ptr() + 16,
@@ -630,7 +631,7 @@ def test_feature_slices_of_wide_products_change_nothing(F, monkeypatch):
             outs.append(got)
         assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
         assert torch.equal(outs[1][:, F:], ow[:, F:])
-    monkeypatch.setenv("SGNN_SPMM_SLICE", "-1")
+    monkeypatch.setenv("SGNN_SPMM_SLICE", "64")
     x = xw[:, 4:4 + F].contiguous()
     init = np.zeros((M, F), dtype=np.float32)
     out = torch.zeros(M, F, device=dev)
@@ -638,3 +639,29 @@ def test_feature_slices_of_wide_products_change_nothing(F, monkeypatch):
     ref = init.copy(); orc.spmm_accumulate(rowptr, col, val, x.cpu().numpy(), ref)
     short = np.diff(rowptr) <= plan.info()["long_row_threshold"]
     assert np.array_equal(out.cpu().numpy()[short], ref[short])
+
+
+def test_feature_slices_at_the_size_where_the_library_chooses_them(monkeypatch):
+    # 1.0 M dense rows of 256 floats (1.02 GB): above the operand size from which the library slices by itself
+    ops = _gpu()
+    from super_gnn_amd import synth
+    dev = torch.device("cuda:0")
+    n, F = 1_000_000, 256
+    rowptr, col = synth.rmat_graph(n, 6_000_000, a=0.57, b=0.19, c=0.19, seed=4, device=dev)
+    w = synth.gcn_norm_weights(rowptr, col)
+    plan = ops.SpmmPlan(rowptr, col, n)
+    assert plan.info()["long_rows"] > 0
+    g = torch.Generator(device=dev).manual_seed(9)
+    x = torch.randn(n, F, generator=g, device=dev)
+    init = torch.randn(n, F, generator=g, device=dev)
+    outs = []
+    for sl in (None, "0"):
+        if sl is None:
+            monkeypatch.delenv("SGNN_SPMM_SLICE", raising=False)
+        else:
+            monkeypatch.setenv("SGNN_SPMM_SLICE", sl)
+        out = init.clone()
+        plan.run(w, x, out, accumulate=True)
+        torch.cuda.synchronize()
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
