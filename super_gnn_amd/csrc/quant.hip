@@ -34,11 +34,14 @@ __device__ __forceinline__ float dpp_f(float v) {
 struct OpMinF { __device__ static float f(float a, float b) { return fminf(a, b); } };
 struct OpMaxF { __device__ static float f(float a, float b) { return fmaxf(a, b); } };
 
-// All-reduce over a group of G consecutive lanes (G in {8, 16, 32, 64}); every lane gets the result.
+// All-reduce over a group of G consecutive lanes (G in {1, 2, 4, 8, 16, 32, 64}); every lane gets the result.
 template <int G, typename Op>
 __device__ __forceinline__ float group_allreduce_f(float v) {
+    if constexpr (G == 1) return v;
     v = Op::f(v, dpp_f<0xB1>(v));
+    if constexpr (G == 2) return v;
     v = Op::f(v, dpp_f<0x4E>(v));
+    if constexpr (G == 4) return v;
     v = Op::f(v, dpp_f<0x141>(v));
     if constexpr (G == 8) return v;
     v = Op::f(v, dpp_f<0x140>(v));
@@ -61,8 +64,11 @@ __device__ __forceinline__ float group_allreduce_f(float v) {
 
 template <int G>
 __device__ __forceinline__ int group_allmin_i(int v) {
+    if constexpr (G == 1) return v;
     v = min(v, dpp_i<0xB1>(v));
+    if constexpr (G == 2) return v;
     v = min(v, dpp_i<0x4E>(v));
+    if constexpr (G == 4) return v;
     v = min(v, dpp_i<0x141>(v));
     if constexpr (G == 8) return v;
     v = min(v, dpp_i<0x140>(v));
@@ -330,7 +336,8 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
 // flight); neighbouring lane groups hold consecutive fp32 rows, i.e. exactly the rows that share a packed
 // byte (four at int2, two at int4), so packing is a shift in each lane followed by an OR across lane
 // groups.  Narrow rows take L = 8: the work per row (reductions, scale, reciprocal, parameter store) is
-// then spread over twice as many elements per lane, which is what limits rows of 64 and 128 floats.
+// then spread over twice as many elements per lane, which is what limits rows of 64 and 128 floats.  Rows
+// of at most 16, 8 and 4 floats take L = 4, 2 and 1, so that a lane group has no idle lanes.
 // ------------------------------------------------------------------------------------------------
 // FULL: F == 4 * L * NV, every lane's every vector lies inside the row (no per-load lane predicates).
 // RAGGED: any F and any 4-byte aligned row start (F = 602, F = 123, a window with an odd leading dimension):
@@ -512,9 +519,12 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
             if constexpr (L == 16) {
                 if constexpr (EPB >= 2) w |= (uint32_t)__shfl_xor((int)w, 16, 64);
                 if constexpr (EPB == 4) w |= (uint32_t)__shfl_xor((int)w, 32, 64);
-            } else {  // L == 8: the neighbouring row sits in the other half of the DPP row (row_ror:8 swaps the halves)
+            } else if constexpr (L == 8) {  // the neighbouring row sits in the other half of the DPP row (row_ror:8 swaps the halves)
                 if constexpr (EPB >= 2) w |= (uint32_t)dpp_i<0x128>((int)w);
                 if constexpr (EPB == 4) w |= (uint32_t)__shfl_xor((int)w, 16, 64);
+            } else {  // L lanes per row, L in {1, 2, 4}: the rows of a packed byte sit L and 2 L lanes apart
+                if constexpr (EPB >= 2) w |= (uint32_t)__shfl_xor((int)w, L, 64);
+                if constexpr (EPB == 4) w |= (uint32_t)__shfl_xor((int)w, 2 * L, 64);
             }
             const bool mine = EPB == 1 ? true : EPB == 2 ? ((d & 1) == (v & 1)) : ((d & 3) == (v & 3));
             if constexpr (STAGED) {
@@ -1621,6 +1631,9 @@ static void dispatch_rows_ragged_wide(const RowsArgs &a, hipStream_t st) {
 template <int BITS>
 static void dispatch_quant16_ragged(const RowsArgs &a, hipStream_t st) {
     const int nvec = (a.F + 3) / 4;
+    if (nvec <= 1) return launch_quant16_ragged<BITS, 1, 1>(a, st);
+    if (nvec <= 2) return launch_quant16_ragged<BITS, 1, 2>(a, st);
+    if (nvec <= 4) return launch_quant16_ragged<BITS, 1, 4>(a, st);
     if (nvec <= 8) return launch_quant16_ragged<BITS, 1, 8>(a, st);
     if (nvec <= 16) return launch_quant16_ragged<BITS, 2, 8>(a, st);
     if (nvec <= 32) return launch_quant16_ragged<BITS, 2, 16>(a, st);
@@ -1731,6 +1744,9 @@ static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
             // rows of up to 128 floats: eight lanes per row (SGNN_QUANT_LAYOUT8=0: sixteen, for comparison)
             static const bool layout8 = [] { const char *e = getenv("SGNN_QUANT_LAYOUT8"); return !(e && e[0] == '0'); }();
             if (layout8 && (a.F % 32 == 0 || nvec <= 16)) {   // (a ragged 17..31-vector row gains nothing from it)
+                if (nvec <= 1) return launch_quant16<BITS, 1, 1>(a, st);
+                if (nvec <= 2) return launch_quant16<BITS, 1, 2>(a, st);
+                if (nvec <= 4) return launch_quant16<BITS, 1, 4>(a, st);
                 if (nvec <= 8) return launch_quant16<BITS, 1, 8>(a, st);
                 if (nvec <= 16) return launch_quant16<BITS, 2, 8>(a, st);
                 if (nvec <= 32) return launch_quant16<BITS, 4, 8>(a, st);

@@ -49,7 +49,10 @@ def test_known_answers(name):
 
 @pytest.mark.parametrize("bits", [8, 4, 2])
 @pytest.mark.parametrize("n,F", [(2000, 128), (1001, 256), (4333, 123), (515, 602), (333, 64), (77, 100), (130, 1024),
-                                 (41, 1200), (9, 4), (63, 16), (50, 2050), (3, 1)])
+                                 (41, 1200), (9, 4), (63, 16), (50, 2050), (3, 1),
+                                 # rows of at most 16 floats: four, two lanes or one lane per row
+                                 (3001, 4), (1027, 8), (2049, 10), (777, 12), (1500, 16), (999, 6), (1001, 3), (513, 2),
+                                 (2500, 1), (800, 5), (700, 13)])
 def test_rows_bit_exact_vs_oracle(bits, n, F):
     g = torch.Generator().manual_seed(n * 31 + F + bits)
     x = torch.randn(n, F, generator=g)
@@ -68,7 +71,7 @@ def test_rows_bit_exact_vs_oracle(bits, n, F):
 
 
 @pytest.mark.parametrize("bits", [8, 4, 2])
-@pytest.mark.parametrize("F", [128, 123, 602])
+@pytest.mark.parametrize("F", [128, 123, 602, 4, 10, 16, 7, 1])
 def test_many_segments_bit_exact(bits, F):
     # the reference script's layout check: 256 random segments (tests/test_quantization_ops.py:130-148)
     rng = np.random.default_rng(bits + F)
