@@ -99,6 +99,25 @@ def test_many_segments_bit_exact(bits, F):
     assert np.all(np.abs(d - d_ref) <= dequant_atol(p_ref[:, 0], p_ref[:, 1], bits)[:, None])
 
 
+@pytest.mark.parametrize("bits", [8, 2])
+@pytest.mark.parametrize("P", [2, 62, 63, 64, 65, 126, 127, 128, 700])
+def test_segment_counts_around_the_table_lookup_blocks(bits, P):
+    # a wavefront looks its segment up 63 table entries at a time: counts on both sides of every block edge, with
+    # empty segments (repeated cut points) and segments shorter than a packed row
+    rng = np.random.default_rng(P * 10 + bits)
+    n, F = 2900, 64
+    x = rng.standard_normal((n, F), dtype=np.float32)
+    cuts = np.sort(rng.integers(0, n + 1, size=P - 1))
+    cuts[: (P - 1) // 4] = cuts[(P - 1) // 4]      # a run of empty segments at the front
+    seg = np.concatenate([[0], cuts, [n]]).astype(np.int32)
+    q_ref, p_ref = orc.quant_rows(x, seg, bits)
+    q, params, d = _quant_gpu(x, seg, bits)
+    assert np.array_equal(params.view(np.uint32), p_ref.view(np.uint32))
+    assert np.array_equal(q, q_ref)
+    d_ref = orc.dequant_rows(q_ref, p_ref, seg, bits, F)
+    assert np.all(np.abs(d - d_ref) <= dequant_atol(p_ref[:, 0], p_ref[:, 1], bits)[:, None])
+
+
 @pytest.mark.parametrize("bits", [8, 4, 2])
 def test_reference_x86_vectors(bits):
     x = RV[f"qrows{bits}_x"]
