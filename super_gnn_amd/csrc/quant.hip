@@ -102,7 +102,7 @@ __device__ __forceinline__ int find_segment(const int32_t *__restrict__ pseg, in
 // entry i of both tables, a ballot counts the entries that do not exceed the key, and the four ends are read out
 // of the lanes that hold them -- where a binary search makes log2(P) dependent loads, plus one more round for
 // the ends, before a wavefront can issue its first data load (eight segments: quantize+pack of 4 M x 64 int2
-// 0.218 -> 0.19 ms).  Longer tables are first narrowed to 63 segments by a binary search over every 63rd entry.
+// 0.218 -> 0.198 ms).  Longer tables are first narrowed to 63 segments by a binary search over every 63rd entry.
 struct WaveSegment { int p, k0, k1, o0, o1; };
 __device__ __forceinline__ WaveSegment wave_find_segment(const int32_t *__restrict__ keys, const int32_t *__restrict__ other,
                                                          int P, int key) {
@@ -126,28 +126,6 @@ __device__ __forceinline__ WaveSegment wave_find_segment(const int32_t *__restri
     w.k1 = __builtin_amdgcn_readlane(mk, k + 1);
     w.o0 = __builtin_amdgcn_readlane(mo, k);
     w.o1 = __builtin_amdgcn_readlane(mo, k + 1);
-    return w;
-}
-
-// For wavefronts that live for one or two stores (the flat dequantizers) a short table is searched faster by the
-// log2(P) dependent scalar loads of a binary search, which hit the scalar cache, than by one round of vector
-// loads (measured at eight segments, 1 M x 256 int2: 0.177 against 0.195 ms; at 256 segments 0.215 against
-// 0.200 ms; at 4096 0.288 against 0.232 ms).  A four-way search with speculative loads of the ends (two rounds of
-// loads instead of four at eight segments) measured the same as the binary search.
-__device__ __forceinline__ WaveSegment wave_find_segment_short_lived(const int32_t *__restrict__ keys,
-                                                                     const int32_t *__restrict__ other, int P, int key) {
-    if (P > 64) return wave_find_segment(keys, other, P, key);
-    int lo = 0, hi = P - 1;
-    while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (keys[mid + 1] > key) hi = mid; else lo = mid + 1;
-    }
-    WaveSegment w;
-    w.p = lo;
-    w.k0 = keys[lo];
-    w.k1 = keys[lo + 1];
-    w.o0 = other[lo];
-    w.o1 = 0;  // not needed by these kernels
     return w;
 }
 
@@ -751,7 +729,7 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_kernel(
     if constexpr (SEGMENTED) {
         const int64_t i0 = ((int64_t)blockIdx.x * (kQBlock / 64) + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))) * (R * 64);
         const int row_w = (int)(POW2 ? (i0 >> g_shift) : (i0 / G));
-        const WaveSegment ws = wave_find_segment_short_lived(seg, pseg, P, row_w);  // the wave's first vector exists, so row_w < seg[P]
+        const WaveSegment ws = wave_find_segment(seg, pseg, P, row_w);  // the wave's first vector exists, so row_w < seg[P]
         w_p = ws.p;
         w_s0 = ws.k0;
         w_s1 = ws.k1;
@@ -826,7 +804,7 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_ragged_kernel(
     if constexpr (SEGMENTED) {  // the segment of the wave's first row, found on wave-uniform values
         const int64_t i0 = ((int64_t)blockIdx.x * (kQBlock / 64) + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))) * (R * 64);
         const int row_w = (int)((i0 * 4) / F);
-        const WaveSegment ws = wave_find_segment_short_lived(seg, pseg, P, row_w);  // the wave's first vector exists, so row_w < seg[P]
+        const WaveSegment ws = wave_find_segment(seg, pseg, P, row_w);  // the wave's first vector exists, so row_w < seg[P]
         w_p = ws.p;
         w_s0 = ws.k0;
         w_s1 = ws.k1;
@@ -936,7 +914,7 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_odd_kernel(
     if constexpr (SEGMENTED) {  // the segment of the wave's first row
         const int64_t i0 = ((int64_t)blockIdx.x * (kQBlock / 64) + __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))) * (R * 64);
         const int row_w = (int)((i0 * 4) / F);
-        ws = wave_find_segment_short_lived(seg, pseg, P, row_w < n_rows ? row_w : n_rows - 1);
+        ws = wave_find_segment(seg, pseg, P, row_w < n_rows ? row_w : n_rows - 1);
     }
     auto slot_of = [&](int row) {
         if constexpr (!SEGMENTED) return row;
@@ -1772,8 +1750,19 @@ static void launch_dequant_flat_r(const RowsArgs &a, int64_t n_rows, hipStream_t
 template <int BITS>
 static void launch_dequant_flat(const RowsArgs &a, int64_t n_rows, hipStream_t st) {
     const int G = a.F / 4;
-    if (BITS != 8 && (G & (G - 1)) == 0) launch_dequant_flat_r<BITS, 1>(a, n_rows, st);
-    else launch_dequant_flat_r<BITS, 2>(a, n_rows, st);
+    // With several segments and sub-byte codes every wavefront first looks its segment up, and the shortest waves
+    // lose: 1 M x 256 int2 in eight segments 0.194 ms with one store per wave, 0.169 with two, 0.160 with four
+    // (one segment: 0.155 / 0.171 / 0.170); int4 0.199 / 0.162 / 0.162.  SGNN_DEQUANT_R=1/2/4 forces a shape.
+    const char *e = getenv("SGNN_DEQUANT_R");
+    int r = e ? atoi(e) : 0;
+    if (r != 1 && r != 2 && r != 4) {
+        if (BITS == 8) r = 2;
+        else if (a.P <= 1) r = (G & (G - 1)) == 0 ? 1 : 2;
+        else r = BITS == 2 && a.F <= 256 ? 4 : 2;
+    }
+    if (r == 4) launch_dequant_flat_r<BITS, 4>(a, n_rows, st);
+    else if (r == 2) launch_dequant_flat_r<BITS, 2>(a, n_rows, st);
+    else launch_dequant_flat_r<BITS, 1>(a, n_rows, st);
 }
 
 template <int BITS, int VEC>
