@@ -1757,7 +1757,7 @@ static void launch_dequant_flat(const RowsArgs &a, int64_t n_rows, hipStream_t s
     int r = e ? atoi(e) : 0;
     if (r != 1 && r != 2 && r != 4) {
         if (BITS == 8) r = 2;
-        else if (a.P <= 1) r = (G & (G - 1)) == 0 ? 1 : 2;
+        else if (a.P <= 1) r = (G & (G - 1)) == 0 ? 1 : BITS == 2 ? 4 : 2;
         else r = BITS == 2 && a.F <= 256 ? 4 : 2;
     }
     if (r == 4) launch_dequant_flat_r<BITS, 4>(a, n_rows, st);
