@@ -296,19 +296,23 @@ def wl_copy(args, ctx):
             "cpu_baseline": None, "extra": {}}
 
 
-def quant_case(ops, x, bits, steps, warmup):
-    """Quantize+pack and unpack+dequantize of x at one width: times, rates, rooflines."""
+def quant_case(ops, x, bits, steps, warmup, segments=1):
+    """Quantize+pack and unpack+dequantize of x at one width: times, rates, rooflines.  segments > 1: the rows
+    are cut at seeded random points into that many per-peer segments, each padded to whole packed rows."""
+    import numpy as np
     import torch
     n, F = x.shape
     epb = 8 // bits
-    seg = torch.tensor([0, n], dtype=torch.int32)
-    q = torch.empty((n + epb - 1) // epb, F, dtype=torch.uint8, device=x.device)
+    cuts = np.sort(np.random.default_rng(segments).integers(0, n, size=segments - 1)).tolist() if segments > 1 else []
+    seg = torch.tensor([0] + cuts + [n], dtype=torch.int32)
+    n_packed = sum(-(-(b_ - a_) // epb) for a_, b_ in zip(seg[:-1].tolist(), seg[1:].tolist()))
+    q = torch.empty(n_packed, F, dtype=torch.uint8, device=x.device)
     p = torch.empty(n, 2, device=x.device)
     d = torch.empty(n, F, device=x.device)
     wl = f"quant_pack_int{bits}_{n}x{F}"
     b = quant_bytes(n, F, bits)
-    ms_q, kq, _ = profiled_steps(lambda: ops.quantize_tensor_for_all_procs(x, q, p, seg, 1, bits), steps, warmup)
-    ms_d, kd, _ = profiled_steps(lambda: ops.dequantize_tensor_for_all_procs(q, d, p, seg, 1, bits), steps, warmup)
+    ms_q, kq, _ = profiled_steps(lambda: ops.quantize_tensor_for_all_procs(x, q, p, seg, segments, bits), steps, warmup)
+    ms_d, kd, _ = profiled_steps(lambda: ops.dequantize_tensor_for_all_procs(q, d, p, seg, segments, bits), steps, warmup)
     kq_ms, kd_ms = kq["quant_pack_rows_kernel"], kd["unpack_dequant_rows_kernel"]
     return {"workload": wl, "bytes": b, "quant_ms": ms_q, "dequant_ms": ms_d,
             "quant_GBps_wall": round(b / ms_q / 1e6, 1), "dequant_GBps_wall": round(b / ms_d / 1e6, 1),
@@ -555,7 +559,7 @@ def wl_quant_widths(args, ctx):
         x = synth.boundary_features(n, F, seed=5, device=ctx["dev"])
         row = {}
         for bits in (8, 4, 2):
-            c = quant_case(ops, x, bits, max(args.steps, 5), max(args.warmup, 2))
+            c = quant_case(ops, x, bits, max(args.steps, 5), max(args.warmup, 2), segments=args.segments)
             row[f"int{bits}"] = {"quant_us": round(c["quant_roofline"]["kernel_ms_per_step"] * 1e3, 1),
                                  "quant_GBps": c["quant_roofline"]["gather_model"]["GBps"],
                                  "dequant_us": round(c["dequant_roofline"]["kernel_ms_per_step"] * 1e3, 1),
@@ -567,7 +571,7 @@ def wl_quant_widths(args, ctx):
         torch.cuda.empty_cache()
     worst = min(r["int2"]["quant_GBps"] for r in table.values())
     return {"metric": "quantize-pack GB/s at int2, slowest row width of the sweep", "value": worst, "unit": "GB/s",
-            "config": {"workload": "quant_widths_256M_floats", "widths": widths}, "ms_per_step": 0.0, "dtype": "u8",
+            "config": {"workload": "quant_widths_256M_floats", "widths": widths, "segments": args.segments}, "ms_per_step": 0.0, "dtype": "u8",
             "roofline": None, "cpu_baseline": None, "extra": {"kernel_rates_by_width": table}}
 
 
@@ -750,6 +754,7 @@ def main():
     ap.add_argument("--bits", type=int, default=2)
     ap.add_argument("--widths", default="32,64,100,123,128,200,256,300,500,600,602,640,1000,1024,1200,2050",
                     help="quant_widths: row widths of the sweep")
+    ap.add_argument("--segments", type=int, default=1, help="quant_widths: cut the rows into this many per-peer segments")
     ap.add_argument("--long-threshold", type=int, default=0, help="SpMM plan: rows longer than this are split (0 = default)")
     ap.add_argument("--piece-edges", type=int, default=0, help="SpMM plan: minimum edges per long-row piece (0 = default)")
     ap.add_argument("--no-extras", action="store_true", help="only the chosen workload (used under rocprofv3)")

@@ -1765,9 +1765,8 @@ static void launch_dequant_flat(const RowsArgs &a, int64_t n_rows, hipStream_t s
     else launch_dequant_flat_r<BITS, 1>(a, n_rows, st);
 }
 
-template <int BITS, int VEC>
-static void launch_dequant_flat_ragged(const RowsArgs &a, int64_t n_rows, hipStream_t st) {
-    constexpr int R = 2;
+template <int BITS, int VEC, int R>
+static void launch_dequant_flat_ragged_r(const RowsArgs &a, int64_t n_rows, hipStream_t st) {
     const int64_t n_elem = n_rows * (int64_t)a.F;
     const int64_t n_vec = (n_elem + 3) / 4;
     const int64_t n_waves = (n_vec + R * 64 - 1) / (R * 64);
@@ -1790,6 +1789,15 @@ static void launch_dequant_flat_ragged(const RowsArgs &a, int64_t n_rows, hipStr
     else
         hipLaunchKernelGGL((unpack_dequant_flat_ragged_kernel<BITS, VEC, R, false>), dim3(nb), dim3(kQBlock), 0, st, a.q_in,
                            a.x_out, a.params, a.seg, a.pseg, a.P, a.F, n_elem);
+}
+
+template <int BITS, int VEC>
+static void launch_dequant_flat_ragged(const RowsArgs &a, int64_t n_rows, hipStream_t st) {
+    const char *e = getenv("SGNN_DEQUANT_R");
+    const int r = e ? atoi(e) : 0;
+    // several segments and sub-byte codes: four stores per wavefront per segment lookup (see launch_dequant_flat)
+    if (r == 4 || (r != 2 && BITS != 8 && a.P > 1)) launch_dequant_flat_ragged_r<BITS, VEC, 4>(a, n_rows, st);
+    else launch_dequant_flat_ragged_r<BITS, VEC, 2>(a, n_rows, st);
 }
 
 template <int BITS>
