@@ -1668,6 +1668,8 @@ static BandShape band_shape(const sgnn_spmm_plan *p, int64_t F, bool even_out) {
     const int nvec = (int)((F + 3) / 4);
     b.n_slices = kNumXCD;
     while (b.n_slices > 1 && (nvec + b.n_slices - 1) / b.n_slices < 16) b.n_slices /= 2;
+    const int forced = env_int("SGNN_SPMM_BAND_SLICES", 0);
+    if (forced == 1 || forced == 2 || forced == 4 || forced == 8) b.n_slices = forced;
     b.slice_floats = 4 * ((nvec + b.n_slices - 1) / b.n_slices);
     b.slice_pad = (b.slice_floats + 15) / 16 * 16;
     b.G = std::max(16, std::min(64, b.slice_pad / 4));
