@@ -1692,7 +1692,7 @@ static void dispatch_quant16_ragged(const RowsArgs &a, hipStream_t st) {
     if (nvec <= 4) return launch_quant16_ragged<BITS, 1, 4>(a, st);
     if (nvec <= 8) return launch_quant16_ragged<BITS, 1, 8>(a, st);
     if (nvec <= 16) return launch_quant16_ragged<BITS, 2, 8>(a, st);
-    if (nvec <= 32) return launch_quant16_ragged<BITS, 2, 16>(a, st);
+    if (nvec <= 32) return launch_quant16_ragged<BITS, 4, 8>(a, st);   // (sixteen lanes with two vectors each: 3 ... 20 % slower)
     if (nvec <= 64) return launch_quant16_ragged<BITS, 4, 16>(a, st);
     if (nvec <= 128) return launch_quant16_ragged<BITS, 8, 16>(a, st);
     if (nvec <= 160) return launch_quant16_ragged<BITS, 10, 16>(a, st);
@@ -1818,7 +1818,9 @@ static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
         if (a.quantize && a.layout16) {
             // rows of up to 128 floats: eight lanes per row (SGNN_QUANT_LAYOUT8=0: sixteen, for comparison)
             static const bool layout8 = [] { const char *e = getenv("SGNN_QUANT_LAYOUT8"); return !(e && e[0] == '0'); }();
-            if (layout8 && (a.F % 32 == 0 || nvec <= 16)) {   // (a ragged 17..31-vector row gains nothing from it)
+            // (with the staged output also for rows of 17 ... 31 vectors, whose groups have idle lanes either way:
+            // F = 72 / 80 3.8-4.7 -> 4.7-5.7 TB/s, F = 100 / 112 +3 ... 6 %)
+            if (layout8) {
                 if (nvec <= 1) return launch_quant16<BITS, 1, 1>(a, st);
                 if (nvec <= 2) return launch_quant16<BITS, 1, 2>(a, st);
                 if (nvec <= 4) return launch_quant16<BITS, 1, 4>(a, st);
