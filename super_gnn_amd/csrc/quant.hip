@@ -2049,11 +2049,14 @@ extern "C" int sgnn_dequant_v1_f32(const uint8_t *q, float *x, const int64_t *ra
     // (SGNN_DEQUANT_V1_FLAT=0 / 1: never / at every width, for comparison)
     static const int flat_mode = [] { const char *e = getenv("SGNN_DEQUANT_V1_FLAT"); return e ? atoi(e) : -1; }();
     if (F % 4 == 0 && aligned(x, 16) && (flat_mode == 1 || (flat_mode != 0 && (F <= 128 || F > 1024)))) {
-        constexpr int R = 2;
+        // stores per wavefront: four measured 1-3 % above two and 10-15 % above one (SGNN_DEQUANT_V1_R=1/2/4 forces one)
+        const char *e = getenv("SGNN_DEQUANT_V1_R");
+        const int r = e ? atoi(e) : 4;
         const int64_t n_vec = n * (F / 4);
-        const int64_t n_waves = (n_vec + R * 64 - 1) / (R * 64);
-        hipLaunchKernelGGL((dequant_v1_flat_kernel<R>), dim3((uint32_t)((n_waves + kQBlock / 64 - 1) / (kQBlock / 64))), block, 0, st,
-                           q, x, range, params, n_vec, (int)(F / 4));
+        const auto waves = [&](int R) { return dim3((uint32_t)(((n_vec + R * 64 - 1) / (R * 64) + kQBlock / 64 - 1) / (kQBlock / 64))); };
+        if (r == 2) hipLaunchKernelGGL((dequant_v1_flat_kernel<2>), waves(2), block, 0, st, q, x, range, params, n_vec, (int)(F / 4));
+        else if (r == 1) hipLaunchKernelGGL((dequant_v1_flat_kernel<1>), waves(1), block, 0, st, q, x, range, params, n_vec, (int)(F / 4));
+        else hipLaunchKernelGGL((dequant_v1_flat_kernel<4>), waves(4), block, 0, st, q, x, range, params, n_vec, (int)(F / 4));
     } else if (F % 4 == 0 && F <= 1024 && aligned(x, 16)) {
         if (F <= 256) hipLaunchKernelGGL((dequant_v1_vec_kernel<1, 4>), grid_r(4), block, 0, st, q, x, range, params, n, (int)F);
         else if (F <= 512) hipLaunchKernelGGL((dequant_v1_vec_kernel<2, 2>), grid_r(2), block, 0, st, q, x, range, params, n, (int)F);
