@@ -1824,6 +1824,12 @@ static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
                 if (nvec <= 1) return launch_quant16<BITS, 1, 1>(a, st);
                 if (nvec <= 2) return launch_quant16<BITS, 1, 2>(a, st);
                 if (nvec <= 4) return launch_quant16<BITS, 1, 4>(a, st);
+                // rows of 5 ... 12 vectors other than the whole eight-lane pass F = 32: four lanes per row (F = 20 / 24:
+                // 3.2-4.3 -> 4.1-5.2 TB/s, F = 28 ... 48: +4 ... 17 %; from 13 vectors on eight lanes win, F = 52 ... 64 by
+                // 6 ... 18 %).  SGNN_QUANT_LAYOUT4=0: eight lanes for all of them.
+                static const bool layout4 = [] { const char *e = getenv("SGNN_QUANT_LAYOUT4"); return !(e && e[0] == '0'); }();
+                if (layout4 && nvec <= 8 && a.F != 32) return launch_quant16<BITS, 2, 4>(a, st);
+                if (layout4 && nvec > 8 && nvec <= 12) return launch_quant16<BITS, 4, 4>(a, st);
                 if (nvec <= 8) return launch_quant16<BITS, 1, 8>(a, st);
                 if (nvec <= 16) return launch_quant16<BITS, 2, 8>(a, st);
                 if (nvec <= 32) return launch_quant16<BITS, 4, 8>(a, st);

@@ -52,7 +52,9 @@ def test_known_answers(name):
                                  (41, 1200), (9, 4), (63, 16), (50, 2050), (3, 1),
                                  # rows of at most 16 floats: four, two lanes or one lane per row
                                  (3001, 4), (1027, 8), (2049, 10), (777, 12), (1500, 16), (999, 6), (1001, 3), (513, 2),
-                                 (2500, 1), (800, 5), (700, 13)])
+                                 (2500, 1), (800, 5), (700, 13),
+                                 # 5 ... 12 vectors per row: four lanes per row, two or four vectors per lane
+                                 (1111, 20), (901, 24), (1203, 28), (777, 36), (650, 44), (1024, 48), (300, 52)])
 def test_rows_bit_exact_vs_oracle(bits, n, F):
     g = torch.Generator().manual_seed(n * 31 + F + bits)
     x = torch.randn(n, F, generator=g)
@@ -71,7 +73,7 @@ def test_rows_bit_exact_vs_oracle(bits, n, F):
 
 
 @pytest.mark.parametrize("bits", [8, 4, 2])
-@pytest.mark.parametrize("F", [128, 123, 602, 4, 10, 16, 7, 1])
+@pytest.mark.parametrize("F", [128, 123, 602, 4, 10, 16, 7, 1, 24, 40])
 def test_many_segments_bit_exact(bits, F):
     # the reference script's layout check: 256 random segments (tests/test_quantization_ops.py:130-148)
     rng = np.random.default_rng(bits + F)
