@@ -6,22 +6,29 @@
 A step is one pass of the hot path over one batch of synthetic input that is already resident in
 HBM.  The default workload is the headline configuration: a weighted-sum SpMM (out += A @ X,
 GCN-normalised edge weights) over an R-MAT power-law graph with 2.45 M nodes / ~62 M stored edges
-at F = 128 fp32.  Unless --no-extras is given the same run also measures, as entries of
-``extra["workloads"]`` with their own kernel times and roofline objects: the dense-degree
+at F = 128 fp32.  Unless --no-extras is given the same run also measures the dense-degree
 community graph at F = 602 (``sbm``), the pre/post-aggregation partition with int2-packed remote
 rows (``prepost``), the small CPU-runnable case (``small``), the int8/int4/int2 quantize+pack and
-unpack+dequantize kernels on 1 M x 256 and 2 M x 128 boundary rows (``quant``), a streaming copy
-(the attainable-bandwidth yardstick) and the CPU baselines timed on this machine's host cores.
-Any of them can be made the headline of the line with --workload.
+unpack+dequantize kernels on 1 M x 256, 2 M x 128, 4 M x 64 and 425 k x 602 boundary rows
+(``quant*``), a streaming copy (the attainable-bandwidth yardstick) and the CPU baselines timed on
+this machine's host cores.  Any of them can be made the headline of the line with --workload.
 
-Roofline objects: ``achieved`` is HBM-side bytes per launch of the dominant kernel (rocprofv3
-FETCH_SIZE + WRITE_SIZE, read from the ``traffic:`` lines of the summaries under profiles/) divided
-by that kernel's average duration, measured here with HIP events on the launch stream; ``frac`` is
-that over the 8 TB/s peak and is therefore at most 1.  The gather-model rate (algorithmic bytes,
-cache hits counted as if they were memory traffic; it can exceed the peak) is reported beside it as
-``gather_model``.  Without a measured traffic figure for the workload ``achieved``/``frac`` are null.
+Output.  stdout carries ONE JSON line of at most LINE_LIMIT bytes: the headline workload's contract
+fields with a flat ``roofline`` and ``cpu_baseline``, and in ``extra`` one flat record per other
+workload (``extra["workloads"]``) plus the int2 quantize+pack rate and roofline fraction as scalars.
+Everything nested (per-kernel times, plans, step rooflines, every roofline object in full) goes to
+stderr as one ``[bench-detail]`` JSON line and to gpurun_out/bench_detail.json.
 
-Prints ONE JSON line on stdout (everything else goes to stderr).
+Roofline objects.  SpMM kernels: ``achieved`` is HBM-side bytes per step of the dominant kernel
+(rocprofv3 FETCH_SIZE + WRITE_SIZE, read from the ``traffic:`` lines of the summaries under
+profiles/) divided by that kernel's time per step, measured here with HIP events on the launch
+stream; ``frac`` is that over the 8 TB/s peak and is therefore at most 1.  The gather-model rate
+(algorithmic bytes, cache hits counted as if they were memory traffic; it can exceed the peak) is
+beside it as ``gather_frac``.  A ``traffic:`` line names the plan shape it was measured on
+(``plan=``); when the running plan differs, or no line covers the workload, achieved / frac /
+traffic are null.  Quantizer kernels read and write every byte once, so their ``achieved`` is the
+algorithmic bytes over the kernel time and ``traffic`` the counter figure where one exists.
+
 """
 import argparse
 import glob
@@ -58,6 +65,7 @@ def load_measured_traffic():
                     "bytes": int(kv["fetch_bytes"]) + int(kv["write_bytes"]),
                     "fetch_bytes": int(kv["fetch_bytes"]), "write_bytes": int(kv["write_bytes"]),
                     "l2_hit": float(kv["l2_hit"]) if "l2_hit" in kv else None,
+                    "plan": kv.get("plan"),
                     "source": "profiles/" + os.path.basename(path)}
             except (KeyError, ValueError):
                 continue
@@ -67,18 +75,39 @@ def load_measured_traffic():
 TRAFFIC = load_measured_traffic()
 
 
-def roofline(workload, kernel, kernel_ms, algorithmic_bytes, launches_per_step=1):
-    """Roofline object of one kernel.  ``kernel_ms`` is per step (all launches of the kernel in one step)."""
+def plan_signature(**kv):
+    """The shape a kernel ran in, as the ``plan=`` token of a traffic line: "key:value,..." in sorted key order."""
+    return ",".join(f"{k}:{kv[k]}" for k in sorted(kv))
+
+
+def roofline(workload, kernel, kernel_ms, algorithmic_bytes, launches_per_step=1, plan=None):
+    """Roofline object of one kernel (flat).  ``kernel_ms`` is per step (all launches of the kernel in one step).
+    ``plan`` is the signature of the shape the kernel ran in now; a traffic figure measured on another shape
+    (its ``plan=`` token differs) is not used: achieved / frac / traffic are then null."""
     t = TRAFFIC.get((workload, kernel))
+    if t and plan is not None and t.get("plan") is not None and t["plan"] != plan:
+        log(f"[bench] WARNING: traffic of {kernel} on {workload} was measured on plan {t['plan']}, this run has {plan}: "
+            f"no roofline fraction is reported from it ({t['source']} needs a new counter run)")
+        t = None
     ach = t["bytes"] / kernel_ms / 1e6 if t else None
     gm = algorithmic_bytes / kernel_ms / 1e6
     return {"bound": "hbm", "achieved": round(ach, 1) if ach else None, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(ach / HBM_PEAK_GBPS, 4) if ach else None,
             "traffic": t["bytes"] if t else None, "traffic_source": t["source"] if t else None,
-            "l2_hit_rate": t["l2_hit"] if t else None,
-            "kernel": kernel, "kernel_ms_per_step": round(kernel_ms, 5), "launches_per_step": launches_per_step,
-            "gather_model": {"algorithmic_bytes": int(algorithmic_bytes), "GBps": round(gm, 1),
-                             "frac_of_peak": round(gm / HBM_PEAK_GBPS, 4)}}
+            "l2_hit": t["l2_hit"] if t else None,
+            "kernel": kernel, "kernel_ms": round(kernel_ms, 5), "launches": launches_per_step,
+            "algorithmic_bytes": int(algorithmic_bytes), "gather_GBps": round(gm, 1),
+            "gather_frac": round(gm / HBM_PEAK_GBPS, 4)}
+
+
+def streaming_roofline(workload, kernel, kernel_ms, algorithmic_bytes):
+    """Roofline object of a kernel that reads and writes every byte once (the quantizers): its algorithmic bytes
+    are its compulsory traffic, so ``achieved`` / ``frac`` are algorithmic bytes over time; ``traffic`` stays the
+    rocprofv3 figure (null where no counter run covers the workload) and ``traffic_frac`` its rate over the peak."""
+    r = roofline(workload, kernel, kernel_ms, algorithmic_bytes)
+    r["traffic_frac"] = r["frac"]
+    r["achieved"], r["frac"] = r["gather_GBps"], r["gather_frac"]
+    return r
 
 
 def step_roofline(workload, per_kernel_ms):
@@ -203,7 +232,7 @@ def cpu_baseline_spmm(rowptr, col, w, x, target_edges=1 << 40, reps=10):
     nnz = int(rp[m])
     rp_s = rp[: m + 1].contiguous()
     col_s = col[:nnz].to(torch.int64).cpu().contiguous()
-    w_s = w[:nnz].cpu().contiguous()
+    w_s = w[:nnz].cpu().contiguous() if w is not None else torch.ones(nnz)
     xh = x.cpu()
     F = xh.shape[1]
     out = torch.zeros(m, F)
@@ -228,6 +257,41 @@ def cpu_baseline_spmm(rowptr, col, w, x, target_edges=1 << 40, reps=10):
     t = float(np.median(ts))
     return {"value": nnz / t / 1e9, "unit": "GEdges/s", "cores": int(T), "host_cpu_count": os.cpu_count(), "kind": kind,
             "sample": f"{m} of {rp.numel() - 1} rows ({nnz} edges) of the same graph, full X, F={F}, 1 warm-up + median of {reps}",
+            "ms": t * 1e3}
+
+
+def cpu_baseline_prepost(rp_l, col_l, x_l, rp_r, col_r, q, prm, wr, bits, target_edges, reps=3):
+    """The CPU path of one pre/post-aggregation step on a row sample: unpack+dequantize ALL remote rows (the C
+    restatement: the reference's routine for it exists for SVE only), then the reference's accumulating SpMM over the
+    leading rows' local edges (gathering from the full local X) and over the same rows' remote edges (gathering
+    from the dequantized rows).  The dequantize time is charged in proportion to the sampled share of the edges."""
+    import numpy as np
+    import torch
+    from oracle import oracle as orc
+    F = x_l.shape[1]
+    qh, ph = q.cpu().numpy(), prm.cpu().numpy()
+    seg = wr.cpu().numpy().astype(np.int64)
+    orc.dequant_rows(qh, ph, seg, bits, F)
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        recv = orc.dequant_rows(qh, ph, seg, bits, F)
+        ts.append(time.perf_counter() - t0)
+    t_dq = float(np.median(ts))
+    recv_d = torch.from_numpy(recv)
+    rp = rp_l.cpu()
+    m = int(torch.searchsorted(rp, torch.tensor(target_edges)).item())
+    m = max(1, min(m, rp.numel() - 1))
+    loc = cpu_baseline_spmm(rp_l[: m + 1], col_l, None, x_l, reps=reps)
+    rem = cpu_baseline_spmm(rp_r[: m + 1], col_r, None, recv_d, reps=reps)
+    nl, nr = int(rp_l[m]), int(rp_r[m])
+    share = (nl + nr) / float(col_l.numel() + col_r.numel())
+    t = (loc["ms"] + rem["ms"]) * 1e-3 + share * t_dq
+    return {"value": (nl + nr) / t / 1e9, "unit": "GEdges/s", "cores": loc["cores"], "host_cpu_count": os.cpu_count(),
+            "kind": loc["kind"],
+            "sample": f"{m} of {rp.numel() - 1} rows ({nl} local + {nr} remote edges), full local X; SpMM legs: {loc['kind']}; "
+                      f"dequantize of all remote rows {t_dq * 1e3:.0f} ms (C port, {orc.num_threads()} threads) charged at the "
+                      f"sampled edge share {share:.3f}; median of {reps}",
             "ms": t * 1e3}
 
 
@@ -292,7 +356,8 @@ def wl_copy(args, ctx):
             "config": {"workload": "stream_copy_1GiB"}, "ms_per_step": ms, "dtype": "f32",
             "roofline": {"bound": "hbm", "achieved": round(b / k_ms / 1e6, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": round(b / k_ms / 1e6 / HBM_PEAK_GBPS, 4), "traffic": b, "traffic_source": "by construction",
-                         "kernel": "stream_copy_kernel", "kernel_ms_per_step": round(k_ms, 5)},
+                         "kernel": "stream_copy_kernel", "kernel_ms": round(k_ms, 5),
+                         "gather_GBps": round(b / k_ms / 1e6, 1), "gather_frac": round(b / k_ms / 1e6 / HBM_PEAK_GBPS, 4)},
             "cpu_baseline": None, "extra": {}}
 
 
@@ -316,8 +381,8 @@ def quant_case(ops, x, bits, steps, warmup, segments=1):
     kq_ms, kd_ms = kq["quant_pack_rows_kernel"], kd["unpack_dequant_rows_kernel"]
     return {"workload": wl, "bytes": b, "quant_ms": ms_q, "dequant_ms": ms_d,
             "quant_GBps_wall": round(b / ms_q / 1e6, 1), "dequant_GBps_wall": round(b / ms_d / 1e6, 1),
-            "quant_roofline": roofline(wl, "quant_pack_rows_kernel", kq_ms, b),
-            "dequant_roofline": roofline(wl.replace("quant_pack", "unpack_dequant"), "unpack_dequant_rows_kernel", kd_ms, b)}
+            "quant_roofline": streaming_roofline(wl, "quant_pack_rows_kernel", kq_ms, b),
+            "dequant_roofline": streaming_roofline(wl.replace("quant_pack", "unpack_dequant"), "unpack_dequant_rows_kernel", kd_ms, b)}
 
 
 def wl_quant(args, ctx, rows=None, feat=None, headline=True):
@@ -330,9 +395,9 @@ def wl_quant(args, ctx, rows=None, feat=None, headline=True):
             continue
         c = quant_case(ops, xq, bits, args.steps if (headline and bits == args.bits) else 10, args.warmup if headline else 3)
         cases[bits] = c
-        log(f"[bench] {n}x{F} int{bits}: quantize+pack kernel {c['quant_roofline']['gather_model']['GBps']:.0f} GB/s "
-            f"({c['quant_roofline']['kernel_ms_per_step'] * 1e3:.1f} us), unpack+dequant kernel "
-            f"{c['dequant_roofline']['gather_model']['GBps']:.0f} GB/s ({c['dequant_roofline']['kernel_ms_per_step'] * 1e3:.1f} us)")
+        log(f"[bench] {n}x{F} int{bits}: quantize+pack kernel {c['quant_roofline']['gather_GBps']:.0f} GB/s "
+            f"({c['quant_roofline']['kernel_ms'] * 1e3:.1f} us), unpack+dequant kernel "
+            f"{c['dequant_roofline']['gather_GBps']:.0f} GB/s ({c['dequant_roofline']['kernel_ms'] * 1e3:.1f} us)")
     main = cases[args.bits]
     cpu_port = cpu_ref = None
     if not args.no_cpu:
@@ -340,12 +405,7 @@ def wl_quant(args, ctx, rows=None, feat=None, headline=True):
     extra = {f"int{b}": {k: v for k, v in c.items() if k != "workload"} for b, c in cases.items()}
     if cpu_ref is not None:
         extra["cpu_port"] = cpu_port
-    # the quantizer's algorithmic bytes ARE its compulsory traffic (one read, one write): the roofline fraction of
-    # a kernel without a traffic figure falls back to them
     rf = main["quant_roofline"]
-    if rf["achieved"] is None:
-        rf = dict(rf, achieved=rf["gather_model"]["GBps"], frac=rf["gather_model"]["frac_of_peak"],
-                  traffic_source="algorithmic bytes (one read + one write per element; no reuse to credit)")
     return {"metric": f"quantize-pack GB/s at int{args.bits}", "value": round(main["bytes"] / main["quant_ms"] / 1e6, 2),
             "unit": "GB/s", "config": {"workload": main["workload"], "rows": n, "F": F, "bits": args.bits},
             "ms_per_step": main["quant_ms"], "dtype": "f32->u8", "roofline": rf,
@@ -438,7 +498,9 @@ def wl_rmat(args, ctx):
             "value": round(nnz / ms / 1e6, 4), "unit": "GEdges/s",
             "config": {"workload": wl, "nodes": M, "edges": nnz, "F": F, "aggregation": "weighted_sum",
                        "accumulate": True, "index_dtype": "int32"},
-            "ms_per_step": ms, "dtype": "f32", "roofline": roofline(wl, dom, per_kernel[dom], dom_bytes, launches[dom]),
+            "ms_per_step": ms, "dtype": "f32",
+            "roofline": roofline(wl, dom, per_kernel[dom], dom_bytes, launches[dom],
+                                 plan=plan_signature(pieces=info["pieces"], long_rows=info["long_rows"])),
             "cpu_baseline": None if args.no_cpu else cpu_baseline_spmm(rowptr, col, w, x), "extra": extra}
 
 
@@ -529,6 +591,10 @@ def wl_prepost(args, ctx):
     info_r = plan_r.info()
     dom_edges = info_r["long_edges"] if "piece" in dom else nr - info_r["long_edges"]
     dom_bytes = dom_edges * (F + 16)  # per remote edge: one packed row of F bytes + params + col/val
+    # the remote edge list is de-duplicated from a device-side draw and differs by a few edges from run to run,
+    # so the signature holds the plan's shape parameters rather than its counts
+    sig = plan_signature(long_row_threshold=info_r["long_row_threshold"], piece_edges=info_r["piece_edges"],
+                         partitioned=info_r["partitioned"])
     total = ms_local + ms_fused
     # named by the requested sizes: the de-duplicated remote edge count varies by a few edges from run to run
     wl = f"prepost_{Ml}n_{args.local_und_edges}ue_local_{Kr}c_{args.remote_edges}e_remote_int{bits}_F{F}"
@@ -543,7 +609,9 @@ def wl_prepost(args, ctx):
     return {"metric": "SpMM GEdges/s, pre/post-aggregation partition (local fp32 + int2-packed remote rows, fused)",
             "value": round((nl + nr) / total / 1e6, 4), "unit": "GEdges/s",
             "config": {"workload": wl, "F": F, "bits": bits, "local_edges": nl, "remote_edges": nr}, "ms_per_step": total, "dtype": "f32",
-            "roofline": roofline(wl, dom, k_fused[dom], dom_bytes, launches[dom]), "cpu_baseline": None, "extra": extra}
+            "roofline": roofline(wl, dom, k_fused[dom], dom_bytes, launches[dom], plan=sig),
+            "cpu_baseline": None if args.no_cpu else cpu_baseline_prepost(rp_l, col_l, x_l, rp_r, col_r, q, prm, wr, bits,
+                                                                          args.cpu_sample_edges), "extra": extra}
 
 
 def wl_quant_widths(args, ctx):
@@ -560,10 +628,10 @@ def wl_quant_widths(args, ctx):
         row = {}
         for bits in (8, 4, 2):
             c = quant_case(ops, x, bits, max(args.steps, 5), max(args.warmup, 2), segments=args.segments)
-            row[f"int{bits}"] = {"quant_us": round(c["quant_roofline"]["kernel_ms_per_step"] * 1e3, 1),
-                                 "quant_GBps": c["quant_roofline"]["gather_model"]["GBps"],
-                                 "dequant_us": round(c["dequant_roofline"]["kernel_ms_per_step"] * 1e3, 1),
-                                 "dequant_GBps": c["dequant_roofline"]["gather_model"]["GBps"]}
+            row[f"int{bits}"] = {"quant_us": round(c["quant_roofline"]["kernel_ms"] * 1e3, 1),
+                                 "quant_GBps": c["quant_roofline"]["gather_GBps"],
+                                 "dequant_us": round(c["dequant_roofline"]["kernel_ms"] * 1e3, 1),
+                                 "dequant_GBps": c["dequant_roofline"]["gather_GBps"]}
         table[str(F)] = row
         log(f"[bench] F={F:5d} rows={n:9d}  quantize+pack GB/s int8/4/2: " + " / ".join(f"{row[f'int{b}']['quant_GBps']:6.0f}" for b in (8, 4, 2)) +
             "   unpack+dequantize GB/s: " + " / ".join(f"{row[f'int{b}']['dequant_GBps']:6.0f}" for b in (8, 4, 2)))
@@ -632,7 +700,9 @@ def wl_sbm(args, ctx):
         extra["packed_operand"] = fused
     return {"metric": f"SpMM GEdges/s (dense-degree community graph, F={F} fp32)", "value": round(nnz / ms / 1e6, 4),
             "unit": "GEdges/s", "config": {"workload": wl, "F": F}, "ms_per_step": ms, "dtype": "f32",
-            "roofline": roofline(wl, dom, per_kernel[dom], dom_bytes, launches[dom]), "cpu_baseline": None, "extra": extra}
+            "roofline": roofline(wl, dom, per_kernel[dom], dom_bytes, launches[dom], plan=plan_signature(**sched)),
+            "cpu_baseline": None if args.no_cpu else cpu_baseline_spmm(rowptr, col, None, x, target_edges=args.cpu_sample_edges, reps=3),
+            "extra": extra}
 
 
 def wl_aggregate(args, ctx):
@@ -712,11 +782,73 @@ WORKLOADS = {"rmat": wl_rmat, "quant": wl_quant, "quant_widths": wl_quant_widths
              "aggregate": wl_aggregate, "sage": wl_sage, "small": wl_small}
 
 
-def brief(r):
-    """A workload's result as an entry of extra["workloads"]."""
-    return {"metric": r["metric"], "value": r["value"], "unit": r["unit"], "config": r["config"],
-            "ms_per_step": round(r["ms_per_step"], 5), "roofline": r["roofline"], "cpu_baseline": r["cpu_baseline"],
-            "extra": r["extra"]}
+def _r(v, nd=4):
+    return round(v, nd) if isinstance(v, float) else v
+
+
+def compact_record(r):
+    """One workload as ONE flat record of the printed line: scalars only."""
+    rf, cpu = r.get("roofline") or {}, r.get("cpu_baseline") or {}
+    rec = {"value": _r(r["value"], 3), "unit": r["unit"], "ms_per_step": _r(float(r["ms_per_step"]), 4),
+           "kernel": rf.get("kernel"), "kernel_ms": _r(rf.get("kernel_ms")), "frac": rf.get("frac"),
+           "gather_frac": rf.get("gather_frac"), "cpu": _r(cpu.get("value"), 4), "cpu_kind": cpu.get("kind")}
+    return {k: v for k, v in rec.items() if v is not None}
+
+
+def quant_records(name, r):
+    """The quantizer workload: one flat record per code width (quantize+pack and unpack+dequantize kernels)."""
+    out = {}
+    for key, c in r["extra"].items():
+        if not key.startswith("int"):
+            continue
+        q, d = c["quant_roofline"], c["dequant_roofline"]
+        rec = {"q_GBps": q["gather_GBps"], "q_frac": q["frac"], "q_traffic_frac": q["traffic_frac"],
+               "dq_GBps": d["gather_GBps"], "dq_frac": d["frac"]}
+        out[f"{name}_{key}"] = {k: v for k, v in rec.items() if v is not None}
+    return out
+
+
+LINE_LIMIT = 4000   # bytes; the harness that reads the line keeps only a bounded tail of stdout
+
+
+def build_line(result, others, steps, warmup):
+    """The ONE JSON line of stdout, from the headline workload's result and the other workloads' results
+    (name -> result dict).  Everything nested (per-kernel tables, plans, per-width rooflines) stays out of it:
+    main() writes that to stderr and to gpurun_out/bench_detail.json."""
+    rf = dict(result["roofline"] or {})
+    for k in ("traffic_source", "algorithmic_bytes", "launches", "gather_GBps", "traffic_frac"):
+        rf.pop(k, None)
+    cpu = result["cpu_baseline"]
+    if cpu is not None:
+        cpu = {"value": _r(float(cpu["value"]), 4), "unit": cpu["unit"], "cores": cpu["cores"], "kind": cpu["kind"],
+               "sample": cpu["sample"]}
+    extra = {}
+    for k, v in (result.get("extra") or {}).items():
+        if isinstance(v, (int, float, str, bool)) or v is None:
+            extra[k] = _r(v)
+    workloads = {}
+    for name, r in others.items():
+        if name.startswith("quant"):
+            workloads.update(quant_records(name, r))
+        else:
+            workloads[name] = compact_record(r)
+    q2 = workloads.get("quant_int2")
+    if q2:   # the second half of the metric, as scalars of its own
+        extra["quant_pack_int2_GBps"], extra["quant_pack_int2_frac"] = q2["q_GBps"], q2["q_frac"]
+        extra["quant_pack_int2_config"] = others["quant"]["config"]["workload"]
+    if workloads:
+        extra["workloads"] = workloads
+    line = {"metric": result["metric"], "value": _r(float(result["value"])), "unit": result["unit"], "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": round(float(result["ms_per_step"]), 5),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": result["dtype"],
+            "data": "synthetic", "config": result["config"], "roofline": rf or None, "cpu_baseline": cpu, "extra": extra}
+    text = json.dumps(line, separators=(",", ":"))
+    if len(text) > LINE_LIMIT:   # never print a line the harness cannot hold: drop the per-workload records first
+        log(f"[bench] WARNING: line of {len(text)} bytes exceeds {LINE_LIMIT}; per-workload records dropped from it")
+        extra.pop("workloads", None)
+        text = json.dumps(line, separators=(",", ":"))
+    assert len(text) <= LINE_LIMIT, len(text)
+    return text
 
 
 def main():
@@ -759,6 +891,8 @@ def main():
     ap.add_argument("--piece-edges", type=int, default=0, help="SpMM plan: minimum edges per long-row piece (0 = default)")
     ap.add_argument("--no-extras", action="store_true", help="only the chosen workload (used under rocprofv3)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--cpu-sample-edges", type=int, default=16_000_000,
+                    help="sbm / prepost: the CPU baseline runs the leading rows holding about this many edges")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this build runs one partition on ONE GPU; there is no multi-GPU path to time "
@@ -773,9 +907,8 @@ def main():
     ctx = {"dev": torch.device("cuda:0"), "stream": ops._stream}
 
     result = WORKLOADS[args.workload](args, ctx)
-    extra = result.pop("extra")
+    others = {}
     if not args.no_extras:
-        others = {}
         saved = (args.steps, args.warmup)
         args.steps, args.warmup = min(args.steps, 10), min(args.warmup, 3)
         for name in ("copy", "quant", "sbm", "prepost", "small"):
@@ -783,29 +916,36 @@ def main():
                 continue
             torch.cuda.empty_cache()
             t0 = time.perf_counter()
-            cpu_saved = args.no_cpu
-            args.no_cpu = args.no_cpu or name in ("sbm", "prepost")
-            others[name] = brief(WORKLOADS[name](args, ctx))
+            others[name] = WORKLOADS[name](args, ctx)
             if name == "quant":   # the narrow rows the live path exchanges (F = 128, 64): more rows for the same bytes;
                 torch.cuda.empty_cache()
-                others["quant_F128"] = brief(wl_quant(args, ctx, rows=2 * args.quant_rows, feat=128, headline=False))
+                others["quant_F128"] = wl_quant(args, ctx, rows=2 * args.quant_rows, feat=128, headline=False)
                 torch.cuda.empty_cache()
-                others["quant_F64"] = brief(wl_quant(args, ctx, rows=4 * args.quant_rows, feat=64, headline=False))
+                others["quant_F64"] = wl_quant(args, ctx, rows=4 * args.quant_rows, feat=64, headline=False)
                 torch.cuda.empty_cache()  # rows that do not start on cache lines: the dense-degree graph's feature width
-                others["quant_F602"] = brief(wl_quant(args, ctx, rows=425_000 * args.quant_rows // 1_000_000, feat=602, headline=False))
-            args.no_cpu = cpu_saved
+                others["quant_F602"] = wl_quant(args, ctx, rows=425_000 * args.quant_rows // 1_000_000, feat=602, headline=False)
             log(f"[bench] extra workload {name}: {time.perf_counter() - t0:.1f}s")
         args.steps, args.warmup = saved
-        extra["workloads"] = others
         if "copy" in others:
-            extra["stream_copy_GBps"] = others["copy"]["value"]
+            result["extra"]["stream_copy_GBps"] = others["copy"]["value"]
 
-    line = {"metric": result["metric"], "value": result["value"], "unit": result["unit"], "n_gpus": 1,
-            "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(result["ms_per_step"], 5),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": result["dtype"],
-            "data": "synthetic", "config": result["config"], "roofline": result["roofline"],
-            "cpu_baseline": result["cpu_baseline"], "extra": extra}
-    print(json.dumps(line), flush=True)
+    detail = {"headline": result, "workloads": others}
+    text = json.dumps(detail)
+    log("[bench-detail] " + text)
+    try:   # the same detail as a file, where the run has a results folder
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "bench_detail.json"), "w") as f:
+            f.write(text + "\n")
+    except OSError:
+        pass
+    sys.stderr.flush()
+    print(build_line(result, others, args.steps, args.warmup), flush=True)
+    sys.stdout.flush()
+    if not any(k.startswith(("ROCPROF", "ROCP_")) for k in os.environ) and "rocprof" not in os.environ.get("LD_PRELOAD", ""):
+        # leave at once: interpreter teardown would otherwise spend seconds returning tens of GB of device memory
+        # and joining the CPU legs' OpenMP pools after the line is out.  Under rocprofv3 the normal exit runs, since
+        # the profiler writes its output from exit handlers.
+        os._exit(0)
 
 
 if __name__ == "__main__":
