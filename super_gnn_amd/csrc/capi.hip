@@ -32,8 +32,8 @@ static std::mutex g_prof_mu;
 static std::atomic<bool> g_prof_on{false};
 static std::vector<ProfRecord> g_prof;
 
-ProfScope::ProfScope(int id, hipStream_t st) : id_(id), st_(st) {
-    if (!g_prof_on) return;
+ProfScope::ProfScope(int id, hipStream_t st, bool enabled) : id_(id), st_(st) {
+    if (!enabled || !g_prof_on) return;
     if (hipEventCreate(&start_) != hipSuccess) { start_ = nullptr; return; }
     (void)hipEventRecord(start_, st_);
 }

@@ -50,7 +50,8 @@ enum KernelId {
 // Records a HIP event pair around the launches made while it is alive, on the launch stream,
 // when profiling is enabled; free otherwise.
 struct ProfScope {
-    ProfScope(int id, hipStream_t st);
+    // enabled = false: never records (callers that must not create events, e.g. under graph capture)
+    ProfScope(int id, hipStream_t st, bool enabled = true);
     ~ProfScope();
     int id_;
     hipStream_t st_;

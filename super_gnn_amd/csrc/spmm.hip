@@ -1086,6 +1086,7 @@ struct ShortArgs {
     const int64_t *rowptr; const int32_t *col; const float *val; DenseSrc dense; float *out;
     const int4 *chunks; int n_chunks; const int32_t *empty_rows; int n_empty;
     int F; int64_t ldo; int accumulate; const float *row_div;
+    bool prof;   // false: no profiling events (the non-allocating entry point creates nothing)
 };
 struct PieceArgs {
     const int32_t *col_long; const int32_t *eperm; const float *val; float *partial;
@@ -1112,14 +1113,14 @@ static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &
     const char *hub_env = getenv("SGNN_SPMM_HUB_LDS");
     const bool hub_lds = hub_env != nullptr && atoi(hub_env) != 0;
     if (BITS == 0 && hub_lds && f.n_long > 0) {
-        ProfScope prof(K_SPMM_PIECE, ls);
+        ProfScope prof(K_SPMM_PIECE, ls, a.prof);
         hipLaunchKernelGGL((spmm_hubrow_lds_kernel<VEC, G, NV>), dim3((uint32_t)f.n_long), dim3(kBlock), 0, ls, a.rowptr, a.col, a.val,
                            a.dense, f.long_rows, f.out, f.F, f.ldo, f.accumulate, f.row_div);
     } else if (f.n_long > 0) {
         {
             // workgroup i serves class i % 8: grid = 8 * (workgroups of the fullest class)
             const uint32_t nb = (uint32_t)kNumXCD * (uint32_t)((s.max_cls_items + GPB - 1) / GPB);
-            ProfScope prof(BITS == 0 ? K_SPMM_PIECE : K_FUSED_PIECE, ls);
+            ProfScope prof(BITS == 0 ? K_SPMM_PIECE : K_FUSED_PIECE, ls, a.prof);
             if (s.eperm)
                 hipLaunchKernelGGL((spmm_piece_kernel<VEC, G, NV, BITS, true>), dim3(nb), dim3(kBlock), 0, ls, s.col_long,
                                    s.eperm, s.val, a.dense, s.partial, s.cls_work, s.max_cls_items, s.F);
@@ -1128,19 +1129,19 @@ static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &
                                    s.eperm, s.val, a.dense, s.partial, s.cls_work, s.max_cls_items, s.F);
         }
         const uint32_t nb = (uint32_t)((f.n_long + GPB - 1) / GPB);
-        ProfScope prof(K_SPMM_LONG_FINAL, ls);
+        ProfScope prof(K_SPMM_LONG_FINAL, ls, a.prof);
         hipLaunchKernelGGL((spmm_long_final_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, ls, f.long_rows,
                            f.long_pbeg, f.partial, f.out, f.n_long, f.F, f.ldo, f.accumulate, f.row_div);
     }
     if (a.n_chunks > 0) {
         const uint32_t nb = (uint32_t)((a.n_chunks + GPB - 1) / GPB);
-        ProfScope prof(BITS == 0 ? K_SPMM_SHORT : K_FUSED_SHORT, st);
+        ProfScope prof(BITS == 0 ? K_SPMM_SHORT : K_FUSED_SHORT, st, a.prof);
         hipLaunchKernelGGL((spmm_short_kernel<VEC, G, NV, BITS>), dim3(nb), dim3(kBlock), 0, st, a.rowptr, a.col, a.val,
                            a.dense, a.out, a.chunks, a.n_chunks, a.F, a.ldo, a.accumulate, a.row_div, nb);
     }
     if (a.n_empty > 0 && (!a.accumulate || a.row_div)) {
         const uint32_t nb = (uint32_t)((a.n_empty + GPB * kEmptyRowsPerGroup - 1) / (GPB * kEmptyRowsPerGroup));
-        ProfScope prof(K_SPMM_EMPTY_ROWS, st);
+        ProfScope prof(K_SPMM_EMPTY_ROWS, st, a.prof);
         hipLaunchKernelGGL((spmm_empty_rows_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, a.empty_rows, a.n_empty,
                            a.out, a.F, a.ldo, a.accumulate, a.row_div);
     }
@@ -1248,6 +1249,7 @@ struct BandSchedule {
     int32_t *eperm_bm = nullptr;       // [nnz] CSR index of each band-major edge
     float *val_bm = nullptr;           // [nnz] edge values in band-major order
     uint64_t val_gen = 0;              // plan bind generation val_bm was filled under (0 = not from a bound array)
+    uint64_t last_use = 0;             // the plan's band_use_clock at this schedule's last product
     int64_t M = 0, K = 0;
     std::vector<int32_t> h_rowptr_bm;  // host: [n_bands * (M+1)] where each (band, row) starts in the band-major arrays
     // The bands cut into chunks, for one pair of limits (rows, edges per chunk); a launch picks the limits from
@@ -1306,6 +1308,7 @@ struct sgnn_spmm_plan {
     uint64_t call_serial = 0;          // products run on this (whole) plan so far
     uint64_t xs_serial = 0;            // the product whose dense operand band_xs holds ...
     int xs_F = 0, xs_slice_pad = 0, xs_slices = 0;  // ... and in which slice layout
+    uint64_t band_use_clock = 0;       // counts band-schedule products (least-recently-used eviction of schedules)
     // Short-row chunks, one list per chunk row limit (7, 15, 31).
     std::vector<int64_t> h_rowptr;
     int4 *chunks[3] = {nullptr, nullptr, nullptr};
@@ -1659,26 +1662,74 @@ struct BandShape {
     int slice_pad;     // floats per restaged slice row (a multiple of 16: rows on 64-byte boundaries)
     int G;             // lanes per group: slice_pad / 4, at least 16, at most 64 (wider slices are walked in tiles)
     int band_cols, n_bands;
+    int f0, F;         // the feature columns [f0, f0 + F) of the product this shape covers (one window)
+    size_t xs_off;     // where this window's restaged operand starts in the workspace, in floats
 };
 
-// How a product of feature width F would be cut into feature slices and column bands.
-static BandShape band_shape(const sgnn_spmm_plan *p, int64_t F, bool even_out) {
+// Feature columns per window of a wide product.  Slices of exactly 64 floats are the band kernel's most efficient
+// shape (a wavefront instruction carries four gathers of 256 bytes, every lane busy), and a window of 512 columns
+// is eight of them, one per XCD.  Wider products run as consecutive windows over the same bands: the reference
+// tiles the feature axis of every row in the same way (spmm.cpp:502-510).
+constexpr int kBandWindowCols = 512;
+constexpr int kMaxBandSchedules = 3;   // band widths a plan keeps schedules for (each holds ~12 bytes per edge)
+constexpr int kBandMaxWindows = 64;
+
+// How a product of feature width F is cut into feature windows, slices and column bands.  Products of up to
+// kBandWindowCols columns are one window whose slices share the eight XCDs evenly.  Wider products take windows
+// of kBandWindowCols columns and a remainder window with slices of at most 64 floats; every window uses the
+// bands of a 64-float slice, so one band-major copy of the edges serves them all.
+struct BandWindows {
+    int n = 0;
+    BandShape w[kBandMaxWindows];
+    size_t xs_floats = 0;   // restaged operand of all windows
+    int total_slices = 0;
+};
+
+static BandShape band_window_shape(const sgnn_spmm_plan *p, int f0, int Fw, bool even_out, bool windowed) {
     BandShape b{};
-    b.even = even_out && F % 2 == 0 && F >= 4;
-    const int nvec = (int)((F + 3) / 4);
-    b.n_slices = kNumXCD;
-    while (b.n_slices > 1 && (nvec + b.n_slices - 1) / b.n_slices < 16) b.n_slices /= 2;
-    const int forced = env_int("SGNN_SPMM_BAND_SLICES", 0);
-    if (forced == 1 || forced == 2 || forced == 4 || forced == 8) b.n_slices = forced;
+    b.f0 = f0;
+    b.F = Fw;
+    b.even = even_out && Fw % 2 == 0 && Fw >= 4 && f0 % 2 == 0;
+    const int nvec = (Fw + 3) / 4;
+    if (windowed) {   // at most 16 float4 per slice
+        b.n_slices = 1;
+        while (b.n_slices < kNumXCD && (nvec + b.n_slices - 1) / b.n_slices > 16) b.n_slices *= 2;
+    } else {
+        b.n_slices = kNumXCD;
+        while (b.n_slices > 1 && (nvec + b.n_slices - 1) / b.n_slices < 16) b.n_slices /= 2;
+        const int forced = env_int("SGNN_SPMM_BAND_SLICES", 0);
+        if (forced == 1 || forced == 2 || forced == 4 || forced == 8) b.n_slices = forced;
+    }
     b.slice_floats = 4 * ((nvec + b.n_slices - 1) / b.n_slices);
     b.slice_pad = (b.slice_floats + 15) / 16 * 16;
     b.G = std::max(16, std::min(64, b.slice_pad / 4));
     int cols = env_int("SGNN_SPMM_BAND_COLS", 0);
-    if (cols <= 0)
-        cols = (int)std::max<int64_t>(256, (int64_t)env_int("SGNN_SPMM_BAND_KB", kBandL2BudgetKB) * 1024 / (b.slice_pad * 4) / 256 * 256);
+    if (cols <= 0) {
+        const int pad = windowed ? 64 : b.slice_pad;   // windows share the bands of a full 64-float slice
+        cols = (int)std::max<int64_t>(256, (int64_t)env_int("SGNN_SPMM_BAND_KB", kBandL2BudgetKB) * 1024 / (pad * 4) / 256 * 256);
+    }
     b.band_cols = cols;
     b.n_bands = (int)std::max<int64_t>(1, (p->K + cols - 1) / cols);
     return b;
+}
+
+static BandWindows band_windows(const sgnn_spmm_plan *p, int64_t F, bool even_out) {
+    BandWindows bw;
+    const int win = env_int("SGNN_SPMM_BAND_WINDOW", kBandWindowCols);   // 0 = never cut a product into windows
+    const bool windowed = win >= 64 && win % 64 == 0 && F > win && (F + win - 1) / win <= kBandMaxWindows;
+    if (!windowed) {
+        bw.n = 1;
+        bw.w[0] = band_window_shape(p, 0, (int)F, even_out, false);
+    } else {
+        for (int64_t f0 = 0; f0 < F; f0 += win)
+            bw.w[bw.n++] = band_window_shape(p, (int)f0, (int)std::min<int64_t>(win, F - f0), even_out, true);
+    }
+    for (int i = 0; i < bw.n; ++i) {
+        bw.w[i].xs_off = bw.xs_floats;
+        bw.xs_floats += (size_t)bw.w[i].n_slices * (size_t)p->K * (size_t)bw.w[i].slice_pad;
+        bw.total_slices += bw.w[i].n_slices;
+    }
+    return bw;
 }
 
 // Whether the band schedule is the one to use: the dense operand does not fit the caches, and every row has
@@ -1757,6 +1808,25 @@ static int band_build_chunks(BandSchedule *bs, int rows_cap, int edge_cap, hipSt
     return SGNN_OK;
 }
 
+// Device allocations of the band schedule: running out of memory is not an error of the product (the row-class
+// schedule needs none of this), so it is told apart from other failures.
+static thread_local bool g_band_oom = false;
+static bool band_build_out_of_memory() {
+    const bool r = g_band_oom;
+    g_band_oom = false;
+    return r;
+}
+#define SGNN_BAND_ALLOC(pp, bytes)                                                             \
+    do {                                                                                       \
+        const hipError_t _me = hipMalloc((pp), (bytes));                                       \
+        if (_me == hipErrorOutOfMemory) {                                                      \
+            (void)hipGetLastError();                                                           \
+            g_band_oom = true;                                                                 \
+            return ::sgnn::fail(SGNN_ERR_HIP, "band schedule: out of device memory");          \
+        }                                                                                      \
+        SGNN_HIP_CHECK(_me);                                                                   \
+    } while (0)
+
 static int band_build(sgnn_spmm_plan *p, int band_cols, int n_bands, hipStream_t st, BandSchedule **out) {
     const int64_t M = p->M, nnz = p->nnz;
     std::unique_ptr<BandSchedule> bs(new BandSchedule());
@@ -1768,8 +1838,8 @@ static int band_build(sgnn_spmm_plan *p, int band_cols, int n_bands, hipStream_t
                  "band schedule too large (%d bands x %lld rows)", n_bands, (long long)M);
     DevTmp<int32_t> lo, cnt_t;
     const int64_t n_lo = M * ((int64_t)n_bands + 1), n_cnt = M * (int64_t)n_bands;
-    SGNN_HIP_CHECK(hipMalloc(&lo.p, sizeof(int32_t) * (size_t)n_lo));
-    SGNN_HIP_CHECK(hipMalloc(&cnt_t.p, sizeof(int32_t) * (size_t)n_cnt));
+    SGNN_BAND_ALLOC(&lo.p, sizeof(int32_t) * (size_t)n_lo);
+    SGNN_BAND_ALLOC(&cnt_t.p, sizeof(int32_t) * (size_t)n_cnt);
     hipLaunchKernelGGL(band_bounds_kernel, dim3((uint32_t)((n_lo + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, p->rowptr, p->col, M,
                        n_bands, band_cols, lo.p);
     hipLaunchKernelGGL(band_counts_kernel, dim3((uint32_t)((n_cnt + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, lo.p, M, n_bands,
@@ -1791,13 +1861,13 @@ static int band_build(sgnn_spmm_plan *p, int band_cols, int n_bands, hipStream_t
     }
     if (run != nnz) return fail(SGNN_ERR_RANGE, "band schedule: %lld of %lld edges fall into the bands", (long long)run, (long long)nnz);
     DevTmp<int32_t> rowptr_bm;   // [n_bands * (M+1)] where each (band, row) starts in the band-major arrays
-    SGNN_HIP_CHECK(hipMalloc(&rowptr_bm.p, sizeof(int32_t) * rp.size()));
+    SGNN_BAND_ALLOC(&rowptr_bm.p, sizeof(int32_t) * rp.size());
     SGNN_HIP_CHECK(hipMemcpyAsync(rowptr_bm.p, rp.data(), sizeof(int32_t) * rp.size(), hipMemcpyHostToDevice, st));
     // the kernel reads up to kBandPad + 3 entries past a chunk's last pair: zero entries (column 0) close the arrays
     const size_t tail = (size_t)kBandPad + 4;
-    SGNN_HIP_CHECK(hipMalloc(&bs->col_bm, sizeof(int32_t) * ((size_t)nnz + tail)));
-    SGNN_HIP_CHECK(hipMalloc(&bs->eperm_bm, sizeof(int32_t) * (size_t)nnz));
-    SGNN_HIP_CHECK(hipMalloc(&bs->val_bm, sizeof(float) * ((size_t)nnz + tail)));
+    SGNN_BAND_ALLOC(&bs->col_bm, sizeof(int32_t) * ((size_t)nnz + tail));
+    SGNN_BAND_ALLOC(&bs->eperm_bm, sizeof(int32_t) * (size_t)nnz);
+    SGNN_BAND_ALLOC(&bs->val_bm, sizeof(float) * ((size_t)nnz + tail));
     SGNN_HIP_CHECK(hipMemsetAsync(bs->col_bm + nnz, 0, sizeof(int32_t) * tail, st));
     SGNN_HIP_CHECK(hipMemsetAsync(bs->val_bm + nnz, 0, sizeof(float) * tail, st));
     hipLaunchKernelGGL(band_scatter_kernel, dim3((uint32_t)((M + 15) / 16)), dim3(kBlock), 0, st, p->rowptr, p->col, M, n_bands,
@@ -1830,13 +1900,13 @@ static BandCaps band_chunk_caps(const sgnn_spmm_plan *p, const BandShape &sh, bo
     edges = std::max(edges, 16);
     const int er = env_int("SGNN_SPMM_BAND_CHUNK_ROWS", 0), ee = env_int("SGNN_SPMM_BAND_CHUNK_EDGES", 0);
     if (er > 0) rows = std::min(er, rows_max);
-    if (ee > 0) edges = std::min(ee, edges_lim);
+    if (ee > 0) edges = std::max(16, std::min(ee, edges_lim) / 16 * 16);   // the next group's float4 tile starts right behind the staged edges
     return BandCaps{rows, edges};
 }
 
 template <bool EVEN, bool WEIGHTED>
 static int launch_band(const BandSchedule *bs, const BandSchedule::ChunkList *cl, const BandShape &sh, int b, const float *val_bm,
-                       const float *xs, float *out, int F, int64_t ldo, hipStream_t st, int device) {
+                       const float *xs, float *out, int64_t ldo, hipStream_t st, int device) {
     const int64_t c0 = cl->chunk_off[(size_t)b], c1 = cl->chunk_off[(size_t)b + 1];
     if (c1 == c0) return SGNN_OK;
     const int gpb = (kBandBlock / 64) * (64 / sh.G);  // lane groups per workgroup
@@ -1859,8 +1929,9 @@ static int launch_band(const BandSchedule *bs, const BandSchedule::ChunkList *cl
             allowed = lds;
         }
     }
-    hipLaunchKernelGGL(kernel, dim3(nb), dim3(kBandBlock), lds, st, bs->col_bm, val_bm, xs, bs->K, out, cl->chunks + 4 * c0,
-                       (int)(c1 - c0), F, ldo, sh.slice_floats, sh.slice_pad, sh.n_slices, sh.G, cl->rows_cap, cl->edge_cap);
+    hipLaunchKernelGGL(kernel, dim3(nb), dim3(kBandBlock), lds, st, bs->col_bm, val_bm, xs + sh.xs_off, bs->K, out + sh.f0,
+                       cl->chunks + 4 * c0, (int)(c1 - c0), sh.F, ldo, sh.slice_floats, sh.slice_pad, sh.n_slices, sh.G, cl->rows_cap,
+                       cl->edge_cap);
     return SGNN_OK;
 }
 
@@ -1874,16 +1945,17 @@ static void launch_fill_or_divide(float *out, int64_t M, int F, int64_t ldo, con
 
 // The product through the band schedule.  may_build = false (the non-allocating entry point): use a schedule
 // only if an earlier call has built it; *done tells whether the product was carried out here.
-static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *val, const DenseSrc &dense, float *out, int64_t F,
+static int spmm_run_band(sgnn_spmm_plan *p, const BandWindows &bw, const float *val, const DenseSrc &dense, float *out, int64_t F,
                          int64_t ldo, int accumulate, const float *row_div, hipStream_t st, bool may_build, bool *done) {
     *done = false;
+    const BandShape &sh0 = bw.w[0];
     BandSchedule *bs = nullptr;
     for (BandSchedule *c : p->bands)
-        if (c->band_cols == sh.band_cols) bs = c;
+        if (c->band_cols == sh0.band_cols) bs = c;
     // The restaged operand lives in the plan the caller holds: the row blocks of a large matrix share one copy,
     // restaged by the first block of a product that takes the band schedule.
     sgnn_spmm_plan *root = p->whole ? p->whole : p;
-    const size_t xs_floats = (size_t)sh.n_slices * (size_t)p->K * (size_t)sh.slice_pad;
+    const size_t xs_floats = bw.xs_floats;
     if (bs == nullptr || xs_floats > root->band_xs_floats) {
         if (!may_build) return SGNN_OK;
         bool sorted = false;
@@ -1891,7 +1963,19 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
         if (rc != SGNN_OK) return rc;
         if (!sorted) return SGNN_OK;  // band edges of a row would not be contiguous: the other schedules take it
         if (bs == nullptr) {
-            if ((rc = band_build(p, sh.band_cols, sh.n_bands, st, &bs)) != SGNN_OK) return rc;
+            // A plan keeps the schedules of at most kMaxBandSchedules band widths (each holds a band-major copy of
+            // the edge list): the one used longest ago makes room.
+            if (p->bands.size() >= (size_t)kMaxBandSchedules) {
+                SGNN_HIP_CHECK(hipDeviceSynchronize());   // queued launches may still read it
+                size_t victim = 0;
+                for (size_t i = 1; i < p->bands.size(); ++i)
+                    if (p->bands[i]->last_use < p->bands[victim]->last_use) victim = i;
+                delete p->bands[victim];
+                p->bands.erase(p->bands.begin() + (long)victim);
+            }
+            rc = band_build(p, sh0.band_cols, sh0.n_bands, st, &bs);
+            if (rc == SGNN_ERR_HIP && band_build_out_of_memory()) return SGNN_OK;  // no room for the band-major copy: the row-class schedule runs
+            if (rc != SGNN_OK) return rc;
             p->bands.push_back(bs);
         }
         if (xs_floats > root->band_xs_floats) {
@@ -1900,21 +1984,30 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
             root->band_xs = nullptr;
             root->band_xs_floats = 0;
             root->xs_serial = 0;
-            SGNN_HIP_CHECK(hipMalloc(&root->band_xs, xs_floats * sizeof(float)));
+            if (hipMalloc(&root->band_xs, xs_floats * sizeof(float)) != hipSuccess) {
+                (void)hipGetLastError();
+                root->band_xs = nullptr;
+                return SGNN_OK;   // no room for the restaged operand: the row-class schedule runs
+            }
             root->band_xs_floats = xs_floats;
         }
     }
-    const BandCaps caps = band_chunk_caps(p, sh, val != nullptr);
-    const BandSchedule::ChunkList *cl = nullptr;
-    for (const BandSchedule::ChunkList &l : bs->lists)
-        if (l.rows_cap == caps.rows && l.edge_cap == caps.edges) cl = &l;
-    if (cl == nullptr) {
-        if (!may_build) return SGNN_OK;
-        const int rc = band_build_chunks(bs, caps.rows, caps.edges, st, &cl);
-        if (rc != SGNN_OK) return rc;
+    const bool weighted = val != nullptr;
+    const BandSchedule::ChunkList *cls[kBandMaxWindows];
+    for (int w = 0; w < bw.n; ++w) {
+        const BandCaps caps = band_chunk_caps(p, bw.w[w], weighted);
+        const BandSchedule::ChunkList *cl = nullptr;
+        for (const BandSchedule::ChunkList &l : bs->lists)
+            if (l.rows_cap == caps.rows && l.edge_cap == caps.edges) cl = &l;
+        if (cl == nullptr) {
+            if (!may_build) return SGNN_OK;
+            const int rc = band_build_chunks(bs, caps.rows, caps.edges, st, &cl);
+            if (rc != SGNN_OK) return rc;
+        }
+        cls[w] = cl;
     }
     const float *val_bm = nullptr;
-    if (val != nullptr) {
+    if (weighted) {
         const bool bound = val == p->bound_val;
         if (!(bound && bs->val_gen == p->bind_gen)) {
             hipLaunchKernelGGL(permute_values_kernel, dim3((uint32_t)((p->nnz + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, val,
@@ -1925,28 +2018,38 @@ static int spmm_run_band(sgnn_spmm_plan *p, const BandShape &sh, const float *va
     }
     const int iF = (int)F;
     if (p->whole == nullptr) ++root->call_serial;  // (a plan of row blocks counts its products in spmm_run)
-    if (!(root->xs_serial == root->call_serial && root->xs_F == iF && root->xs_slice_pad == sh.slice_pad && root->xs_slices == sh.n_slices)) {
-        ProfScope prof(K_SPMM_BAND_RESTAGE, st);
-        const int64_t n = (int64_t)sh.n_slices * p->K * (sh.slice_pad / 4);
-        hipLaunchKernelGGL(band_restage_kernel, dim3((uint32_t)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, dense.x, dense.ldx,
-                           root->band_xs, p->K, iF, sh.slice_floats, sh.slice_pad, sh.n_slices);
+    bs->last_use = ++root->band_use_clock;
+    if (!(root->xs_serial == root->call_serial && root->xs_F == iF && root->xs_slice_pad == sh0.slice_pad && root->xs_slices == bw.total_slices)) {
+        ProfScope prof(K_SPMM_BAND_RESTAGE, st, may_build);
+        for (int w = 0; w < bw.n; ++w) {
+            const BandShape &sh = bw.w[w];
+            const int64_t n = (int64_t)sh.n_slices * p->K * (sh.slice_pad / 4);
+            hipLaunchKernelGGL(band_restage_kernel, dim3((uint32_t)((n + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, dense.x + sh.f0,
+                               dense.ldx, root->band_xs + sh.xs_off, p->K, sh.F, sh.slice_floats, sh.slice_pad, sh.n_slices);
+        }
         root->xs_serial = root->call_serial;
-        root->xs_F = iF; root->xs_slice_pad = sh.slice_pad; root->xs_slices = sh.n_slices;
+        root->xs_F = iF; root->xs_slice_pad = sh0.slice_pad; root->xs_slices = bw.total_slices;
     }
-    const int ev = sh.even ? 2 : 1;  // vector width of the fill / divide passes
+    // vector width of the fill / divide passes over whole rows of out
+    const int ev = (ldo % 2 == 0 && F % 2 == 0 && F >= 4 && aligned(out, 8)) ? 2 : 1;
     if (!accumulate) {
         if (ev == 2) launch_fill_or_divide<2>(out, p->M, iF, ldo, nullptr, st);
         else launch_fill_or_divide<1>(out, p->M, iF, ldo, nullptr, st);
     }
     {
-        ProfScope prof(K_SPMM_BAND, st);
-        for (int b = 0; b < bs->n_bands; ++b) {
-            int rc;
-            if (val_bm) rc = sh.even ? launch_band<true, true>(bs, cl, sh, b, val_bm, root->band_xs, out, iF, ldo, st, p->device)
-                                     : launch_band<false, true>(bs, cl, sh, b, val_bm, root->band_xs, out, iF, ldo, st, p->device);
-            else rc = sh.even ? launch_band<true, false>(bs, cl, sh, b, val_bm, root->band_xs, out, iF, ldo, st, p->device)
-                              : launch_band<false, false>(bs, cl, sh, b, val_bm, root->band_xs, out, iF, ldo, st, p->device);
-            if (rc != SGNN_OK) return rc;
+        ProfScope prof(K_SPMM_BAND, st, may_build);
+        // window after window, band after band: a window's accumulators make all their trips through `out` while
+        // its columns of `out` are the only ones in flight
+        for (int w = 0; w < bw.n; ++w) {
+            const BandShape &sh = bw.w[w];
+            for (int b = 0; b < bs->n_bands; ++b) {
+                int rc;
+                if (val_bm) rc = sh.even ? launch_band<true, true>(bs, cls[w], sh, b, val_bm, root->band_xs, out, ldo, st, p->device)
+                                         : launch_band<false, true>(bs, cls[w], sh, b, val_bm, root->band_xs, out, ldo, st, p->device);
+                else rc = sh.even ? launch_band<true, false>(bs, cls[w], sh, b, val_bm, root->band_xs, out, ldo, st, p->device)
+                                  : launch_band<false, false>(bs, cls[w], sh, b, val_bm, root->band_xs, out, ldo, st, p->device);
+                if (rc != SGNN_OK) return rc;
+            }
         }
     }
     if (row_div) {
@@ -1962,9 +2065,9 @@ extern "C" int sgnn_spmm_plan_schedule(const sgnn_spmm_plan *p, int64_t F, int64
     SGNN_REQUIRE(p != nullptr && info != nullptr, "null argument");
     SGNN_REQUIRE(F > 0 && F < (1 << 24), "feature width F=%lld out of range", (long long)F);
     if (!p->parts.empty()) p = p->parts[0];  // row blocks decide one by one; the first one's answer is reported
-    const BandShape sh = band_shape(p, F, true);
-    info[0] = (band_wanted(p, F, sh) && p->cols_sorted != 0) ? 1 : 0;
-    info[1] = sh.band_cols; info[2] = sh.n_bands; info[3] = sh.n_slices;
+    const BandWindows bw = band_windows(p, F, true);
+    info[0] = (band_wanted(p, F, bw.w[0]) && p->cols_sorted != 0) ? 1 : 0;
+    info[1] = bw.w[0].band_cols; info[2] = bw.w[0].n_bands; info[3] = bw.total_slices;
     return SGNN_OK;
 }
 
@@ -2029,10 +2132,10 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
         vec = 2;
     }
     if (bits == 0 && !is_slice) {
-        const BandShape sh = band_shape(p, F, ldo % 2 == 0 && aligned(out, 8));
-        if (band_wanted(p, F, sh)) {
+        const BandWindows bw = band_windows(p, F, ldo % 2 == 0 && aligned(out, 8));
+        if (band_wanted(p, F, bw.w[0])) {
             bool done = false;
-            const int rc = spmm_run_band(p, sh, val, dense, out, F, ldo, accumulate, row_div, st, scratch == nullptr, &done);
+            const int rc = spmm_run_band(p, bw, val, dense, out, F, ldo, accumulate, row_div, st, scratch == nullptr, &done);
             if (rc != SGNN_OK || done) return rc;
         }
         // Wide fp32 rows of a large operand: one product per slice of the feature axis, one after the other.  The rows
@@ -2078,7 +2181,7 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     const int which = gw == 8 ? 0 : gw == 16 ? 1 : 2;
     SGNN_REQUIRE(p->n_chunks[which] >= 0, "plan has no chunk list for this feature width (plan creation failed?)");
     ShortArgs a{p->rowptr, p->col, val, dense, out, p->chunks[which], (int)p->n_chunks[which], p->empty_rows,
-                (int)p->n_empty, (int)F, ldo, accumulate, row_div};
+                (int)p->n_empty, (int)F, ldo, accumulate, row_div, scratch == nullptr};
     if (scratch == nullptr && p->side == nullptr && p->n_long > 0 && env_int("SGNN_SPMM_OVERLAP", 0) != 0) {
         SGNN_HIP_CHECK(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));  // default priority
         SGNN_HIP_CHECK(hipEventCreateWithFlags(&p->ev_fork, hipEventDisableTiming));

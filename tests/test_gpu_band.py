@@ -25,20 +25,30 @@ def _force(monkeypatch, cols):
     monkeypatch.setenv("SGNN_SPMM_BAND_COLS", str(cols))
 
 
-@pytest.mark.parametrize("M,K,F,deg,cols", [
-    (700, 900, 602, 40, 128),     # the wide odd width: float2 lanes, 8 slices of 38 vectors, 8 bands
-    (500, 1000, 128, 30, 100),    # float4, 2 slices x 4 row groups; band width not a power of two
-    (300, 800, 256, 25, 256),     # 4 slices x 2 row groups
-    (257, 600, 64, 20, 64),       # one slice, 8 row groups
-    (300, 500, 123, 20, 70),      # scalar lanes
-    (200, 400, 100, 15, 50),      # float4 with a ragged last slice
-    (150, 300, 2052, 9, 40),      # slices wider than one register tile
-    (90, 200, 4, 6, 16), (90, 200, 1, 6, 16), (64, 100, 10, 5, 7),
-    (400, 5000, 602, 12, 37),     # 136 bands, most (row, band) pairs empty
+@pytest.mark.parametrize("M,K,F,deg,cols,window", [
+    (700, 900, 602, 40, 128, None),    # a window of 512 columns (8 slices of 64 floats) + one of 90 (2 slices of 48, 12 of 16 lanes)
+    (700, 900, 602, 40, 128, 0),       # the same in one piece: float2 lanes, 8 slices of 38 vectors, 8 bands
+    (500, 1000, 128, 30, 100, None),   # float4, 2 slices x 4 row groups; band width not a power of two
+    (300, 800, 256, 25, 256, None),    # 4 slices x 2 row groups
+    (257, 600, 64, 20, 64, None),      # one slice, 8 row groups
+    (300, 500, 123, 20, 70, None),     # scalar lanes
+    (200, 400, 100, 15, 50, None),     # float4 with a ragged last slice
+    (150, 300, 2052, 9, 40, 0),        # in one piece: slices wider than one register tile
+    (150, 300, 2052, 9, 40, None),     # four windows and a remainder of one float4
+    (90, 200, 4, 6, 16, None), (90, 200, 1, 6, 16, None), (64, 100, 10, 5, 7, None),
+    (400, 5000, 602, 12, 37, None),    # 136 bands, most (row, band) pairs empty
+    (300, 700, 768, 25, 90, None),     # 512 + 256: the second window is 4 slices x 2 row groups
+    (260, 600, 1024, 20, 64, None),    # two full windows
+    (200, 500, 514, 15, 50, None),     # remainder of two floats
+    (200, 500, 513, 15, 50, None),     # odd width: scalar lanes in both windows
+    (200, 500, 1100, 15, 50, None),    # 512 + 512 + 76
+    (220, 450, 330, 18, 45, 128),      # windows of 128 columns: 128 + 128 + 74
 ])
-def test_band_schedule_bit_identical_to_oracle(M, K, F, deg, cols, monkeypatch):
+def test_band_schedule_bit_identical_to_oracle(M, K, F, deg, cols, window, monkeypatch):
     ops = _ops()
     _force(monkeypatch, cols)
+    if window is not None:
+        monkeypatch.setenv("SGNN_SPMM_BAND_WINDOW", str(window))
     rowptr, col, val = random_csr(M, K, deg, seed=M + F, empty_frac=0.1, hubs=3, hub_deg=min(K, 700))
     rng = np.random.default_rng(F)
     x = rng.standard_normal((K, F), dtype=np.float32)
@@ -225,7 +235,8 @@ def test_schedule_is_chosen_from_the_matrix_shape():
     dev = torch.device("cuda:0")
     rp, cl = synth.sbm_graph(60000, 10, 0.02, 0.001, seed=3, device=dev)              # ~170 edges per row
     dense = ops.SpmmPlan(rp, cl, 60000)
-    assert dense.schedule(602)["band"] == 1 and dense.schedule(602)["n_slices"] == 8
+    assert dense.schedule(602)["band"] == 1 and dense.schedule(602)["n_slices"] == 10   # a window of 8 slices + one of 2
+    assert dense.schedule(512)["n_slices"] == 8 and dense.schedule(256)["n_slices"] == 4
     assert dense.schedule(64)["band"] == 0                                             # 15 MB of X: cache-resident
     rp, cl = synth.rmat_graph(200000, 2500000, seed=1, device=dev)                     # 25 edges per row
     power = ops.SpmmPlan(rp, cl, 200000)
