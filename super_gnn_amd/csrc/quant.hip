@@ -645,6 +645,339 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
+// Fused quantize + pack over a run of consecutive rows: any row width from 16 floats, rows contiguous in memory.
+//
+// A wavefront takes `gw` consecutive packed rows, i.e. gw * EPB fp32 rows (at most 64), which lie one after the
+// other in memory.  Each row is cut into VPR = ceil(F / 4) float4 vectors and the chunk's rows * VPR vectors are
+// dealt to the lanes in order: lane l holds vectors l, l + 64, ... .  A load instruction therefore fetches 64
+// consecutive vectors -- 1 KB of consecutive bytes when F % 4 == 0, a few rows' worth of them otherwise -- and no
+// lane slot idles because a row is not a whole number of lane-group passes (the lane-group kernels leave 25 of 32
+// slots busy at F = 100).  What those kernels get from their fixed row -> lane mapping goes through a
+// wave-private piece of LDS here:
+//   A  every lane reduces each of its vectors to (min, max) and writes the pair to LDS;
+//   B  the lanes are regrouped, 64 / rows lanes per row: each group reduces its row's pairs, computes zero_point,
+//      scale and the reciprocal, stores the params and leaves them in a row table in LDS;
+//   C  every lane quantizes its vectors with their rows' table entries and writes the four code bytes of each
+//      to a code array in LDS (int8 with F % 4 == 0: straight to memory);
+//   D  the lanes walk the output run (gw * F consecutive bytes) in aligned 4-byte words, 256 bytes per store
+//      instruction: a word is the OR of the EPB rows' code words, fetched from the code array at their byte
+//      offsets and shifted to their bit positions.
+// The last vector of a row with F % 4 != 0 is loaded element by element and padded with copies of its first
+// element (copies change neither min nor max nor the first-zero rule); vector slots without a row (past the end
+// of the chunk, or the row slots a segment's short last group leaves empty) hold zeros, which quantize to code 0
+// under the empty slot's neutral params.
+// Signed zeros: v_min_f32 / v_max_f32 order -0 < +0, so a zero minimum is -0 exactly when the row holds a -0
+// and a zero maximum is +0 exactly when it holds a +0; the sign of the row's FIRST zero (what the reference's
+// strict compares keep, quantization_arm.cpp:98-101) needs a second pass over the elements only when a row
+// may hold zeros of both signs.
+// ------------------------------------------------------------------------------------------------
+constexpr int kStreamRows = 64;   // fp32 rows per wavefront chunk, at most (one lane per row in the set-up)
+__host__ __device__ constexpr int stream_wave_bytes(int nv) {
+    // (min, max) pair per vector -- later the code bytes, which need half of it (+ 16 for the funnel reads) --, row
+    // table (float4, neutral entries past the last row), row ids, row flags
+    return nv * 512 + 16 + (kStreamRows + 4) * 16 + kStreamRows * (4 + 4);
+}
+
+// RAGGED: F % 4 != 0, or an output buffer that is not 4-byte aligned.
+template <int BITS, int NV, bool RAGGED, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
+    const float *__restrict__ x, uint8_t *__restrict__ q, const ParamBuf pb, const int32_t *__restrict__ seg,
+    const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F, int gw, int n_units, int n_rows) {
+    constexpr int EPB = 8 / BITS;
+    constexpr int kWaveBytes = stream_wave_bytes(NV);
+    static_assert(kWaveBytes % 16 == 0, "wave pieces of LDS must keep 16-byte alignment");
+    static_assert(WAVES * kWaveBytes <= 64 * 1024, "static LDS of a workgroup");
+    __shared__ __align__(16) uint8_t lds_all[WAVES * kWaveBytes];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int unit = blockIdx.x * WAVES + wv;
+    if (unit >= n_units) return;   // wave-uniform
+    uint8_t *base = lds_all + wv * kWaveBytes;
+    float2 *ent = reinterpret_cast<float2 *>(base);
+    float4 *rowtab = reinterpret_cast<float4 *>(base + NV * 512 + 16);   // (zero_point, scale, 1 / scale, needs the exact division)
+    int *rowid = reinterpret_cast<int *>(rowtab + kStreamRows + 4);
+    int *rowflag = rowid + kStreamRows;
+    uint8_t *codes = base;   // the pairs are dead by the time the codes are written
+
+    const int g0 = __builtin_amdgcn_readfirstlane(unit) * gw;
+    const int ng = n_packed - g0 < gw ? n_packed - g0 : gw;
+    const int npr = ng * EPB;          // fp32 row slots of the chunk (the last group of a segment may leave some empty)
+    const int VPR = (F + 3) >> 2;      // vectors per row; npr * VPR <= NV * 64
+
+    // ---- the chunk's rows: lane i looks up row slot i --------------------------------------------------------
+    int my_row = -1;
+    {
+        WaveSegment ws{0, 0, 0, 0, 0};
+        if (single_rows < 0) ws = wave_find_segment(pseg, seg, P, g0);
+        if (lane < npr) {
+            int64_t row0, rend;
+            locate_packed_row_w(seg, pseg, P, single_rows, g0 + lane / EPB, ws, EPB, row0, rend);
+            const int64_t r = row0 + lane % EPB;
+            if (r < rend) my_row = (int)r;
+        }
+        rowid[lane] = my_row;
+        rowflag[lane] = 0;
+        rowtab[lane] = make_float4(0.0f, 1.0f, 1.0f, 0.0f);
+        if (lane < 4) rowtab[kStreamRows + lane] = make_float4(0.0f, 1.0f, 1.0f, 0.0f);
+    }
+    const unsigned long long vb = __ballot(my_row >= 0);
+    const int n_valid = __popcll(vb);
+    const int r_first = __builtin_amdgcn_readfirstlane(my_row);
+    // rows consecutive in memory, empty slots only at the end: row slot p holds row r_first + p for p < n_valid
+    const bool run = (vb & (vb + 1)) == 0 && (vb & 1) && __ballot(my_row >= 0 && my_row != r_first + lane) == 0;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+
+    // ---- loads ------------------------------------------------------------------------------------------------
+    // (row slot, vector inside the row) of each of the lane's vectors: advanced by 64 vectors per step
+    const int dpr = 64 / VPR, dcv = 64 % VPR;
+    int prv[NV];
+    float xv[NV][4];
+    uint32_t first_mask = 0;   // bit v: vector v starts its row
+    uint32_t short_mask = 0;   // bit v: vector v is the short last vector of its row (F % 4 elements)
+    (void)short_mask;
+    {
+        int pr = lane / VPR, cv = lane - pr * VPR;
+        if (run) {
+            // The common case: one base address, 32-bit element offsets, every vector a 16-byte load -- a row's short
+            // last vector too, which then reaches into the next row and is cut back after all loads are out; only the
+            // one that would reach past the end of the tensor is moved back to end with it.  Vectors that every lane
+            // holds (all but the last one or two of the chunk) are loaded without a lane predicate.
+            const float *xb = x + (int64_t)r_first * F;
+            const int n_sv = n_valid * VPR;
+            const uint32_t eo_max = (uint32_t)((n_rows - r_first) * F - 4);   // (a chunk is far smaller than 2^31 elements)
+            const int cv_short = (F & 3) != 0 ? VPR - 1 : -1;   // the vector of a row that holds fewer than four elements
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                prv[v] = pr < kStreamRows ? pr : kStreamRows;   // (slots past the chunk: the neutral table entry)
+                uint32_t eo = RAGGED ? (uint32_t)(pr * F + 4 * cv) : (uint32_t)(4 * (v * 64 + lane));
+                if constexpr (RAGGED) eo = eo < eo_max ? eo : eo_max;
+                if ((v + 1) * 64 <= n_sv) {   // wave-uniform
+                    vec4_load_nt_unaligned(xv[v], xb + eo);
+                    if (cv == 0) first_mask |= 1u << v;
+                    if (RAGGED && cv == cv_short) short_mask |= 1u << v;
+                } else {
+                    xv[v][0] = 0.0f; xv[v][1] = 0.0f; xv[v][2] = 0.0f; xv[v][3] = 0.0f;
+                    if (v * 64 + lane < n_sv) {
+                        vec4_load_nt_unaligned(xv[v], xb + eo);
+                        if (cv == 0) first_mask |= 1u << v;
+                        if (RAGGED && cv == cv_short) short_mask |= 1u << v;
+                    }
+                }
+                pr += dpr;
+                cv += dcv;
+                if (cv >= VPR) { cv -= VPR; ++pr; }
+            }
+            if constexpr (RAGGED) {   // cut the short vectors back to their F % 4 elements, padded with copies of the first
+                const int nt = F & 3;
+                if (__ballot(short_mask != 0) != 0) {
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) {
+                        if ((short_mask >> v) & 1u) {
+                            const uint32_t eo = (uint32_t)(prv[v] * F + 4 * (VPR - 1));
+                            if (eo > eo_max) {   // the tensor's last vector was loaded eo - eo_max elements early
+                                const int d = (int)(eo - eo_max);
+                                const float a1 = xv[v][1], a2 = xv[v][2], a3 = xv[v][3];
+                                xv[v][0] = d == 1 ? a1 : d == 2 ? a2 : a3;
+                                xv[v][1] = d == 1 ? a2 : a3;
+                                xv[v][2] = a3;
+                            }
+#pragma unroll
+                            for (int t = 1; t < 4; ++t)
+                                if (t >= nt) xv[v][t] = xv[v][0];
+                        }
+                    }
+                }
+            }
+        } else {
+            // a chunk that spans the end of a segment: row by row through the chunk's row table
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                prv[v] = pr < kStreamRows ? pr : kStreamRows;
+                const int r = pr < npr ? rowid[pr] : -1;
+                xv[v][0] = 0.0f; xv[v][1] = 0.0f; xv[v][2] = 0.0f; xv[v][3] = 0.0f;
+                if (r >= 0) {
+                    const float *xp = x + (int64_t)r * F + 4 * cv;
+                    const float first = __builtin_nontemporal_load(xp);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) xv[v][t] = (t == 0 || 4 * cv + t < F) ? __builtin_nontemporal_load(xp + t) : first;
+                    if (cv == 0) first_mask |= 1u << v;
+                }
+                pr += dpr;
+                cv += dcv;
+                if (cv >= VPR) { cv -= VPR; ++pr; }
+            }
+        }
+    }
+
+    // ---- A: (min, max) of every vector -----------------------------------------------------------------------
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const float m = fminf(fminf(xv[v][0], xv[v][1]), fminf(xv[v][2], xv[v][3]));
+        const float M = fmaxf(fmaxf(xv[v][0], xv[v][1]), fmaxf(xv[v][2], xv[v][3]));
+        ent[v * 64 + lane] = make_float2(m, M);
+        // a NaN is sticky only as element 0 of its row
+        if (((first_mask >> v) & 1u) && xv[v][0] != xv[v][0]) rowflag[prv[v]] = 1;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- B: per-row reduction, LR lanes per row --------------------------------------------------------------
+    int lr_shift = 0;   // LR = largest power of two <= 64 / npr
+    while ((npr << (lr_shift + 1)) <= 64) ++lr_shift;
+    const int LR = 1 << lr_shift;
+    const int row_b = lane >> lr_shift, li = lane & (LR - 1);
+    const bool has_row = row_b < npr;
+    const int e_lo = has_row ? row_b * VPR : 0, e_hi = has_row ? e_lo + VPR : 0;   // the row's vectors
+    float mn = INFINITY, mx = -INFINITY;
+    for (int e = e_lo + li; e < e_hi; e += LR) {
+        const float2 p = ent[e];
+        mn = fminf(mn, p.x);
+        mx = fmaxf(mx, p.y);
+    }
+    for (int o = 1; o < LR; o <<= 1) {
+        mn = fminf(mn, __shfl_xor(mn, o, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    }
+    const bool row_valid = has_row && rowid[has_row ? row_b : 0] >= 0;
+    // the sign of the row's first zero, where both signs may occur (see the header)
+    {
+        const bool mn0 = mn == 0.0f, mx0 = mx == 0.0f;
+        const bool neg0 = mn0 && (__float_as_uint(mn) >> 31) != 0;     // the row holds a -0 (known when mn == 0)
+        const bool pos0 = mx0 && (__float_as_uint(mx) >> 31) == 0;     // the row holds a +0 (known when mx == 0)
+        const bool unsure = row_valid && ((mn0 && neg0 && !(mx0 && !pos0)) || (mx0 && pos0 && !(mn0 && !neg0)));
+        if (__ballot(unsure) != 0) {   // wave-uniform, rare: first zero of every row by position
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                int k0 = INT_MAX;
+#pragma unroll
+                for (int t = 3; t >= 0; --t)
+                    if (xv[v][t] == 0.0f) k0 = (((v * 64 + lane) * 4 + t) << 1) | (int)(__float_as_uint(xv[v][t]) >> 31);
+                ent[v * 64 + lane].x = __int_as_float(k0);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            int key = INT_MAX;
+            for (int e = e_lo + li; e < e_hi; e += LR) key = min(key, __float_as_int(ent[e].x));
+            for (int o = 1; o < LR; o <<= 1) key = min(key, __shfl_xor(key, o, 64));
+            const float z = (key & 1) ? -0.0f : 0.0f;
+            if (mn0) mn = z;
+            if (mx0) mx = z;
+        }   // (else every zero of the row has the sign the reduction shows)
+    }
+    if (has_row && rowflag[has_row ? row_b : 0] != 0) {
+        mn = __int_as_float(0x7fc00000);
+        mx = mn;
+    }
+    {
+        float s = (mx - mn) / (float)((1 << BITS) - 1);
+        if (s == 0.0f) s = 1.0f;
+        const bool exact_row = !(s >= 0x1p-100f && s <= 0x1p100f);
+        if (row_valid && li == 0) {   // (empty row slots keep their neutral entry)
+            rowtab[row_b] = make_float4(mn, s, __builtin_amdgcn_rcpf(s), exact_row ? 1.0f : 0.0f);
+            store_params(pb, rowid[row_b], mn, s);
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- C: codes (the guard-band reciprocal of quant_pack_rows16_kernel) -------------------------------------
+    constexpr float kGuard = BITS == 8 ? 0x1p-13f : BITS == 4 ? 0x1p-17f : 0x1p-19f;
+    uint8_t *out_run = q + (int64_t)g0 * F;                         // the chunk's ng * F output bytes
+    const int mis = RAGGED ? (int)(reinterpret_cast<uintptr_t>(out_run) & 3) : 0;
+    bool lane_exact = false;
+    uint32_t words[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const float4 ta = rowtab[prv[v]];
+        if (ta.w != 0.0f) lane_exact = true;
+        uint32_t word = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float qf = (xv[v][t] - ta.x) * ta.z;
+            const float ri = rintf(qf);
+            if (!(fabsf(qf - ri) < 0.5f - kGuard)) lane_exact = true;   // also true for a NaN quotient
+            word = __builtin_amdgcn_cvt_pk_u8_f32(ri, t, word);
+        }
+        words[v] = word;
+    }
+    if (lane_exact) {   // this lane redoes its elements with the IEEE division
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const float4 ta = rowtab[prv[v]];
+            uint32_t word = 0;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) word |= quant_code(xv[v][t], ta.x, ta.y) << (8 * t);
+            words[v] = word;
+        }
+    }
+    if (EPB == 1 && !RAGGED) {   // code words are output words
+        uint32_t *q32 = reinterpret_cast<uint32_t *>(out_run);
+#pragma unroll
+        for (int v = 0; v < NV; ++v)
+            if (v * 64 + lane < npr * VPR) __builtin_nontemporal_store(words[v], q32 + v * 64 + lane);
+        return;
+    }
+#pragma unroll
+    for (int v = 0; v < NV; ++v) reinterpret_cast<uint32_t *>(codes)[v * 64 + lane] = words[v];
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+
+    // ---- D: pack and store ------------------------------------------------------------------------------------
+    // code byte of (row slot p, column j): codes[p * pitch + j]
+    const int pitch = 4 * VPR;
+    const int nbytes = ng * F;
+    const int nw = (mis + nbytes + 3) >> 2;
+    const uint32_t *codes32 = reinterpret_cast<const uint32_t *>(codes);
+    uint32_t *q32 = reinterpret_cast<uint32_t *>(out_run - mis);
+    // (packed row, column) of the LAST byte of a lane's word (never negative): advanced by 256 bytes per round
+    const int dgr = 256 / F, djc = 256 % F;
+    int b0 = 4 * lane - mis;
+    int gr = (b0 + 3) / F, jc = b0 + 3 - gr * F;
+    for (int w = lane; w < nw; w += 64) {
+        if (!RAGGED) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int k = 0; k < EPB; ++k) word |= codes32[((gr * EPB + k) * pitch + jc - 3) >> 2] << ((EPB - 1 - k) * BITS);
+            __builtin_nontemporal_store(word, q32 + w);
+        } else if (b0 >= 0 && b0 + 3 < nbytes) {
+            // jc >= 3: four bytes of packed row gr; else the first 3 - jc bytes are the end of packed row gr - 1
+            const int nA = jc >= 3 ? 0 : 3 - jc;
+            const uint32_t keep = 0xffffffffu << (8 * nA);
+            uint32_t word = 0;
+#pragma unroll
+            for (int k = 0; k < EPB; ++k) {
+                const int off = (gr * EPB + k) * pitch + jc - 3;
+                const uint32_t c = __builtin_amdgcn_alignbyte(codes32[(off >> 2) + 1], codes32[off >> 2], (uint32_t)(off & 3));
+                word |= (c & keep) << ((EPB - 1 - k) * BITS);
+            }
+            if (nA != 0) {
+#pragma unroll
+                for (int k = 0; k < EPB; ++k) {
+                    const int off = ((gr - 1) * EPB + k) * pitch + F + jc - 3;
+                    const uint32_t c = __builtin_amdgcn_alignbyte(codes32[(off >> 2) + 1], codes32[off >> 2], (uint32_t)(off & 3));
+                    word |= (c & ~keep) << ((EPB - 1 - k) * BITS);
+                }
+            }
+            __builtin_nontemporal_store(word, q32 + w);
+        } else {   // the first or the last word of the run, partly outside it
+            for (int t = 0; t < 4; ++t) {
+                const int b = b0 + t;
+                if (b < 0 || b >= nbytes) continue;
+                const int c = jc - 3 + t;
+                const int g = c < 0 ? gr - 1 : gr, j = c < 0 ? c + F : c;
+                uint32_t byte = 0;
+#pragma unroll
+                for (int k = 0; k < EPB; ++k) byte |= (uint32_t)codes[(g * EPB + k) * pitch + j] << ((EPB - 1 - k) * BITS);
+                out_run[b] = (uint8_t)byte;
+            }
+        }
+        b0 += 256;
+        gr += dgr;
+        jc += djc;
+        if (jc >= F) { jc -= F; ++gr; }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Unpack + dequantize, row-group layout.  Same work decomposition as the quantize kernel.
 // ------------------------------------------------------------------------------------------------
 template <int BITS, int VEC, int G, int NV>
@@ -1608,6 +1941,11 @@ __global__ __launch_bounds__(kQBlock) void row_slots_kernel(const int32_t *__res
 // ------------------------------------------------------------------------------------------------
 // Launch tables.
 // ------------------------------------------------------------------------------------------------
+static int env_flag(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return e ? atoi(e) : dflt;
+}
+
 struct RowsArgs {
     RowSrc x_in; uint8_t *q_out;                                     // quantize
     const uint8_t *q_in; float *x_out;                               // dequantize
@@ -1720,6 +2058,56 @@ static void launch_quant16(const RowsArgs &a, hipStream_t st) {
     else
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
                            a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
+}
+
+// Lane-slot shape of the stream quantizer for rows of F floats: NV vectors per lane (one of the instantiated
+// values) and gw packed rows per wavefront, chosen to fill the wavefront's NV * 64 vector slots.
+static bool stream_shape(int F, int epb, int *nv_out, int *gw_out) {
+    static const int nvs[] = {4, 8, 10, 12, 16, 20};
+    const int vpr = (F + 3) / 4;
+    double best = 0.0;
+    for (int nv : nvs) {
+        // More vectors per lane cost registers and LDS, hence wavefronts per CU: beyond 10 only when a packed row needs it
+        // (measured: 16 vectors per lane run at 4.1-4.6 TB/s where 8-10 reach 5.4-6.0).
+        if (best > 0.0 && nv > 10) break;
+        const int gw = std::min(nv * 64 / (epb * vpr), kStreamRows / epb);
+        if (gw < 1) continue;
+        const double fill = (double)gw * epb * vpr / (nv * 64);
+        if (fill > best + 0.025) {
+            best = fill;
+            *nv_out = nv;
+            *gw_out = gw;
+        }
+    }
+    return best > 0.0;
+}
+
+template <int BITS, int NV, bool RAGGED>
+static void launch_quant_stream_nv(const RowsArgs &a, int gw, hipStream_t st) {
+    constexpr int WAVES = stream_wave_bytes(NV) * 4 <= 64 * 1024 ? 4 : 2;
+    const int n_units = (a.n_packed + gw - 1) / gw;
+    const int nb = (n_units + WAVES - 1) / WAVES;
+    ProfScope prof(K_QUANT_PACK_ROWS, st);
+    hipLaunchKernelGGL((quant_pack_stream_kernel<BITS, NV, RAGGED, WAVES>), dim3(nb), dim3(64 * WAVES), 0, st, a.x_in.x, a.q_out,
+                       a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, gw, n_units, (int)a.x_in.n_src);
+}
+
+template <int BITS>
+static bool launch_quant_stream(const RowsArgs &a, hipStream_t st) {
+    int nv = 0, gw = 0;
+    if (a.x_in.index != nullptr || a.x_in.ld != a.F || a.F < 16 || !stream_shape(a.F, 8 / BITS, &nv, &gw)) return false;
+    const bool ragged = a.F % 4 != 0 || !aligned(a.q_out, 4);
+#define SGNN_STREAM(NV_)                                                       \
+    case NV_:                                                                  \
+        if (ragged) launch_quant_stream_nv<BITS, NV_, true>(a, gw, st);        \
+        else launch_quant_stream_nv<BITS, NV_, false>(a, gw, st);              \
+        break
+    switch (nv) {
+        SGNN_STREAM(4); SGNN_STREAM(8); SGNN_STREAM(10); SGNN_STREAM(12); SGNN_STREAM(16); SGNN_STREAM(20);
+        default: return false;
+    }
+#undef SGNN_STREAM
+    return true;
 }
 
 template <int BITS, int R>
@@ -1869,6 +2257,15 @@ static void dispatch_rows(int vec, const RowsArgs &a, hipStream_t st) {
     else dispatch_rows_shape<BITS, 1>(a.F, a, st);
 }
 
+// Widths the stream quantizer takes by default (measured at 256 M elements per width, all three code widths): rows
+// of whole float4 in 4-byte aligned buffers, except the multiples of 64 floats up to 768, which are whole passes
+// of the sixteen-lane kernel (F = 128 / 256: 6.2 against 5.7-6.1 TB/s).  It gains most where a row leaves lane
+// slots of that kernel idle: F = 20 / 36 / 72 / 100 / 160: 4.3-5.7 -> 5.5-6.2 TB/s.  Rows that are not whole
+// float4 keep the lane-group kernels (F = 602: 5.4-5.7 against 5.0-5.4 TB/s; F = 123: 4.4-4.7 either way).
+static bool stream_wanted(int F, int vec) {
+    return vec == 4 && !(F % 64 == 0 && F <= 768);
+}
+
 static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp32_ptr, const void *u8_ptr,
                     hipStream_t st) {
     SGNN_REQUIRE(bits == 8 || bits == 4 || bits == 2, "bits=%d, expected 8, 4 or 2", bits);
@@ -1889,7 +2286,12 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
     if (a.F % 4 == 0 && ld % 4 == 0 && aligned(fp32_ptr, 16) && aligned(u8_ptr, 4)) vec = 4;
     else if (a.F % 2 == 0 && ld % 2 == 0 && aligned(fp32_ptr, 8) && aligned(u8_ptr, 2)) vec = 2;
     SGNN_REQUIRE(aligned(a.params.p, a.params.bf16 ? 4 : 8), "params must be %d-byte aligned", a.params.bf16 ? 4 : 8);
-    if (!a.quantize && vec == 4 && a.flat) {
+    const int stream = env_flag("SGNN_QUANT_STREAM", -1);   // 1: every width the stream quantizer can take, 0: never
+    bool taken = false;
+    if (a.quantize && !a.exact_division && (stream > 0 || (stream < 0 && stream_wanted(a.F, vec))))
+        taken = bits == 8 ? launch_quant_stream<8>(a, st) : bits == 4 ? launch_quant_stream<4>(a, st) : launch_quant_stream<2>(a, st);
+    if (taken) {
+    } else if (!a.quantize && vec == 4 && a.flat) {
         if (bits == 8) launch_dequant_flat<8>(a, n_rows, st);
         else if (bits == 4) launch_dequant_flat<4>(a, n_rows, st);
         else launch_dequant_flat<2>(a, n_rows, st);

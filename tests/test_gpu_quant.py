@@ -590,3 +590,49 @@ def test_offsets_beyond_four_gigabytes():
         d_got = d[bounds[i] + tail:bounds[i + 1]].cpu().numpy()
         assert np.all(np.abs(d_got - d_ref) <= dequant_atol(p_ref[:, 0], p_ref[:, 1], bits)[:, None])
         pstart += pk[i]
+
+
+def _special_rows(n, F, rng):
+    """Random rows with the cases the per-row rules turn on: outliers, a constant row, NaN as element 0 and later,
+    infinities, and rows whose minimum or maximum is a zero with zeros of both signs at random places."""
+    x = rng.standard_normal((n, F)).astype(np.float32)
+    x[::10] *= 100.0
+    if n < 40:
+        return x
+    x[3] = 0.5
+    x[5, 0] = np.nan
+    x[6, F // 2] = np.nan
+    x[7, F - 1] = np.inf
+    x[8, 1] = -np.inf
+    for r in range(12, 40):     # signed zeros: non-negative rows (min is a zero), non-positive rows (max is one), all-zero rows
+        kind = r % 4
+        row = np.abs(x[r]) if kind in (0, 1) else -np.abs(x[r]) if kind == 2 else np.zeros(F, np.float32)
+        k = rng.integers(1, 6)
+        pos = rng.choice(F, size=min(k, F), replace=False)
+        row[pos] = np.where(rng.random(pos.size) < 0.5, np.float32(0.0), np.float32(-0.0))
+        if kind == 3:
+            row[:] = np.where(rng.random(F) < (0.5 if r % 8 == 3 else 0.02), np.float32(-0.0), np.float32(0.0))
+        if r % 5 == 0:
+            row[pos] = -0.0     # zeros of one sign only
+        x[r] = row
+    return x
+
+
+@pytest.mark.parametrize("stream", ["0", "1"])
+@pytest.mark.parametrize("bits", [8, 4, 2])
+@pytest.mark.parametrize("F", [16, 20, 36, 100, 123, 128, 200, 301, 602, 1000, 1200, 1433])
+def test_stream_and_lane_group_quantizers_write_the_oracles_bytes(stream, bits, F, monkeypatch):
+    """SGNN_QUANT_STREAM forces (1) or forbids (0) the quantizer that walks a run of consecutive rows vector by
+    vector; by default the library picks per width.  Either kernel must write exactly the oracle's bytes and
+    params: ragged per-peer segments (short last groups, a chunk spanning two segments), special rows."""
+    monkeypatch.setenv("SGNN_QUANT_STREAM", stream)
+    rng = np.random.default_rng(1000 * bits + F)
+    n = 997
+    x = _special_rows(n, F, rng)
+    for seg in ([0, n], [0, 1, 2, 7, 7, 130, 131, 555, n]):
+        q_ref, p_ref = orc.quant_rows(x, seg, bits)
+        q, params, d = _quant_gpu(x, seg, bits)
+        nan_ref = np.isnan(p_ref)
+        assert np.array_equal(np.isnan(params), nan_ref), seg
+        assert np.array_equal(params[~nan_ref].view(np.uint32), p_ref[~nan_ref].view(np.uint32)), seg
+        assert np.array_equal(q, q_ref), seg
