@@ -1952,38 +1952,40 @@ struct RowsArgs {
     ParamBuf params;                                                 // written by quantize, read by dequantize
     const int32_t *seg; const int32_t *pseg; int P; int n_packed; int F; bool quantize;
     int64_t single_rows;  // the row count when P == 1 (kernels then read no segment table), else -1
-    bool layout16;        // diagnostic switch: one fp32 row per 16 lanes (default) vs per lane group
     bool flat;            // dequantize over the flat output (default) vs the row-tiled kernels
     bool exact_division;  // diagnostic: IEEE division for every element (the results are identical either way)
 };
 
-template <int BITS, int VEC, int G, int NV>
+// ONLY = 1: shapes the quantizer never takes (rows of up to 1024 aligned floats go to the sixteen-lane and stream
+// kernels); ONLY = 2: shapes the dequantizer never takes.
+template <int BITS, int VEC, int G, int NV, int ONLY = 0>
 static void launch_rows(const RowsArgs &a, hipStream_t st) {
     constexpr int NPR = kRowsPerGroup / (8 / BITS);
     constexpr int GPB = kQBlock / G;
     const int n_units = (a.n_packed + NPR - 1) / NPR;
     const int nb = (n_units + GPB - 1) / GPB;
     ProfScope prof(a.quantize ? K_QUANT_PACK_ROWS : K_UNPACK_DEQUANT_ROWS, st);
-    if (a.quantize && a.exact_division)
-        hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
-                           a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
-    else if (a.quantize)
-        hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV, false>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
-                           a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
-    else
+    if constexpr (ONLY != 1) {
+        if (a.quantize && a.exact_division) {
+            hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
+                               a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
+            return;
+        }
+        if (a.quantize) {
+            hipLaunchKernelGGL((quant_pack_rows_kernel<BITS, VEC, G, NV, false>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
+                               a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
+            return;
+        }
+    }
+    if constexpr (ONLY != 2)
         hipLaunchKernelGGL((unpack_dequant_rows_kernel<BITS, VEC, G, NV>), dim3(nb), dim3(kQBlock), 0, st, a.q_in,
                            a.x_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
 // Rows that are not a whole number of lane-group passes (every width but 4 * L * NV floats) write their packed
-// bytes through the wave-private LDS stage (SGNN_QUANT_STAGED=0: straight from the lanes, for comparison).  Measured
-// on MI355X at 256 M elements: F = 300 / 600 / 1000 5.2-5.9 -> 6.0-6.2 TB/s, F = 602 4.7-5.2 -> 5.6-5.9 TB/s; rows that
-// are whole passes (F = 64 ... 1024 in steps of the lane-group width) gain nothing from it and keep the direct stores.
-static bool quant_staged_output() {
-    static const bool on = [] { const char *e = getenv("SGNN_QUANT_STAGED"); return !(e && e[0] == '0'); }();
-    return on;
-}
-
+// bytes through the wave-private LDS stage.  Measured on MI355X at 256 M elements against stores straight from the
+// lanes: F = 300 / 600 / 1000 5.2-5.9 -> 6.0-6.2 TB/s, F = 602 4.7-5.2 -> 5.6-5.9 TB/s; rows that are whole passes
+// (F = 64 ... 1024 in steps of the lane-group width) gain nothing from it and keep the direct stores.
 template <int BITS, int NV, int L>
 static void launch_quant16_ragged(const RowsArgs &a, hipStream_t st) {
     constexpr int RL = NV >= 4 ? 1 : 4 / NV;
@@ -1993,12 +1995,8 @@ static void launch_quant16_ragged(const RowsArgs &a, hipStream_t st) {
     const int n_units = (int)((padded + RW * RL - 1) / (RW * RL));
     const int nb = (n_units + kQBlock / 64 - 1) / (kQBlock / 64);
     ProfScope prof(K_QUANT_PACK_ROWS, st);
-    if (quant_staged_output())
-        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L, true, true>), dim3(nb), dim3(kQBlock), 0, st,
-                           a.x_in, a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
-    else
-        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L, true>), dim3(nb), dim3(kQBlock), 0, st, a.x_in,
-                           a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
+    hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L, true, true>), dim3(nb), dim3(kQBlock), 0, st,
+                       a.x_in, a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
 // The same for rows of 1025 ... 2560 floats: a wavefront holds four rows in registers, NV vectors per lane each.
@@ -2052,12 +2050,9 @@ static void launch_quant16(const RowsArgs &a, hipStream_t st) {
     else if (a.F == 4 * L * NV)
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, true, L>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
                            a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
-    else if (quant_staged_output())
+    else
         hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L, false, true>), dim3(nb), dim3(kQBlock), 0, st,
                            a.x_in, a.q_out, a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
-    else
-        hipLaunchKernelGGL((quant_pack_rows16_kernel<BITS, NV, RL, false, false, L>), dim3(nb), dim3(kQBlock), 0, st, a.x_in, a.q_out,
-                           a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, n_units);
 }
 
 // Lane-slot shape of the stream quantizer for rows of F floats: NV vectors per lane (one of the instantiated
@@ -2140,14 +2135,11 @@ static void launch_dequant_flat(const RowsArgs &a, int64_t n_rows, hipStream_t s
     const int G = a.F / 4;
     // With several segments and sub-byte codes every wavefront first looks its segment up, and the shortest waves
     // lose: 1 M x 256 int2 in eight segments 0.194 ms with one store per wave, 0.169 with two, 0.160 with four
-    // (one segment: 0.155 / 0.171 / 0.170); int4 0.199 / 0.162 / 0.162.  SGNN_DEQUANT_R=1/2/4 forces a shape.
-    const char *e = getenv("SGNN_DEQUANT_R");
-    int r = e ? atoi(e) : 0;
-    if (r != 1 && r != 2 && r != 4) {
-        if (BITS == 8) r = 2;
-        else if (a.P <= 1) r = (G & (G - 1)) == 0 ? 1 : BITS == 2 ? 4 : 2;
-        else r = BITS == 2 && a.F <= 256 ? 4 : 2;
-    }
+    // (one segment: 0.155 / 0.171 / 0.170); int4 0.199 / 0.162 / 0.162.
+    int r;
+    if (BITS == 8) r = 2;
+    else if (a.P <= 1) r = (G & (G - 1)) == 0 ? 1 : BITS == 2 ? 4 : 2;
+    else r = BITS == 2 && a.F <= 256 ? 4 : 2;
     if (r == 4) launch_dequant_flat_r<BITS, 4>(a, n_rows, st);
     else if (r == 2) launch_dequant_flat_r<BITS, 2>(a, n_rows, st);
     else launch_dequant_flat_r<BITS, 1>(a, n_rows, st);
@@ -2181,10 +2173,8 @@ static void launch_dequant_flat_ragged_r(const RowsArgs &a, int64_t n_rows, hipS
 
 template <int BITS, int VEC>
 static void launch_dequant_flat_ragged(const RowsArgs &a, int64_t n_rows, hipStream_t st) {
-    const char *e = getenv("SGNN_DEQUANT_R");
-    const int r = e ? atoi(e) : 0;
     // several segments and sub-byte codes: four stores per wavefront per segment lookup (see launch_dequant_flat)
-    if (r == 4 || (r != 2 && BITS != 8 && a.P > 1)) launch_dequant_flat_ragged_r<BITS, VEC, 4>(a, n_rows, st);
+    if (BITS != 8 && a.P > 1) launch_dequant_flat_ragged_r<BITS, VEC, 4>(a, n_rows, st);
     else launch_dequant_flat_ragged_r<BITS, VEC, 2>(a, n_rows, st);
 }
 
@@ -2203,45 +2193,39 @@ static void launch_rows_wide(const RowsArgs &a, hipStream_t st) {
 template <int BITS, int VEC>
 static void dispatch_rows_shape(int nvec, const RowsArgs &a, hipStream_t st) {
     if constexpr (VEC == 4) {
-        if (a.quantize && a.layout16) {
-            // rows of up to 128 floats: eight lanes per row (SGNN_QUANT_LAYOUT8=0: sixteen, for comparison)
-            static const bool layout8 = [] { const char *e = getenv("SGNN_QUANT_LAYOUT8"); return !(e && e[0] == '0'); }();
-            // (with the staged output also for rows of 17 ... 31 vectors, whose groups have idle lanes either way:
-            // F = 72 / 80 3.8-4.7 -> 4.7-5.7 TB/s, F = 100 / 112 +3 ... 6 %)
-            if (layout8) {
-                if (nvec <= 1) return launch_quant16<BITS, 1, 1>(a, st);
-                if (nvec <= 2) return launch_quant16<BITS, 1, 2>(a, st);
-                if (nvec <= 4) return launch_quant16<BITS, 1, 4>(a, st);
-                // rows of 5 ... 12 vectors other than the whole eight-lane pass F = 32: four lanes per row (F = 20 / 24:
-                // 3.2-4.3 -> 4.1-5.2 TB/s, F = 28 ... 48: +4 ... 17 %; from 13 vectors on eight lanes win, F = 52 ... 64 by
-                // 6 ... 18 %).  SGNN_QUANT_LAYOUT4=0: eight lanes for all of them.
-                static const bool layout4 = [] { const char *e = getenv("SGNN_QUANT_LAYOUT4"); return !(e && e[0] == '0'); }();
-                if (layout4 && nvec <= 8 && a.F != 32) return launch_quant16<BITS, 2, 4>(a, st);
-                if (layout4 && nvec > 8 && nvec <= 12) return launch_quant16<BITS, 4, 4>(a, st);
-                if (nvec <= 8) return launch_quant16<BITS, 1, 8>(a, st);
-                if (nvec <= 16) return launch_quant16<BITS, 2, 8>(a, st);
-                if (nvec <= 32) return launch_quant16<BITS, 4, 8>(a, st);
-            }
-            if (nvec <= 16) return launch_quant16<BITS, 1>(a, st);
-            if (nvec <= 32) return launch_quant16<BITS, 2>(a, st);
+        if (a.quantize) {
+            // rows of up to 128 floats: eight lanes per row (with the staged output also for rows of 17 ... 31 vectors,
+            // whose groups have idle lanes either way: F = 72 / 80 3.8-4.7 -> 4.7-5.7 TB/s, F = 100 / 112 +3 ... 6 %)
+            if (nvec <= 1) return launch_quant16<BITS, 1, 1>(a, st);
+            if (nvec <= 2) return launch_quant16<BITS, 1, 2>(a, st);
+            if (nvec <= 4) return launch_quant16<BITS, 1, 4>(a, st);
+            // rows of 5 ... 12 vectors other than the whole eight-lane pass F = 32: four lanes per row (F = 20 / 24:
+            // 3.2-4.3 -> 4.1-5.2 TB/s, F = 28 ... 48: +4 ... 17 %; from 13 vectors on eight lanes win, F = 52 ... 64 by
+            // 6 ... 18 %)
+            if (nvec <= 8 && a.F != 32) return launch_quant16<BITS, 2, 4>(a, st);
+            if (nvec > 8 && nvec <= 12) return launch_quant16<BITS, 4, 4>(a, st);
+            if (nvec <= 8) return launch_quant16<BITS, 1, 8>(a, st);
+            if (nvec <= 16) return launch_quant16<BITS, 2, 8>(a, st);
+            if (nvec <= 32) return launch_quant16<BITS, 4, 8>(a, st);
             if (nvec <= 64) return launch_quant16<BITS, 4>(a, st);
             if (nvec <= 128) return launch_quant16<BITS, 8>(a, st);
             if (nvec <= 160) return launch_quant16<BITS, 10>(a, st);
             if (nvec <= 256) return launch_quant16<BITS, 16>(a, st);
         }
     }
-    if (nvec <= 16) return launch_rows<BITS, VEC, 16, 1>(a, st);
-    if (nvec <= 32) return launch_rows<BITS, VEC, 32, 1>(a, st);
-    if (nvec <= 64) return launch_rows<BITS, VEC, 64, 1>(a, st);
-    if (nvec <= 128) return launch_rows<BITS, VEC, 64, 2>(a, st);
+    constexpr int kDq = VEC == 4 ? 1 : 0;   // (VEC == 4: the quantizer has returned above for rows of up to 256 vectors)
+    if (nvec <= 16) return launch_rows<BITS, VEC, 16, 1, kDq>(a, st);
+    if (nvec <= 32) return launch_rows<BITS, VEC, 32, 1, kDq>(a, st);
+    if (nvec <= 64) return launch_rows<BITS, VEC, 64, 1, kDq>(a, st);
+    if (nvec <= 128) return launch_rows<BITS, VEC, 64, 2, kDq>(a, st);
     if constexpr (VEC == 4) {
-        if (nvec <= 192) return launch_rows<BITS, VEC, 64, 3>(a, st);
-        if (nvec <= 256) return launch_rows<BITS, VEC, 64, 4>(a, st);
+        if (nvec <= 192) return launch_rows<BITS, VEC, 64, 3, 1>(a, st);
+        if (nvec <= 256) return launch_rows<BITS, VEC, 64, 4, 1>(a, st);
         if (a.quantize) {  // rows of up to 2048 floats still fit a wavefront's registers (four rows, NV vectors per lane each)
-            if (nvec <= 320) return launch_rows<BITS, VEC, 64, 5>(a, st);
-            if (nvec <= 384) return launch_rows<BITS, VEC, 64, 6>(a, st);
-            if (nvec <= 512) return launch_rows<BITS, VEC, 64, 8>(a, st);
-            if (nvec <= 640) return launch_rows<BITS, VEC, 64, 10>(a, st);
+            if (nvec <= 320) return launch_rows<BITS, VEC, 64, 5, 2>(a, st);
+            if (nvec <= 384) return launch_rows<BITS, VEC, 64, 6, 2>(a, st);
+            if (nvec <= 512) return launch_rows<BITS, VEC, 64, 8, 2>(a, st);
+            if (nvec <= 640) return launch_rows<BITS, VEC, 64, 10, 2>(a, st);
         }
     } else {
         if (nvec <= 256) return launch_rows<BITS, VEC, 64, 4>(a, st);
@@ -2301,7 +2285,7 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
         if (bits == 8) even ? launch_dequant_flat_ragged<8, 2>(a, n_rows, st) : launch_dequant_flat_ragged<8, 1>(a, n_rows, st);
         else if (bits == 4) even ? launch_dequant_flat_ragged<4, 2>(a, n_rows, st) : launch_dequant_flat_ragged<4, 1>(a, n_rows, st);
         else even ? launch_dequant_flat_ragged<2, 2>(a, n_rows, st) : launch_dequant_flat_ragged<2, 1>(a, n_rows, st);
-    } else if (a.quantize && vec != 4 && a.layout16 && !a.exact_division && a.F <= 1024) {
+    } else if (a.quantize && vec != 4 && !a.exact_division && a.F <= 1024) {
         if (bits == 8) dispatch_quant16_ragged<8>(a, st);
         else if (bits == 4) dispatch_quant16_ragged<4>(a, st);
         else dispatch_quant16_ragged<2>(a, st);
@@ -2362,7 +2346,6 @@ static int quant_pack_rows_impl(const RowSrc &src, uint8_t *q, void *params, int
     a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = true;
     a.single_rows = P == 1 ? n_rows : -1;
     { const char *e = getenv("SGNN_QUANT_EXACT_DIV"); a.exact_division = e && e[0] == '1'; }
-    { const char *e = getenv("SGNN_QUANT_LAYOUT16"); a.layout16 = !(e && e[0] == '0'); }
     return run_rows(a, bits, n_rows, src.x, q, (hipStream_t)stream);
 }
 
@@ -2375,7 +2358,6 @@ static int unpack_dequant_rows_impl(const uint8_t *q, float *x, const void *para
     a.q_in = q; a.x_out = x; a.params = ParamBuf{const_cast<void *>(params), params_bf16}; a.seg = seg; a.pseg = pseg;
     a.P = P; a.n_packed = (int)n_packed_rows; a.F = (int)F; a.quantize = false;
     a.single_rows = P == 1 ? n_rows : -1;
-    { const char *e = getenv("SGNN_QUANT_LAYOUT16"); a.layout16 = !(e && e[0] == '0'); }
     { const char *e = getenv("SGNN_DEQUANT_FLAT"); a.flat = !(e && e[0] == '0'); }
     return run_rows(a, bits, n_rows, x, q, (hipStream_t)stream);
 }
@@ -2418,8 +2400,7 @@ extern "C" int sgnn_quant_v1_f32(const float *x, uint8_t *q, const int64_t *rang
     const dim3 grid((uint32_t)nb), block(kQBlock);
     const auto grid_r = [&](int rows) { return dim3((uint32_t)((nb + rows - 1) / rows)); };
     hipStream_t st = (hipStream_t)stream;
-    static const bool group_layout = [] { const char *e = getenv("SGNN_QUANT_V1_GROUPS"); return !(e && e[0] == '0'); }();
-    if (group_layout && F % 4 == 0 && F <= 512 && aligned(x, 16)) {   // (wider rows: a wavefront per row is faster)
+    if (F % 4 == 0 && F <= 512 && aligned(x, 16)) {   // (wider rows: a wavefront per row is faster)
         const auto grid_g = [&](int rows_per_wave) {
             const int64_t waves = (n + rows_per_wave - 1) / rows_per_wave;
             return dim3((uint32_t)((waves + kQBlock / 64 - 1) / (kQBlock / 64)));
@@ -2453,18 +2434,12 @@ extern "C" int sgnn_dequant_v1_f32(const uint8_t *q, float *x, const int64_t *ra
     const dim3 grid((uint32_t)nb), block(kQBlock);
     const auto grid_r = [&](int rows) { return dim3((uint32_t)((nb + rows - 1) / rows)); };
     hipStream_t st = (hipStream_t)stream;
-    // narrow rows (a wavefront per row leaves lanes idle) and rows beyond the vector kernel's width: flat output
-    // (SGNN_DEQUANT_V1_FLAT=0 / 1: never / at every width, for comparison)
-    static const int flat_mode = [] { const char *e = getenv("SGNN_DEQUANT_V1_FLAT"); return e ? atoi(e) : -1; }();
-    if (F % 4 == 0 && aligned(x, 16) && (flat_mode == 1 || (flat_mode != 0 && (F <= 128 || F > 1024)))) {
-        // stores per wavefront: four measured 1-3 % above two and 10-15 % above one (SGNN_DEQUANT_V1_R=1/2/4 forces one)
-        const char *e = getenv("SGNN_DEQUANT_V1_R");
-        const int r = e ? atoi(e) : 4;
+    // narrow rows (a wavefront per row leaves lanes idle) and rows beyond the vector kernel's width: flat output,
+    // four stores per wavefront (measured 1-3 % above two and 10-15 % above one)
+    if (F % 4 == 0 && aligned(x, 16) && (F <= 128 || F > 1024)) {
         const int64_t n_vec = n * (F / 4);
-        const auto waves = [&](int R) { return dim3((uint32_t)(((n_vec + R * 64 - 1) / (R * 64) + kQBlock / 64 - 1) / (kQBlock / 64))); };
-        if (r == 2) hipLaunchKernelGGL((dequant_v1_flat_kernel<2>), waves(2), block, 0, st, q, x, range, params, n_vec, (int)(F / 4));
-        else if (r == 1) hipLaunchKernelGGL((dequant_v1_flat_kernel<1>), waves(1), block, 0, st, q, x, range, params, n_vec, (int)(F / 4));
-        else hipLaunchKernelGGL((dequant_v1_flat_kernel<4>), waves(4), block, 0, st, q, x, range, params, n_vec, (int)(F / 4));
+        const dim3 waves((uint32_t)(((n_vec + 4 * 64 - 1) / (4 * 64) + kQBlock / 64 - 1) / (kQBlock / 64)));
+        hipLaunchKernelGGL((dequant_v1_flat_kernel<4>), waves, block, 0, st, q, x, range, params, n_vec, (int)(F / 4));
     } else if (F % 4 == 0 && F <= 1024 && aligned(x, 16)) {
         if (F <= 256) hipLaunchKernelGGL((dequant_v1_vec_kernel<1, 4>), grid_r(4), block, 0, st, q, x, range, params, n, (int)F);
         else if (F <= 512) hipLaunchKernelGGL((dequant_v1_vec_kernel<2, 2>), grid_r(2), block, 0, st, q, x, range, params, n, (int)F);

@@ -102,6 +102,8 @@ __device__ __forceinline__ void fetch_row(Fetched<VEC, NV, BITS> &r, const Dense
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             if (!act[v]) continue;
+            // (ordinary loads: marking the code rows non-temporal, to keep the (zero_point, scale) table in the L2, cut the
+            // fetched bytes by 4 % and cost 10 % of the kernel's time: rows that share a packed row hit in cache)
             if constexpr (VEC == 4) r.w[v] = *reinterpret_cast<const uint32_t *>(qr + off[v]);
             else if constexpr (VEC == 2) r.w[v] = *reinterpret_cast<const uint16_t *>(qr + off[v]);
             else r.w[v] = qr[off[v]];
@@ -1092,7 +1094,6 @@ struct PieceArgs {
     const int32_t *col_long; const int32_t *eperm; const float *val; float *partial;
     const int4 *cls_work;
     int max_cls_items; int F;
-    hipStream_t side; hipEvent_t ev_fork, ev_join;  // side != null: long rows run beside the short rows
 };
 struct FinalArgs {
     const int32_t *long_rows; const int32_t *long_pbeg; const float *partial; float *out; int n_long;
@@ -1102,14 +1103,9 @@ struct FinalArgs {
 template <int VEC, int G, int NV, int BITS>
 static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &f, hipStream_t st) {
     constexpr int GPB = kBlock / G;
-    // The long rows (pieces + final sum) and the short rows write disjoint output rows.  With a side
-    // stream they are issued side by side: fork after the caller's earlier work, join before returning.
+    // The long rows (pieces + final sum) and the short rows write disjoint output rows; all kernels go to the
+    // caller's stream one after the other (issuing the long rows on a second stream measured -1 ... +5 %).
     hipStream_t ls = st;
-    if (s.side != nullptr && f.n_long > 0 && a.n_chunks > 0) {
-        (void)hipEventRecord(s.ev_fork, st);
-        (void)hipStreamWaitEvent(s.side, s.ev_fork, 0);
-        ls = s.side;
-    }
     const char *hub_env = getenv("SGNN_SPMM_HUB_LDS");
     const bool hub_lds = hub_env != nullptr && atoi(hub_env) != 0;
     if (BITS == 0 && hub_lds && f.n_long > 0) {
@@ -1144,10 +1140,6 @@ static void launch_all(const ShortArgs &a, const PieceArgs &s, const FinalArgs &
         ProfScope prof(K_SPMM_EMPTY_ROWS, st, a.prof);
         hipLaunchKernelGGL((spmm_empty_rows_kernel<VEC, G, NV>), dim3(nb), dim3(kBlock), 0, st, a.empty_rows, a.n_empty,
                            a.out, a.F, a.ldo, a.accumulate, a.row_div);
-    }
-    if (ls != st) {
-        (void)hipEventRecord(s.ev_join, ls);
-        (void)hipStreamWaitEvent(st, s.ev_join, 0);
     }
 }
 
@@ -1281,8 +1273,6 @@ struct sgnn_spmm_plan {
     int32_t *long_pbeg = nullptr;   // [n_long + 1] first piece of each long row
     int32_t *col_long = nullptr;    // [long_edges] columns regrouped by class inside each long row
     int32_t *eperm = nullptr;       // [long_edges] original edge index of each regrouped edge
-    hipStream_t side = nullptr;     // long rows run here, beside the short rows on the caller's stream
-    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
     float *val_long = nullptr;      // [long_edges] bound edge values in regrouped order (sgnn_spmm_plan_bind_values)
     const float *bound_val = nullptr;  // the caller's array val_long was taken from
     int32_t *eslot_csr = nullptr;      // [nnz] row_slot[col[e]] in CSR order (sgnn_spmm_plan_bind_row_slots)
@@ -1322,11 +1312,8 @@ static int build_chunks(sgnn_spmm_plan *p, int which, hipStream_t st) {
     // About 64 edges per chunk on large matrices (measured plateau 32-96 on the power-law graph; 128
     // is 4 % slower, 256 15 %), and never so few chunks that the chip idles: a small matrix is cut
     // finer, down to 16 edges, until there are about kChunkGroupsWanted lane groups for the 256 CUs.
-    int target = env_int("SGNN_SPMM_CHUNK_EDGES", 0);
-    if (target <= 0) {
-        const int64_t short_edges = p->nnz - p->long_edges;
-        target = (int)std::min<int64_t>(64, std::max<int64_t>(16, short_edges / env_int("SGNN_SPMM_CHUNK_GROUPS", kChunkGroupsWanted)));
-    }
+    const int64_t short_edges = p->nnz - p->long_edges;
+    const int target = (int)std::min<int64_t>(64, std::max<int64_t>(16, short_edges / kChunkGroupsWanted));
     const std::vector<int64_t> &rp = p->h_rowptr;
     std::vector<int4> out;
     const int64_t M = p->M;
@@ -1367,9 +1354,6 @@ extern "C" int sgnn_spmm_plan_destroy(sgnn_spmm_plan *p) {
     (void)hipFree(p->val_long);
     (void)hipFree(p->eslot_csr);
     (void)hipFree(p->eslot_long);
-    if (p->ev_fork) (void)hipEventDestroy(p->ev_fork);
-    if (p->ev_join) (void)hipEventDestroy(p->ev_join);
-    if (p->side) (void)hipStreamDestroy(p->side);
     (void)hipFree(p->partial);
     (void)hipFree(p->empty_rows);
     for (int i = 0; i < 3; ++i) (void)hipFree(p->chunks[i]);
@@ -1531,7 +1515,7 @@ static int plan_create_impl(sgnn_spmm_plan *p, const int64_t *rowptr, const void
         // and the workgroups running together on an XCD sweep the dense matrix band by band instead of
         // touching all of it at once (measured: -3 % piece-kernel time on the power-law graph; sorting by
         // the exact first column instead piles the hot low columns into the same moment and costs +5 %).
-        if (p->partitioned && env_int("SGNN_SPMM_PIECE_ORDER", 1) >= 1) {
+        if (p->partitioned) {
             for (int c = 0; c < kNumXCD; ++c)
                 std::stable_sort(cls_items[c].begin(), cls_items[c].end(),
                                  [&](int32_t a, int32_t b) { return item_key[a] < item_key[b]; });
@@ -1616,8 +1600,8 @@ extern "C" int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int
     SGNN_REQUIRE(nnz == 0 || col != nullptr, "col is null with nnz=%lld", (long long)nnz);
     sgnn_spmm_plan *p = new sgnn_spmm_plan();
     p->M = M; p->K = K; p->nnz = nnz;
-    p->long_thresh = long_row_threshold > 0 ? long_row_threshold : env_int("SGNN_SPMM_LONG_THRESHOLD", kDefaultLongThreshold);
-    p->piece_edges = piece_edges > 0 ? piece_edges : env_int("SGNN_SPMM_PIECE_EDGES", kDefaultPieceEdges);
+    p->long_thresh = long_row_threshold > 0 ? long_row_threshold : kDefaultLongThreshold;
+    p->piece_edges = piece_edges > 0 ? piece_edges : kDefaultPieceEdges;
     const int64_t part_cap = part_edge_cap();
     const int rc = nnz <= part_cap ? plan_create_impl(p, rowptr, col, col_is_i64, (hipStream_t)stream)
                                    : plan_create_parts(p, rowptr, col, col_is_i64, part_cap, (hipStream_t)stream);
@@ -2182,13 +2166,7 @@ static int spmm_run(sgnn_spmm_plan *p, const float *val, const DenseSrc &dense, 
     SGNN_REQUIRE(p->n_chunks[which] >= 0, "plan has no chunk list for this feature width (plan creation failed?)");
     ShortArgs a{p->rowptr, p->col, val, dense, out, p->chunks[which], (int)p->n_chunks[which], p->empty_rows,
                 (int)p->n_empty, (int)F, ldo, accumulate, row_div, scratch == nullptr};
-    if (scratch == nullptr && p->side == nullptr && p->n_long > 0 && env_int("SGNN_SPMM_OVERLAP", 0) != 0) {
-        SGNN_HIP_CHECK(hipStreamCreateWithFlags(&p->side, hipStreamNonBlocking));  // default priority
-        SGNN_HIP_CHECK(hipEventCreateWithFlags(&p->ev_fork, hipEventDisableTiming));
-        SGNN_HIP_CHECK(hipEventCreateWithFlags(&p->ev_join, hipEventDisableTiming));
-    }
-    PieceArgs s{p->col_long, p->eperm, val, partial, p->cls_work, p->max_cls_items, (int)F,
-                scratch == nullptr ? p->side : nullptr, p->ev_fork, p->ev_join};
+    PieceArgs s{p->col_long, p->eperm, val, partial, p->cls_work, p->max_cls_items, (int)F};
     if (val != nullptr && val == p->bound_val && p->val_long != nullptr) {
         s.eperm = nullptr;   // values already sit in regrouped order: contiguous reads, no indirection
         s.val = p->val_long;
