@@ -140,10 +140,17 @@ int sgnn_spmm_csr_f32(sgnn_spmm_plan *plan, const float *val, const float *x, fl
  *   - every call on one GPU shares that GPU's scratch: two calls whose kernels may overlap in time
  *     (different streams, different host threads) race on it.  Calls queued on one stream are safe.
  *     Nothing in the scratch has to start at zero: each call writes every partial it later reads;
- *   - a matrix that sgnn_spmm_plan_schedule reports as band-scheduled runs that schedule here only if an
- *     earlier sgnn_spmm_csr_f32 call has already built it for a width >= F and the same kind of weights
- *     (val given or NULL: the two cut the bands into different chunks); building allocates.  Otherwise the
- *     row-class kernels run, whose long rows are summed per piece instead of in one chain. */
+ *   - a matrix that sgnn_spmm_plan_schedule reports as band-scheduled runs that schedule here only if earlier
+ *     sgnn_spmm_csr_f32 calls on this plan have already built everything it needs (building allocates): the
+ *     band-major edge copy for this product's band width (info[1] of sgnn_spmm_plan_schedule; every F > 512
+ *     shares one, narrower products have one per padded slice width), a restaged-operand workspace at least as
+ *     large as this F needs, and the chunk list for the same kind of weights (val given or NULL: the two cut the
+ *     bands into different chunks).  The simple way to guarantee that is one sgnn_spmm_csr_f32 call with the same
+ *     F and the same kind of weights beforehand.  Otherwise the row-class kernels run: same result on rows of up
+ *     to 128 edges, bit for bit; longer rows are summed per piece instead of in one chain (within the fp32
+ *     tolerance, not the same bits);
+ *   - the scratch address is looked up when a plan is created, so the call itself performs no lazy symbol
+ *     lookup, and it records no profiling events (sgnn_profile_enable does not see its kernels). */
 int sgnn_spmm_csr_f32_noalloc(sgnn_spmm_plan *plan, const float *val, const float *x, float *out,
                               int64_t F, int64_t ldx, int64_t ldo, int accumulate,
                               const float *row_div, sgnn_stream_t stream);

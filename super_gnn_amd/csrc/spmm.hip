@@ -1609,6 +1609,10 @@ extern "C" int sgnn_spmm_plan_create(const int64_t *rowptr, const void *col, int
         sgnn_spmm_plan_destroy(p);
         return rc;
     }
+    // The non-allocating entry point must not be the first to look the scratch array's address up (a lazy symbol
+    // lookup inside what may be a graph capture): plan creation, which synchronises and allocates anyway, does it.
+    float *scratch = nullptr;
+    (void)scratch_for_current_device(&scratch);
     *plan_out = p;
     return SGNN_OK;
 }

@@ -94,3 +94,91 @@ def test_refuses_what_does_not_fit_the_scratch():
         assert lib.sgnn_spmm_csr_f32_noalloc(plan._h, w.data_ptr(), x2.data_ptr(), o2.data_ptr(), F2, F2, F2, 1, None, st) == 0
         torch.cuda.synchronize()
         assert torch.equal(o1, o2)
+
+
+def _call(lib, check, fn, plan, w, x, out, F, accumulate=1, div=None):
+    check(fn(plan._h, w.data_ptr() if w is not None else None, x.data_ptr(), out.data_ptr(), F, F, F, accumulate,
+             div.data_ptr() if div is not None else None, torch.cuda.current_stream().cuda_stream))
+
+
+def test_allocates_nothing_and_replays_from_a_captured_graph():
+    import super_gnn_amd  # noqa: F401
+    from super_gnn_amd import supergnn_ops as ops
+    from super_gnn_amd._lib import lib, check
+    dev = torch.device("cuda:0")
+    M, K, F = 5000, 4000, 128
+    rowptr, col, val = random_csr(M, K, 15, seed=311, empty_frac=0.1, hubs=30, hub_deg=3000)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    w = torch.from_numpy(val).to(dev)
+    x = torch.randn(K, F, generator=torch.Generator().manual_seed(1)).to(dev)
+    want = torch.zeros(M, F, device=dev)
+    _call(lib, check, lib.sgnn_spmm_csr_f32, plan, w, x, want, F)
+    out = torch.zeros(M, F, device=dev)
+    _call(lib, check, lib.sgnn_spmm_csr_f32_noalloc, plan, w, x, out, F)      # warm
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        out.zero_()
+        _call(lib, check, lib.sgnn_spmm_csr_f32_noalloc, plan, w, x, out, F)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "device memory moved during non-allocating calls"
+    assert torch.equal(out, want)
+    # under capture (an allocation or a lazy symbol lookup would invalidate the capture), then replays with eager work between
+    graph = torch.cuda.CUDAGraph()
+    gout = torch.zeros(M, F, device=dev)
+    with torch.cuda.graph(graph):
+        gout.zero_()
+        _call(lib, check, lib.sgnn_spmm_csr_f32_noalloc, plan, w, x, gout, F)
+    for i in range(3):
+        gout.fill_(float(i + 7))
+        out.normal_()                 # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(gout, want), f"replay {i}"
+
+
+@pytest.mark.parametrize("switch,value,F", [("SGNN_SPMM_BAND", "1", 602), ("SGNN_SPMM_BAND", "1", 128),
+                                              ("SGNN_SPMM_SLICE", "128", 256), ("SGNN_SPMM_PART_EDGES", "20000", 64)])
+def test_other_schedules_through_the_non_allocating_entry_point(switch, value, F, monkeypatch):
+    """Band schedule (taken here only once the allocating entry point has built it), feature slices (the scratch limit
+    applies per slice) and row-block plans: the non-allocating call gives the allocating call's bits."""
+    import super_gnn_amd  # noqa: F401
+    from super_gnn_amd import supergnn_ops as ops
+    from super_gnn_amd._lib import lib, check
+    dev = torch.device("cuda:0")
+    monkeypatch.setenv(switch, value)
+    if switch == "SGNN_SPMM_BAND":
+        monkeypatch.setenv("SGNN_SPMM_BAND_COLS", "200")
+    M, K = 3000, 2500
+    rowptr, col, val = random_csr(M, K, 20, seed=F, empty_frac=0.1, hubs=12, hub_deg=2000)
+    deg = np.diff(rowptr)
+    plan = ops.SpmmPlan(torch.from_numpy(rowptr).to(dev), torch.from_numpy(col).to(dev), K)
+    w = torch.from_numpy(val).to(dev)
+    xn = np.random.default_rng(F).standard_normal((K, F), dtype=np.float32)
+    x = torch.from_numpy(xn).to(dev)
+    short = torch.from_numpy(deg <= 128).to(dev)
+    if switch == "SGNN_SPMM_BAND":
+        # nothing built yet: the row-class kernels answer -- reference order on short rows, the fp32 bar on long ones
+        first = torch.zeros(M, F, device=dev)
+        _call(lib, check, lib.sgnn_spmm_csr_f32_noalloc, plan, w, x, first, F)
+        ref = np.zeros((M, F), np.float32)
+        orc.spmm_accumulate(rowptr, col, val, xn, ref)
+        assert np.array_equal(first.cpu().numpy()[deg <= 128], ref[deg <= 128])
+        assert_spmm_close(first.cpu().numpy(), ref, orc.spmm_f64(rowptr, col, val, xn, None), abs_sum64(rowptr, col, val, xn, None),
+                          deg, what="noalloc before the band schedule exists")
+    want = torch.zeros(M, F, device=dev)
+    _call(lib, check, lib.sgnn_spmm_csr_f32, plan, w, x, want, F)          # builds what the schedule needs
+    got = torch.zeros(M, F, device=dev)
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    _call(lib, check, lib.sgnn_spmm_csr_f32_noalloc, plan, w, x, got, F)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "device memory moved during the non-allocating call"
+    assert torch.equal(got, want), f"{switch}={value}, F={F}"
+    assert torch.equal(got[short], want[short])
+    if switch == "SGNN_SPMM_BAND":
+        assert plan.schedule(F)["band"] == 1
+        ref = np.zeros((M, F), np.float32)
+        orc.spmm_accumulate(rowptr, col, val, xn, ref)
+        assert np.array_equal(got.cpu().numpy(), ref), "band schedule through the non-allocating call: CSR order on every row"
