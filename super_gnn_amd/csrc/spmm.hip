@@ -24,6 +24,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <functional>
+#include <list>
 #include <memory>
 #include <mutex>
 #include <vector>
@@ -1251,7 +1252,7 @@ struct BandSchedule {
         int4 *chunks = nullptr;            // all bands' chunk records (four int4 each, see spmm_band_kernel), band after band
         std::vector<int64_t> chunk_off;    // [n_bands + 1] each band's range of chunks
     };
-    std::vector<ChunkList> lists;
+    std::list<ChunkList> lists;   // (a list: launches keep pointers to its elements while further lists are built)
     ~BandSchedule() {
         (void)hipFree(col_bm); (void)hipFree(eperm_bm); (void)hipFree(val_bm);
         for (ChunkList &l : lists) (void)hipFree(l.chunks);
@@ -1659,6 +1660,7 @@ struct BandShape {
 // is eight of them, one per XCD.  Wider products run as consecutive windows over the same bands: the reference
 // tiles the feature axis of every row in the same way (spmm.cpp:502-510).
 constexpr int kBandWindowCols = 512;
+constexpr int kBandMinGroup = 8;   // lanes per group, at least (lane i of a group holds row i's offset: up to 7 rows per chunk)
 constexpr int kMaxBandSchedules = 3;   // band widths a plan keeps schedules for (each holds ~12 bytes per edge)
 constexpr int kBandMaxWindows = 64;
 
@@ -1679,9 +1681,19 @@ static BandShape band_window_shape(const sgnn_spmm_plan *p, int f0, int Fw, bool
     b.F = Fw;
     b.even = even_out && Fw % 2 == 0 && Fw >= 4 && f0 % 2 == 0;
     const int nvec = (Fw + 3) / 4;
-    if (windowed) {   // at most 16 float4 per slice
-        b.n_slices = 1;
-        while (b.n_slices < kNumXCD && (nvec + b.n_slices - 1) / b.n_slices > 16) b.n_slices *= 2;
+    if (windowed) {
+        // At most 16 float4 per slice (the bands are sized for 64-float slices).  A gather instruction costs the same
+        // whatever its lanes carry, so the cut that needs the fewest of them wins: slices / (lane groups per wavefront).
+        // A remainder of 90 columns takes 2 slices of 12 float4, five lane groups per wavefront (0.4 instructions per
+        // edge against 0.5 for 2 slices in groups of 16 lanes or 4 slices of 6 float4).
+        double best = 1e30;
+        for (int n = 1; n <= kNumXCD; n *= 2) {
+            const int vps = (nvec + n - 1) / n;
+            if (vps > 16) continue;
+            const int g = std::max(kBandMinGroup, (4 * vps + 15) / 16 * 4);
+            const double cost = (double)n / (64 / g);
+            if (cost < best - 1e-9) { best = cost; b.n_slices = n; }
+        }
     } else {
         b.n_slices = kNumXCD;
         while (b.n_slices > 1 && (nvec + b.n_slices - 1) / b.n_slices < 16) b.n_slices /= 2;
@@ -1690,7 +1702,7 @@ static BandShape band_window_shape(const sgnn_spmm_plan *p, int f0, int Fw, bool
     }
     b.slice_floats = 4 * ((nvec + b.n_slices - 1) / b.n_slices);
     b.slice_pad = (b.slice_floats + 15) / 16 * 16;
-    b.G = std::max(16, std::min(64, b.slice_pad / 4));
+    b.G = std::max(windowed ? kBandMinGroup : 16, std::min(64, b.slice_pad / 4));
     int cols = env_int("SGNN_SPMM_BAND_COLS", 0);
     if (cols <= 0) {
         const int pad = windowed ? 64 : b.slice_pad;   // windows share the bands of a full 64-float slice
@@ -1877,7 +1889,11 @@ static BandCaps band_chunk_caps(const sgnn_spmm_plan *p, const BandShape &sh, bo
     const int gpb = (kBandBlock / 64) * (64 / sh.G);
     const int64_t budget = (int64_t)80 * 1024 / gpb, row_bytes = (int64_t)sh.G * 16, bpe = weighted ? 8 : 4;
     const int64_t avg = std::max<int64_t>(1, p->nnz / std::max<int64_t>(1, p->M) / std::max(1, sh.n_bands));
-    const int rows_lim = weighted ? kBandRowsWeighted : kBandRows, edges_lim = weighted ? kBandEdgesWeighted : kBandEdges;
+    // (the kernel stages a chunk's pairs in a fixed number of rounds of 4 * G pairs: narrow groups stage fewer)
+    constexpr int kRoundsU = (kBandEdges + kBandPad + 63) / 64, kRoundsW = (kBandEdgesWeighted + kBandPad + 63) / 64;
+    const int rows_lim = weighted ? kBandRowsWeighted : kBandRows;
+    const int edges_lim = std::min(weighted ? kBandEdgesWeighted : kBandEdges,
+                                   ((weighted ? kRoundsW : kRoundsU) * 4 * sh.G - kBandPad - kBandWindow) / 16 * 16);
     const int rows_max = std::min(rows_lim, sh.G - 1);   // lane i of a group holds row i's offset, lane `rows` the end
     int rows = (int)std::max<int64_t>(1, std::min<int64_t>(rows_max, (budget - kBandPad * bpe) / (row_bytes + bpe * avg)));
     int edges = 0;

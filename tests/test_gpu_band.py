@@ -26,7 +26,7 @@ def _force(monkeypatch, cols):
 
 
 @pytest.mark.parametrize("M,K,F,deg,cols,window", [
-    (700, 900, 602, 40, 128, None),    # a window of 512 columns (8 slices of 64 floats) + one of 90 (2 slices of 48, 12 of 16 lanes)
+    (700, 900, 602, 40, 128, None),    # a window of 512 columns (8 slices of 64 floats) + one of 90 (2 slices of 48: groups of 12 lanes)
     (700, 900, 602, 40, 128, 0),       # the same in one piece: float2 lanes, 8 slices of 38 vectors, 8 bands
     (500, 1000, 128, 30, 100, None),   # float4, 2 slices x 4 row groups; band width not a power of two
     (300, 800, 256, 25, 256, None),    # 4 slices x 2 row groups
@@ -40,6 +40,8 @@ def _force(monkeypatch, cols):
     (300, 700, 768, 25, 90, None),     # 512 + 256: the second window is 4 slices x 2 row groups
     (260, 600, 1024, 20, 64, None),    # two full windows
     (200, 500, 514, 15, 50, None),     # remainder of two floats
+    (240, 520, 542, 17, 60, None),     # remainder of 30 columns: one slice, groups of 8 lanes
+    (230, 510, 580, 17, 60, None),     # remainder of 68 columns: 2 slices of 36 (groups of 12 lanes)
     (200, 500, 513, 15, 50, None),     # odd width: scalar lanes in both windows
     (200, 500, 1100, 15, 50, None),    # 512 + 512 + 76
     (220, 450, 330, 18, 45, 128),      # windows of 128 columns: 128 + 128 + 74
