@@ -2244,10 +2244,11 @@ static void dispatch_rows(int vec, const RowsArgs &a, hipStream_t st) {
 // Widths the stream quantizer takes by default (measured at 256 M elements per width, all three code widths): rows
 // of whole float4 in 4-byte aligned buffers, except the multiples of 64 floats up to 768, which are whole passes
 // of the sixteen-lane kernel (F = 128 / 256: 6.2 against 5.7-6.1 TB/s).  It gains most where a row leaves lane
-// slots of that kernel idle: F = 20 / 36 / 72 / 100 / 160: 4.3-5.7 -> 5.5-6.2 TB/s.  Rows that are not whole
-// float4 keep the lane-group kernels (F = 602: 5.4-5.7 against 5.0-5.4 TB/s; F = 123: 4.4-4.7 either way).
+// slots of that kernel idle: F = 20 / 36 / 72 / 100 / 160: 4.4-5.7 -> 5.6-6.3 TB/s.  Narrower rows that are not whole
+// float4 keep the lane-group kernels (F = 602: 5.4-5.7 against 5.1-5.5 TB/s; F = 123: 4.4-4.7 either way); beyond
+// 1024 floats the stream kernel takes every row a wavefront can hold (F = 2050: 3.7 -> 4.7 TB/s at int8 and int4).
 static bool stream_wanted(int F, int vec) {
-    return vec == 4 && !(F % 64 == 0 && F <= 768);
+    return (vec == 4 && !(F % 64 == 0 && F <= 768)) || F > 1024;
 }
 
 static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp32_ptr, const void *u8_ptr,

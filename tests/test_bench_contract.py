@@ -27,9 +27,8 @@ def test_measured_traffic_of_every_default_workload_is_tracked():
             ("rmat_2450000n_62000000e_F128_gcn_weighted_sum", "spmm_short_kernel"),
             ("rmat_2450000n_62000000e_F128_gcn_weighted_sum", "spmm_long_final_kernel"),
             ("sbm_233000n_113597648e_F602_sum", "spmm_band_kernel"),
-            ("quant_pack_int2_1000000x256", "quant_pack_rows_kernel"), ("unpack_dequant_int2_1000000x256", "unpack_dequant_rows_kernel"),
-            ("quant_pack_int2_2000000x128", "quant_pack_rows_kernel"), ("quant_pack_int2_4000000x64", "quant_pack_rows_kernel"),
-            ("quant_pack_int2_425000x602", "quant_pack_rows_kernel"), ("unpack_dequant_int2_425000x602", "unpack_dequant_rows_kernel"),
+            *[(f"{k}_int{b}_{shape}", f"{k}_rows_kernel") for k in ("quant_pack", "unpack_dequant") for b in (8, 4, 2)
+              for shape in ("1000000x256", "2000000x128", "4000000x64", "425000x602")],
             ("prepost_8000000n_160000000ue_local_2000000c_80000000e_remote_int2_F128", "spmm_piece_kernel(dq)"),
             ("prepost_8000000n_160000000ue_local_2000000c_80000000e_remote_int2_F128", "spmm_piece_kernel(local)"),
             ("prepost_8000000n_160000000ue_local_2000000c_80000000e_remote_int2_F128", "spmm_short_kernel(local)")]
@@ -37,6 +36,8 @@ def test_measured_traffic_of_every_default_workload_is_tracked():
         t = b.TRAFFIC.get(key)
         assert t is not None, f"no traffic line for {key} under profiles/"
         assert t["bytes"] == t["fetch_bytes"] + t["write_bytes"] > 0 and t["source"].startswith("profiles/")
+        if not key[0].startswith(("quant_pack", "unpack_dequant")):
+            assert t["plan"], f"the traffic line of {key} does not say which plan shape it was measured on"
 
 
 def test_roofline_fraction_is_measured_traffic_over_time_over_peak():
