@@ -44,7 +44,7 @@ int sgnn_version(void);
  * ------------------------------------------------------------------------------------------- */
 
 /* Per-matrix schedule: 32-bit column indices, the row classes and their work lists.
- *   short rows : chunks of consecutive rows (~128 edges), one lane group per chunk;
+ *   short rows : chunks of consecutive rows (about 64 edges), one lane group per chunk;
  *   long rows  : edges regrouped by column class (a hash of col, 8 classes) and cut into pieces, one
  *                lane group per piece, workgroup i serving class i % 8 so that each XCD's L2 caches
  *                its own class of dense rows; partial sums land in a buffer owned by the plan.  The
