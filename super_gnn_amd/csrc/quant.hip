@@ -672,6 +672,11 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
 // may hold zeros of both signs.
 // ------------------------------------------------------------------------------------------------
 constexpr int kStreamRows = 64;   // fp32 rows per wavefront chunk, at most (one lane per row in the set-up)
+// Four bytes of LDS at any byte address: gfx950's LDS serves a misaligned 32-bit access in one instruction.
+__device__ __forceinline__ uint32_t lds_load_u32_unaligned(const uint8_t *p) {
+    typedef uint32_t u32u __attribute__((aligned(1)));
+    return *reinterpret_cast<const u32u *>(p);
+}
 __host__ __device__ constexpr int stream_wave_bytes(int nv) {
     // (min, max) pair per vector -- later the code bytes, which need half of it (+ 16 for the funnel reads) --, row
     // table (float4, neutral entries past the last row), row ids, row flags
@@ -945,15 +950,13 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
             uint32_t word = 0;
 #pragma unroll
             for (int k = 0; k < EPB; ++k) {
-                const int off = (gr * EPB + k) * pitch + jc - 3;
-                const uint32_t c = __builtin_amdgcn_alignbyte(codes32[(off >> 2) + 1], codes32[off >> 2], (uint32_t)(off & 3));
+                const uint32_t c = lds_load_u32_unaligned(codes + (gr * EPB + k) * pitch + jc - 3);
                 word |= (c & keep) << ((EPB - 1 - k) * BITS);
             }
             if (nA != 0) {
 #pragma unroll
                 for (int k = 0; k < EPB; ++k) {
-                    const int off = ((gr - 1) * EPB + k) * pitch + F + jc - 3;
-                    const uint32_t c = __builtin_amdgcn_alignbyte(codes32[(off >> 2) + 1], codes32[off >> 2], (uint32_t)(off & 3));
+                    const uint32_t c = lds_load_u32_unaligned(codes + ((gr - 1) * EPB + k) * pitch + F + jc - 3);
                     word |= (c & ~keep) << ((EPB - 1 - k) * BITS);
                 }
             }
@@ -2058,12 +2061,14 @@ static void launch_quant16(const RowsArgs &a, hipStream_t st) {
 // Lane-slot shape of the stream quantizer for rows of F floats: NV vectors per lane (one of the instantiated
 // values) and gw packed rows per wavefront, chosen to fill the wavefront's NV * 64 vector slots.
 static bool stream_shape(int F, int epb, int *nv_out, int *gw_out) {
-    static const int nvs[] = {4, 8, 10, 12, 16, 20};
+    // Eight vectors per lane first: a wavefront's fixed work (row look-up, per-row reduction, output set-up: ~140 vector
+    // instructions) is then shared by eight vectors at 27 KB of LDS per workgroup.  Four only for rows so narrow that 64
+    // rows do not fill eight; ten and more cost registers and LDS, hence wavefronts per CU, and are taken only for a
+    // clearly better fill or when a packed row needs them (16 vectors per lane: 4.1-4.6 TB/s where 8-10 reach 5.4-6.0).
+    static const int nvs[] = {8, 4, 10, 12, 16, 20};
     const int vpr = (F + 3) / 4;
     double best = 0.0;
     for (int nv : nvs) {
-        // More vectors per lane cost registers and LDS, hence wavefronts per CU: beyond 10 only when a packed row needs it
-        // (measured: 16 vectors per lane run at 4.1-4.6 TB/s where 8-10 reach 5.4-6.0).
         if (best > 0.0 && nv > 10) break;
         const int gw = std::min(nv * 64 / (epb * vpr), kStreamRows / epb);
         if (gw < 1) continue;
@@ -2241,14 +2246,18 @@ static void dispatch_rows(int vec, const RowsArgs &a, hipStream_t st) {
     else dispatch_rows_shape<BITS, 1>(a.F, a, st);
 }
 
-// Widths the stream quantizer takes by default (measured at 256 M elements per width, all three code widths): rows
-// of whole float4 in 4-byte aligned buffers, except the multiples of 64 floats up to 768, which are whole passes
-// of the sixteen-lane kernel (F = 128 / 256: 6.2 against 5.7-6.1 TB/s).  It gains most where a row leaves lane
-// slots of that kernel idle: F = 20 / 36 / 72 / 100 / 160: 4.4-5.7 -> 5.6-6.3 TB/s.  Narrower rows that are not whole
-// float4 keep the lane-group kernels (F = 602: 5.4-5.7 against 5.1-5.5 TB/s; F = 123: 4.4-4.7 either way); beyond
-// 1024 floats the stream kernel takes every row a wavefront can hold (F = 2050: 3.7 -> 4.7 TB/s at int8 and int4).
+// Widths the stream quantizer takes by default (measured at 256 M elements per width, all three code widths):
+//   - rows of whole float4 in aligned buffers, except the multiples of 64 floats up to 768, which are whole passes of
+//     the sixteen-lane kernel (F = 128 / 256: 6.3 against 5.8-6.1 TB/s).  It gains most where a row leaves lane slots of
+//     that kernel idle: F = 20 / 36 / 72 / 100 / 160: 4.4-5.7 -> 5.6-6.3 TB/s;
+//   - rows of up to 256 floats that are not whole float4 or sit in unaligned buffers, where the lane-group kernels'
+//     per-row 16-byte pieces at 4-byte alignments cost most (F = 123: 4.4-4.8 -> 5.2-5.5 TB/s, F = 37: 3.5-3.9 -> 5.1-5.2;
+//     wider ragged rows keep the lane-group kernels: F = 602 5.5-5.8 against 5.3-5.7 TB/s);
+//   - beyond 1024 floats every row a wavefront can hold (F = 2050: 3.7 -> 4.7 TB/s at int8 and int4).
 static bool stream_wanted(int F, int vec) {
-    return (vec == 4 && !(F % 64 == 0 && F <= 768)) || F > 1024;
+    if (F > 1024) return true;
+    if (vec == 4) return !(F % 64 == 0 && F <= 768);
+    return F <= 256;
 }
 
 static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp32_ptr, const void *u8_ptr,
