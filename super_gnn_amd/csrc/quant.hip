@@ -1239,7 +1239,7 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_ragged_kernel(
 template <int BITS, int R, bool SEGMENTED>
 __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_odd_kernel(
     const uint8_t *__restrict__ q, float *__restrict__ x, const ParamBuf pb, const int32_t *__restrict__ seg,
-    const int32_t *__restrict__ pseg, int P, int F, int n_rows, int64_t n_elem) {
+    const int32_t *__restrict__ pseg, int P, int F, int n_rows, int64_t n_elem, int n_packed) {
     constexpr int EPB = 8 / BITS;
     constexpr uint32_t MASK = (1u << BITS) - 1u;
     const int lane = threadIdx.x & 63;
@@ -1262,47 +1262,48 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_odd_kernel(
         }
         return pseg[lo] * EPB + (row - seg[lo]);
     };
-    uint32_t code[R][4];
+    // (row, column) of each vector's first element: one division for the lane's first vector, then 256 elements per round
+    const int dr = 256 / F, dc = 256 % F;
+    int row_a = (int)((base * 4) / F);
+    int c_a = (int)(base * 4 - (int64_t)row_a * F);
+    const int64_t q_bytes = (int64_t)n_packed * F;   // (at least 4: F >= 4 on this path)
+    typedef uint32_t u32u __attribute__((aligned(1)));
+    uint32_t wa[R], wb[R];
+    int sh_a[R], sh_b[R];
     float2 psa[R], psb[R];
     int na[R];
 #pragma unroll
     for (int u = 0; u < R; ++u) {
         const int64_t i = base + u * 64;
-        na[u] = 0;
+        na[u] = 4;
         psa[u] = psb[u] = make_float2(0.0f, 0.0f);
-#pragma unroll
-        for (int k = 0; k < 4; ++k) code[u][k] = 0;
-        if (i >= n_vec) continue;
-        const int64_t e0 = i * 4;
-        const int row_a = (int)(e0 / F);
-        const int c_a = (int)(e0 - (int64_t)row_a * F);
-        na[u] = F - c_a < 4 ? F - c_a : 4;
-        const bool has_b = na[u] < 4 && row_a + 1 < n_rows;
-        const bool wave_whole = __ballot(na[u] != 4) == 0ull;   // every active lane's vector lies inside one row
-        const int slot_a = slot_of(row_a);
-        psa[u] = load_params(pb, row_a);
-        const uint8_t *src_a = q + (int64_t)(slot_a / EPB) * F + c_a;
-        const int shift_a = (EPB - 1 - (slot_a % EPB)) * BITS;
-        const uint8_t *src_b = src_a;
-        int shift_b = 0;
-        if (has_b) {
-            const int slot_b = slot_of(row_a + 1);
-            psb[u] = load_params(pb, row_a + 1);
-            src_b = q + (int64_t)(slot_b / EPB) * F - na[u];   // piece k of row B is its column k - n_a
-            shift_b = (EPB - 1 - (slot_b % EPB)) * BITS;
+        wa[u] = wb[u] = 0;
+        sh_a[u] = sh_b[u] = 0;
+        if (i < n_vec) {
+            na[u] = F - c_a < 4 ? F - c_a : 4;
+            const int slot_a = slot_of(row_a);
+            psa[u] = load_params(pb, row_a);
+            sh_a[u] = (EPB - 1 - (slot_a % EPB)) * BITS;
+            // The vector's four code bytes with one 4-byte load at their natural address (bytes past the end of row A, if
+            // any, are not used).  A load that would reach past the end of the buffer starts d bytes earlier and is
+            // shifted back; no branch around a load, so all of a lane's loads are in flight together.
+            const int64_t off_a = (int64_t)(slot_a / EPB) * F + c_a;
+            const int64_t off_ac = off_a < q_bytes - 4 ? off_a : q_bytes - 4;
+            wa[u] = *reinterpret_cast<const u32u *>(q + off_ac) >> (8 * (int)(off_a - off_ac));
+            if (na[u] < 4 && row_a + 1 < n_rows) {   // the vector's tail lies in the next row: its columns 0 ... 3 - n_a
+                const int slot_b = slot_of(row_a + 1);
+                psb[u] = load_params(pb, row_a + 1);
+                sh_b[u] = (EPB - 1 - (slot_b % EPB)) * BITS;
+                // piece k of row B is its column k - n_a: a load that would start before the buffer starts at its
+                // first byte and is shifted forth
+                const int64_t off_b = (int64_t)(slot_b / EPB) * F - na[u];
+                const int64_t off_bc = off_b > 0 ? off_b : 0;
+                wb[u] = *reinterpret_cast<const u32u *>(q + off_bc) << (8 * (int)(off_bc - off_b));
+            }
         }
-        if (wave_whole) {   // one 4-byte load at the bytes' natural address
-            typedef uint32_t u32u __attribute__((aligned(1)));
-            const uint32_t w = *reinterpret_cast<const u32u *>(src_a);
-#pragma unroll
-            for (int k = 0; k < 4; ++k) code[u][k] = (w >> (8 * k + shift_a)) & MASK;
-            continue;
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const bool in_a = k < na[u];
-            if (in_a || has_b) code[u][k] = ((in_a ? src_a : src_b)[k] >> (in_a ? shift_a : shift_b)) & MASK;
-        }
+        row_a += dr;
+        c_a += dc;
+        if (c_a >= F) { c_a -= F; ++row_a; }
     }
 #pragma unroll
     for (int u = 0; u < R; ++u) {
@@ -1311,8 +1312,10 @@ __global__ __launch_bounds__(kQBlock) void unpack_dequant_flat_odd_kernel(
         float o[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const float2 ps = k < na[u] ? psa[u] : psb[u];
-            o[k] = fmaf((float)code[u][k], ps.y, ps.x);
+            const bool in_a = k < na[u];
+            const uint32_t c = ((in_a ? wa[u] : wb[u]) >> (8 * k + (in_a ? sh_a[u] : sh_b[u]))) & MASK;
+            const float2 ps = in_a ? psa[u] : psb[u];
+            o[k] = fmaf((float)c, ps.y, ps.x);
         }
         if (i * 4 + 4 <= n_elem) {
             vec_store_nt<4>(x + i * 4, o);
@@ -2162,10 +2165,10 @@ static void launch_dequant_flat_ragged_r(const RowsArgs &a, int64_t n_rows, hipS
     if (VEC == 1 && a.F >= 4 && two_rows) {
         if (BITS != 8 && a.P > 1)
             hipLaunchKernelGGL((unpack_dequant_flat_odd_kernel<BITS, R, true>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, a.x_out,
-                               a.params, a.seg, a.pseg, a.P, a.F, (int)n_rows, n_elem);
+                               a.params, a.seg, a.pseg, a.P, a.F, (int)n_rows, n_elem, a.n_packed);
         else
             hipLaunchKernelGGL((unpack_dequant_flat_odd_kernel<BITS, R, false>), dim3(nb), dim3(kQBlock), 0, st, a.q_in, a.x_out,
-                               a.params, a.seg, a.pseg, a.P, a.F, (int)n_rows, n_elem);
+                               a.params, a.seg, a.pseg, a.P, a.F, (int)n_rows, n_elem, a.n_packed);
         return;
     }
     if (BITS != 8 && a.P > 1)
