@@ -9,7 +9,7 @@ GCN-normalised edge weights) over an R-MAT power-law graph with 2.45 M nodes / ~
 at F = 128 fp32.  Unless --no-extras is given the same run also measures the dense-degree
 community graph at F = 602 (``sbm``), the pre/post-aggregation partition with int2-packed remote
 rows (``prepost``), the small CPU-runnable case (``small``), the int8/int4/int2 quantize+pack and
-unpack+dequantize kernels on 1 M x 256, 2 M x 128, 4 M x 64 and 425 k x 602 boundary rows
+unpack+dequantize kernels on 1 M x 256, 2 M x 128, 4 M x 64, 425 k x 602 and 2.56 M x 100 boundary rows
 (``quant*``), a streaming copy (the attainable-bandwidth yardstick) and the CPU baselines timed on
 this machine's host cores.  Any of them can be made the headline of the line with --workload.
 
@@ -924,6 +924,8 @@ def main():
                 others["quant_F64"] = wl_quant(args, ctx, rows=4 * args.quant_rows, feat=64, headline=False)
                 torch.cuda.empty_cache()  # rows that do not start on cache lines: the dense-degree graph's feature width
                 others["quant_F602"] = wl_quant(args, ctx, rows=425_000 * args.quant_rows // 1_000_000, feat=602, headline=False)
+                torch.cuda.empty_cache()  # rows that are not whole lane-group passes (the stream quantizer): ogbn-products' width
+                others["quant_F100"] = wl_quant(args, ctx, rows=2_560_000 * args.quant_rows // 1_000_000, feat=100, headline=False)
             log(f"[bench] extra workload {name}: {time.perf_counter() - t0:.1f}s")
         args.steps, args.warmup = saved
         if "copy" in others:

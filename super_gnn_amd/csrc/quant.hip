@@ -231,13 +231,28 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_kernel(
             if constexpr (RAGGED) {
                 if (off[v] + VEC <= F) {
                     vec4_load_nt_unaligned(xv[r][v], xr + off[v]);
-                } else {  // missing elements: copies of the first one (they change neither min nor max nor the first zero)
-                    xv[r][v][0] = xr[off[v]];
+                } else {  // the row's short last vector: its elements one by one (padded below, once every load is out)
 #pragma unroll
-                    for (int k = 1; k < VEC; ++k) xv[r][v][k] = off[v] + k < F ? xr[off[v] + k] : xv[r][v][0];
+                    for (int k = 0; k < VEC; ++k)
+                        if (off[v] + k < F) xv[r][v][k] = xr[off[v] + k];
                 }
             } else {
                 vec_load_nt<VEC>(xv[r][v], xr + off[v]);
+            }
+        }
+    }
+    if constexpr (RAGGED) {
+        // missing elements: copies of the vector's first one (they change neither min nor max nor the first zero).  Done
+        // after the loads: a use of a loaded value between two loads would make every load wait for the one before.
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                if (valid[r] && act[v] && off[v] + VEC > F) {
+#pragma unroll
+                    for (int k = 1; k < VEC; ++k)
+                        if (off[v] + k >= F) xv[r][v][k] = xv[r][v][0];
+                }
             }
         }
     }
@@ -455,13 +470,28 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
             if constexpr (RAGGED) {
                 if (off[v] + VEC <= F) {
                     vec4_load_nt_unaligned(xv[rl][v], xr + off[v]);
-                } else {
-                    xv[rl][v][0] = xr[off[v]];
+                } else {  // the row's short last vector: its elements one by one (padded below, once every load is out)
 #pragma unroll
-                    for (int k = 1; k < VEC; ++k) xv[rl][v][k] = off[v] + k < F ? xr[off[v] + k] : xv[rl][v][0];
+                    for (int k = 0; k < VEC; ++k)
+                        if (off[v] + k < F) xv[rl][v][k] = xr[off[v] + k];
                 }
             } else {
                 vec_load_nt<VEC>(xv[rl][v], xr + off[v]);
+            }
+        }
+    }
+    if constexpr (RAGGED) {
+        // missing elements: copies of the vector's first one.  Done after the loads: a use of a loaded value between two
+        // loads would make every load wait for the one before.
+#pragma unroll
+        for (int rl = 0; rl < RL; ++rl) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                if (valid[rl] && act[v] && off[v] + VEC > F) {
+#pragma unroll
+                    for (int k = 1; k < VEC; ++k)
+                        if (off[v] + k >= F) xv[rl][v][k] = xv[rl][v][0];
+                }
             }
         }
     }

@@ -28,7 +28,7 @@ def test_measured_traffic_of_every_default_workload_is_tracked():
             ("rmat_2450000n_62000000e_F128_gcn_weighted_sum", "spmm_long_final_kernel"),
             ("sbm_233000n_113597648e_F602_sum", "spmm_band_kernel"),
             *[(f"{k}_int{b}_{shape}", f"{k}_rows_kernel") for k in ("quant_pack", "unpack_dequant") for b in (8, 4, 2)
-              for shape in ("1000000x256", "2000000x128", "4000000x64", "425000x602")],
+              for shape in ("1000000x256", "2000000x128", "4000000x64", "425000x602", "2560000x100")],
             ("prepost_8000000n_160000000ue_local_2000000c_80000000e_remote_int2_F128", "spmm_piece_kernel(dq)"),
             ("prepost_8000000n_160000000ue_local_2000000c_80000000e_remote_int2_F128", "spmm_piece_kernel(local)"),
             ("prepost_8000000n_160000000ue_local_2000000c_80000000e_remote_int2_F128", "spmm_short_kernel(local)")]
@@ -68,7 +68,7 @@ def _canned_results(b):
                       "kernel_rooflines": {"x": {"y": {"z": 1}}}, "edge_values_bound_to_plan": True}}
     others = {}
     for name, (n, F) in {"quant": (1_000_000, 256), "quant_F128": (2_000_000, 128), "quant_F64": (4_000_000, 64),
-                         "quant_F602": (425_000, 602)}.items():
+                         "quant_F602": (425_000, 602), "quant_F100": (2_560_000, 100)}.items():
         extra = {}
         for bits in (8, 4, 2):
             w = f"quant_pack_int{bits}_{n}x{F}"
