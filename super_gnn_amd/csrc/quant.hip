@@ -778,7 +778,9 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
             // holds (all but the last one or two of the chunk) are loaded without a lane predicate.
             const float *xb = x + (int64_t)r_first * F;
             const int n_sv = n_valid * VPR;
-            const uint32_t eo_max = (uint32_t)((n_rows - r_first) * F - 4);   // (a chunk is far smaller than 2^31 elements)
+            // (a chunk is far smaller than 2^31 elements; the rest of the tensor need not be)
+            const int64_t e_rest = (int64_t)(n_rows - r_first) * F - 4;
+            const uint32_t eo_max = e_rest < 0x7fffffff ? (uint32_t)e_rest : 0x7fffffffu;
             const int cv_short = (F & 3) != 0 ? VPR - 1 : -1;   // the vector of a row that holds fewer than four elements
 #pragma unroll
             for (int v = 0; v < NV; ++v) {

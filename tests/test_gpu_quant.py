@@ -253,11 +253,12 @@ def test_facades_and_errors():
                         torch.zeros(0, 2, device="cuda"), 2)
 
 
-@pytest.mark.parametrize("n,F", [(1_000_000, 256), (2_000_000, 128), (4_000_000, 64)])
+@pytest.mark.parametrize("n,F", [(1_000_000, 256), (2_000_000, 128), (4_000_000, 64), (2_560_000, 100), (425_000, 602)])
 @pytest.mark.parametrize("bits", [8, 4, 2])
 def test_full_size_properties(bits, n, F):
     # the sweep's full shape (1M x 256, 10% outlier rows) and the same bytes as rows of 128 and 64 floats (the
-    # widths the layers exchange; they take the eight-lanes-per-row kernel): size-independent properties plus an
+    # widths the layers exchange; they take the eight-lanes-per-row kernel), ogbn-products' 100 floats (the quantizer
+    # that walks runs of rows) and reddit's 602 (rows on 8-byte boundaries): size-independent properties plus an
     # exact comparison of every row with the oracle
     from super_gnn_amd import synth
     ops = _ops()
@@ -556,11 +557,14 @@ def test_buffers_at_odd_addresses(bits, F):
         assert (o[:xoff] == 7.0).all() and (o[xoff + n * F:] == 7.0).all(), "floats outside the rows were written"
 
 
-def test_offsets_beyond_four_gigabytes():
-    # 9 M x 128 fp32 = 4.6 GB: byte offsets of the last rows do not fit 32 bits.  Params against torch's
+@pytest.mark.parametrize("n,F", [(9_000_000, 128), (11_000_000, 100), (9_000_000, 123)])
+def test_offsets_beyond_four_gigabytes(n, F):
+    # 9 M x 128 fp32 = 4.6 GB: byte offsets of the last rows do not fit 32 bits, and neither does the number of
+    # ELEMENTS behind the first rows at F = 100 / 123 (the widths that take the quantizer which walks runs of rows,
+    # the second one with rows that are not whole float4).  Params against torch's
     # min/max, the round-trip bound everywhere, and the last rows of every segment bit-exact against the oracle.
     ops = _ops()
-    n, F, bits, P = 9_000_000, 128, 2, 3
+    bits, P = 2, 3
     epb = 8 // bits
     g = torch.Generator(device="cuda"); g.manual_seed(41)
     x = torch.randn(n, F, generator=g, device="cuda")
