@@ -692,15 +692,32 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
 //   D  the lanes walk the output run (gw * F consecutive bytes) in aligned 4-byte words, 256 bytes per store
 //      instruction: a word is the OR of the EPB rows' code words, fetched from the code array at their byte
 //      offsets and shifted to their bit positions.
-// The last vector of a row with F % 4 != 0 is loaded element by element and padded with copies of its first
-// element (copies change neither min nor max nor the first-zero rule); vector slots without a row (past the end
-// of the chunk, or the row slots a segment's short last group leaves empty) hold zeros, which quantize to code 0
-// under the empty slot's neutral params.
+// The last vector of a row with F % 4 != 0 is loaded whole (it reaches into the next row) and, once every load is
+// out, cut back to its F % 4 elements and padded with copies of its first element (copies change neither min nor
+// max nor the first-zero rule).  Vector slots behind the chunk's last row (the rest of the lane's last vector or
+// two, or the row slots a segment's short last group leaves empty) repeat the chunk's last vector, so that no load
+// needs a predicate; phase B never reads their pairs and phase C clears their code words.
+// The kernel is sized so that it waits on memory and not on instruction issue (~66 vector instructions per float4
+// at int2): no lane predicates or row bookkeeping around the loads (the row slot of a vector is one 24-bit
+// multiply), the rule for a NaN as a row's first element looked at only when some vector starts with a NaN, one
+// guard-band test per lane instead of one per element.
 // Signed zeros: v_min_f32 / v_max_f32 order -0 < +0, so a zero minimum is -0 exactly when the row holds a -0
 // and a zero maximum is +0 exactly when it holds a +0; the sign of the row's FIRST zero (what the reference's
 // strict compares keep, quantization_arm.cpp:98-101) needs a second pass over the elements only when a row
 // may hold zeros of both signs.
 // ------------------------------------------------------------------------------------------------
+// v_min_f32 / v_max_f32 as they are: fminf / fmaxf quiet their operands first (one more instruction each), which
+// results of earlier min / max operations do not need.  A NaN operand loses against a number, as in fminf / fmaxf.
+__device__ __forceinline__ float min_bare(float a, float b) {
+    float r;
+    asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ __forceinline__ float max_bare(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
 constexpr int kStreamRows = 64;   // fp32 rows per wavefront chunk, at most (one lane per row in the set-up)
 // Four bytes of LDS at any byte address: gfx950's LDS serves a misaligned 32-bit access in one instruction.
 __device__ __forceinline__ uint32_t lds_load_u32_unaligned(const uint8_t *p) {
@@ -717,7 +734,8 @@ __host__ __device__ constexpr int stream_wave_bytes(int nv) {
 template <int BITS, int NV, bool RAGGED, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
     const float *__restrict__ x, uint8_t *__restrict__ q, const ParamBuf pb, const int32_t *__restrict__ seg,
-    const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F, int gw, int n_units, int n_rows) {
+    const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F, int gw, int n_units, int n_rows,
+    uint32_t vpr_magic) {
     constexpr int EPB = 8 / BITS;
     constexpr int kWaveBytes = stream_wave_bytes(NV);
     static_assert(kWaveBytes % 16 == 0, "wave pieces of LDS must keep 16-byte alignment");
@@ -762,97 +780,98 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 
     // ---- loads ------------------------------------------------------------------------------------------------
-    // (row slot, vector inside the row) of each of the lane's vectors: advanced by 64 vectors per step
-    const int dpr = 64 / VPR, dcv = 64 % VPR;
+    // Vector slot v * 64 + lane of the chunk is vector (slot % VPR) of row slot (slot / VPR); the quotient comes from
+    // one 24-bit multiply (vpr_magic = ceil(2^21 / VPR), exact for slot * VPR < 2^21).
     int prv[NV];
     float xv[NV][4];
-    uint32_t first_mask = 0;   // bit v: vector v starts its row
-    uint32_t short_mask = 0;   // bit v: vector v is the short last vector of its row (F % 4 elements)
-    (void)short_mask;
-    {
-        int pr = lane / VPR, cv = lane - pr * VPR;
-        if (run) {
-            // The common case: one base address, 32-bit element offsets, every vector a 16-byte load -- a row's short
-            // last vector too, which then reaches into the next row and is cut back after all loads are out; only the
-            // one that would reach past the end of the tensor is moved back to end with it.  Vectors that every lane
-            // holds (all but the last one or two of the chunk) are loaded without a lane predicate.
-            const float *xb = x + (int64_t)r_first * F;
-            const int n_sv = n_valid * VPR;
-            // (a chunk is far smaller than 2^31 elements; the rest of the tensor need not be)
-            const int64_t e_rest = (int64_t)(n_rows - r_first) * F - 4;
-            const uint32_t eo_max = e_rest < 0x7fffffff ? (uint32_t)e_rest : 0x7fffffffu;
-            const int cv_short = (F & 3) != 0 ? VPR - 1 : -1;   // the vector of a row that holds fewer than four elements
+    // run: slots up to `last` hold vectors; the slots behind them (the rest of the last one or two of the lane's
+    // vectors) repeat the last vector, so that their loads need no predicate, and their code words are cleared in C.
+    const int n_sv = run ? n_valid * VPR : 0;
+    const int last = run ? n_sv - 1 : INT_MAX;
+    const int n_full = run ? n_sv >> 6 : NV;   // the lane's vectors below this index are real in every lane (wave-uniform)
+    if (run) {
+        // The common case: one base address, 32-bit element offsets, every vector a 16-byte load -- a row's short last
+        // vector too, which then reaches into the next row and is cut back after all loads are out; only the one that
+        // would reach past the end of the tensor is moved back to end with it.
+        const float *xb = x + (int64_t)r_first * F;
+        // (a chunk is far smaller than 2^31 elements; the rest of the tensor need not be)
+        const int64_t e_rest = (int64_t)(n_rows - r_first) * F - 4;
+        const uint32_t eo_max = e_rest < 0x7fffffff ? (uint32_t)e_rest : 0x7fffffffu;
+        const int pad = 4 * VPR - F;   // elements a row's last vector lacks
 #pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                prv[v] = pr < kStreamRows ? pr : kStreamRows;   // (slots past the chunk: the neutral table entry)
-                uint32_t eo = RAGGED ? (uint32_t)(pr * F + 4 * cv) : (uint32_t)(4 * (v * 64 + lane));
-                if constexpr (RAGGED) eo = eo < eo_max ? eo : eo_max;
-                if ((v + 1) * 64 <= n_sv) {   // wave-uniform
-                    vec4_load_nt_unaligned(xv[v], xb + eo);
-                    if (cv == 0) first_mask |= 1u << v;
-                    if (RAGGED && cv == cv_short) short_mask |= 1u << v;
-                } else {
-                    xv[v][0] = 0.0f; xv[v][1] = 0.0f; xv[v][2] = 0.0f; xv[v][3] = 0.0f;
-                    if (v * 64 + lane < n_sv) {
-                        vec4_load_nt_unaligned(xv[v], xb + eo);
-                        if (cv == 0) first_mask |= 1u << v;
-                        if (RAGGED && cv == cv_short) short_mask |= 1u << v;
-                    }
-                }
-                pr += dpr;
-                cv += dcv;
-                if (cv >= VPR) { cv -= VPR; ++pr; }
+        for (int v = 0; v < NV; ++v) {
+            const int sl = v * 64 + lane < last ? v * 64 + lane : last;
+            const int pr = (int)(__umul24((uint32_t)sl, vpr_magic) >> 21);
+            prv[v] = pr;
+            uint32_t eo = 4u * (uint32_t)sl;
+            if constexpr (RAGGED) {
+                eo -= (uint32_t)(pr * pad);
+                eo = eo < eo_max ? eo : eo_max;
             }
-            if constexpr (RAGGED) {   // cut the short vectors back to their F % 4 elements, padded with copies of the first
-                const int nt = F & 3;
-                if (__ballot(short_mask != 0) != 0) {
+            // (a 32-bit byte offset from the chunk's first row: base register + lane offset addressing)
+            vec4_load_nt_unaligned(xv[v], reinterpret_cast<const float *>(reinterpret_cast<const char *>(xb) + 4u * eo));
+        }
+        if constexpr (RAGGED) {
+            const int nt = F & 3;
+            if (nt != 0) {   // cut the short vectors back to their F % 4 elements, padded with copies of the first
+                if (r_first + n_valid == n_rows) {   // the tensor's last vector was loaded `pad` elements early
 #pragma unroll
                     for (int v = 0; v < NV; ++v) {
-                        if ((short_mask >> v) & 1u) {
-                            const uint32_t eo = (uint32_t)(prv[v] * F + 4 * (VPR - 1));
-                            if (eo > eo_max) {   // the tensor's last vector was loaded eo - eo_max elements early
-                                const int d = (int)(eo - eo_max);
-                                const float a1 = xv[v][1], a2 = xv[v][2], a3 = xv[v][3];
-                                xv[v][0] = d == 1 ? a1 : d == 2 ? a2 : a3;
-                                xv[v][1] = d == 1 ? a2 : a3;
-                                xv[v][2] = a3;
-                            }
-#pragma unroll
-                            for (int t = 1; t < 4; ++t)
-                                if (t >= nt) xv[v][t] = xv[v][0];
+                        const int sl = v * 64 + lane < last ? v * 64 + lane : last;
+                        if (sl == last) {
+                            const float a1 = xv[v][1], a2 = xv[v][2], a3 = xv[v][3];
+                            xv[v][0] = pad == 1 ? a1 : pad == 2 ? a2 : a3;
+                            xv[v][1] = pad == 1 ? a2 : a3;
+                            xv[v][2] = a3;
                         }
                     }
                 }
-            }
-        } else {
-            // a chunk that spans the end of a segment: row by row through the chunk's row table
 #pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                prv[v] = pr < kStreamRows ? pr : kStreamRows;
-                const int r = pr < npr ? rowid[pr] : -1;
-                xv[v][0] = 0.0f; xv[v][1] = 0.0f; xv[v][2] = 0.0f; xv[v][3] = 0.0f;
-                if (r >= 0) {
-                    const float *xp = x + (int64_t)r * F + 4 * cv;
-                    const float first = __builtin_nontemporal_load(xp);
+                for (int v = 0; v < NV; ++v) {
+                    const int sl = v * 64 + lane < last ? v * 64 + lane : last;
+                    const bool sh = sl - prv[v] * VPR == VPR - 1;
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) xv[v][t] = (t == 0 || 4 * cv + t < F) ? __builtin_nontemporal_load(xp + t) : first;
-                    if (cv == 0) first_mask |= 1u << v;
+                    for (int t = 1; t < 4; ++t) xv[v][t] = (sh && t >= nt) ? xv[v][0] : xv[v][t];
                 }
-                pr += dpr;
-                cv += dcv;
-                if (cv >= VPR) { cv -= VPR; ++pr; }
             }
+        }
+    } else {
+        // a chunk that spans the end of a segment: row by row through the chunk's row table
+        const int dpr = 64 / VPR, dcv = 64 % VPR;
+        int pr = lane / VPR, cv = lane - pr * VPR;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            prv[v] = pr < kStreamRows ? pr : kStreamRows;   // (slots past the chunk: the neutral table entry)
+            const int r = pr < npr ? rowid[pr] : -1;
+            xv[v][0] = 0.0f; xv[v][1] = 0.0f; xv[v][2] = 0.0f; xv[v][3] = 0.0f;
+            if (r >= 0) {
+                const float *xp = x + (int64_t)r * F + 4 * cv;
+                const float first = __builtin_nontemporal_load(xp);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) xv[v][t] = (t == 0 || 4 * cv + t < F) ? __builtin_nontemporal_load(xp + t) : first;
+            }
+            pr += dpr;
+            cv += dcv;
+            if (cv >= VPR) { cv -= VPR; ++pr; }
         }
     }
 
     // ---- A: (min, max) of every vector -----------------------------------------------------------------------
+    bool nan0 = false;   // a NaN is sticky only as element 0 of its row: look closer when some vector starts with one
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         const float m = fminf(fminf(xv[v][0], xv[v][1]), fminf(xv[v][2], xv[v][3]));
         const float M = fmaxf(fmaxf(xv[v][0], xv[v][1]), fmaxf(xv[v][2], xv[v][3]));
         ent[v * 64 + lane] = make_float2(m, M);
-        // a NaN is sticky only as element 0 of its row
-        if (((first_mask >> v) & 1u) && xv[v][0] != xv[v][0]) rowflag[prv[v]] = 1;
+        nan0 |= xv[v][0] != xv[v][0];
+    }
+    if (__ballot(nan0) != 0) {   // wave-uniform, rare
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int sl = v * 64 + lane;
+            const int pr = run ? (int)(__umul24((uint32_t)(sl < last ? sl : last), vpr_magic) >> 21) : sl / VPR;
+            if (sl <= last && pr < npr && sl - pr * VPR == 0 && xv[v][0] != xv[v][0]) rowflag[pr] = 1;
+        }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -865,14 +884,15 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
     const bool has_row = row_b < npr;
     const int e_lo = has_row ? row_b * VPR : 0, e_hi = has_row ? e_lo + VPR : 0;   // the row's vectors
     float mn = INFINITY, mx = -INFINITY;
+    // (the pairs are results of min / max already: the bare instructions, without a quieting pass over their operands)
     for (int e = e_lo + li; e < e_hi; e += LR) {
         const float2 p = ent[e];
-        mn = fminf(mn, p.x);
-        mx = fmaxf(mx, p.y);
+        mn = min_bare(mn, p.x);
+        mx = max_bare(mx, p.y);
     }
     for (int o = 1; o < LR; o <<= 1) {
-        mn = fminf(mn, __shfl_xor(mn, o, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        mn = min_bare(mn, __shfl_xor(mn, o, 64));
+        mx = max_bare(mx, __shfl_xor(mx, o, 64));
     }
     const bool row_valid = has_row && rowid[has_row ? row_b : 0] >= 0;
     // the sign of the row's first zero, where both signs may occur (see the header)
@@ -922,6 +942,10 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
     const int mis = RAGGED ? (int)(reinterpret_cast<uintptr_t>(out_run) & 3) : 0;
     bool lane_exact = false;
     uint32_t words[NV];
+    // The largest distance of a quotient from its rounded value over all of the lane's elements decides once for the
+    // lane.  A NaN quotient (a NaN element behind the first of its row) drops out of the maximum: its code is 0 from
+    // the conversion here as from the saturating conversion of quant_code.
+    float far = 0.0f;
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         const float4 ta = rowtab[prv[v]];
@@ -931,11 +955,12 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
         for (int t = 0; t < 4; ++t) {
             const float qf = (xv[v][t] - ta.x) * ta.z;
             const float ri = rintf(qf);
-            if (!(fabsf(qf - ri) < 0.5f - kGuard)) lane_exact = true;   // also true for a NaN quotient
+            far = fmaxf(far, fabsf(qf - ri));
             word = __builtin_amdgcn_cvt_pk_u8_f32(ri, t, word);
         }
         words[v] = word;
     }
+    if (!(far < 0.5f - kGuard)) lane_exact = true;
     if (lane_exact) {   // this lane redoes its elements with the IEEE division
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
@@ -946,6 +971,9 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
             words[v] = word;
         }
     }
+#pragma unroll
+    for (int v = 0; v < NV; ++v)   // slots behind the chunk's last vector hold copies of it: their codes are zero
+        if (v >= n_full && v * 64 + lane > last) words[v] = 0;
     if (EPB == 1 && !RAGGED) {   // code words are output words
         uint32_t *q32 = reinterpret_cast<uint32_t *>(out_run);
 #pragma unroll
@@ -2095,15 +2123,19 @@ static void launch_quant16(const RowsArgs &a, hipStream_t st) {
 
 // Lane-slot shape of the stream quantizer for rows of F floats: NV vectors per lane (one of the instantiated
 // values) and gw packed rows per wavefront, chosen to fill the wavefront's NV * 64 vector slots.
-static bool stream_shape(int F, int epb, int *nv_out, int *gw_out) {
-    // Eight vectors per lane first: a wavefront's fixed work (row look-up, per-row reduction, output set-up: ~140 vector
-    // instructions) is then shared by eight vectors at 27 KB of LDS per workgroup.  Four only for rows so narrow that 64
-    // rows do not fill eight; ten and more cost registers and LDS, hence wavefronts per CU, and are taken only for a
-    // clearly better fill or when a packed row needs them (16 vectors per lane: 4.1-4.6 TB/s where 8-10 reach 5.4-6.0).
-    static const int nvs[] = {8, 4, 10, 12, 16, 20};
+static bool stream_shape(int F, int epb, bool ragged, int *nv_out, int *gw_out) {
+    // Rows of whole float4: four vectors per lane first.  The kernel then waits on memory, not on instruction issue,
+    // and what counts is how many wavefronts a CU holds (15 KB of LDS per workgroup, ~45 registers: F = 128 / 256
+    // 5.8-6.1 -> 6.1-6.5 TB/s against eight); eight where four would leave more than 2.5 % more slots empty.  The
+    // ragged path does more per wavefront (short vectors, output words that straddle rows) and shares it among eight
+    // vectors first (F = 123 / 250: 5.3 / 5.4 -> 5.6 / 5.9 TB/s against four).  Ten and more cost registers and LDS
+    // and are taken only for a clearly better fill or when a packed row needs them.
+    static const int nvs_aligned[] = {4, 8, 10, 12, 16, 20}, nvs_ragged[] = {8, 4, 10, 12, 16, 20};
+    const int *nvs = ragged ? nvs_ragged : nvs_aligned;
     const int vpr = (F + 3) / 4;
     double best = 0.0;
-    for (int nv : nvs) {
+    for (int k = 0; k < 6; ++k) {
+        const int nv = nvs[k];
         if (best > 0.0 && nv > 10) break;
         const int gw = std::min(nv * 64 / (epb * vpr), kStreamRows / epb);
         if (gw < 1) continue;
@@ -2122,16 +2154,19 @@ static void launch_quant_stream_nv(const RowsArgs &a, int gw, hipStream_t st) {
     constexpr int WAVES = stream_wave_bytes(NV) * 4 <= 64 * 1024 ? 4 : 2;
     const int n_units = (a.n_packed + gw - 1) / gw;
     const int nb = (n_units + WAVES - 1) / WAVES;
+    const uint32_t vpr = (uint32_t)(a.F + 3) / 4;   // (at most NV * 64 <= 1280: the kernel divides slots by it with one multiply)
     ProfScope prof(K_QUANT_PACK_ROWS, st);
     hipLaunchKernelGGL((quant_pack_stream_kernel<BITS, NV, RAGGED, WAVES>), dim3(nb), dim3(64 * WAVES), 0, st, a.x_in.x, a.q_out,
-                       a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, gw, n_units, (int)a.x_in.n_src);
+                       a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, gw, n_units, (int)a.x_in.n_src,
+                       (uint32_t)(((1u << 21) + vpr - 1) / vpr));
 }
 
 template <int BITS>
 static bool launch_quant_stream(const RowsArgs &a, hipStream_t st) {
     int nv = 0, gw = 0;
-    if (a.x_in.index != nullptr || a.x_in.ld != a.F || a.F < 16 || !stream_shape(a.F, 8 / BITS, &nv, &gw)) return false;
+    if (a.x_in.index != nullptr || a.x_in.ld != a.F || a.F < 16) return false;
     const bool ragged = a.F % 4 != 0 || !aligned(a.q_out, 4);
+    if (!stream_shape(a.F, 8 / BITS, ragged, &nv, &gw)) return false;
 #define SGNN_STREAM(NV_)                                                       \
     case NV_:                                                                  \
         if (ragged) launch_quant_stream_nv<BITS, NV_, true>(a, gw, st);        \
@@ -2283,16 +2318,17 @@ static void dispatch_rows(int vec, const RowsArgs &a, hipStream_t st) {
 
 // Widths the stream quantizer takes by default (measured at 256 M elements per width, all three code widths):
 //   - rows of whole float4 in aligned buffers, except the multiples of 64 floats up to 768, which are whole passes of
-//     the sixteen-lane kernel (F = 128 / 256: 6.3 against 5.8-6.1 TB/s).  It gains most where a row leaves lane slots of
-//     that kernel idle: F = 20 / 36 / 72 / 100 / 160: 4.4-5.7 -> 5.6-6.3 TB/s;
+//     the sixteen-lane kernel (F = 128 / 256: level with it at int4 / int2, 3-6 % behind at int8).  It gains most where
+//     a row leaves lane slots of that kernel idle: F = 20 / 36 / 72 / 100 / 160: 4.4-5.7 -> 5.9-6.3 TB/s;
 //   - rows of up to 256 floats that are not whole float4 or sit in unaligned buffers, where the lane-group kernels'
-//     per-row 16-byte pieces at 4-byte alignments cost most (F = 123: 4.4-4.8 -> 5.2-5.5 TB/s, F = 37: 3.5-3.9 -> 5.1-5.2;
-//     wider ragged rows keep the lane-group kernels: F = 602 5.5-5.8 against 5.3-5.7 TB/s);
+//     per-row 16-byte pieces at 4-byte alignments cost most (F = 123: 4.4-4.8 -> 5.5-5.6 TB/s, F = 37: 3.4-3.9 -> 5.4-5.5);
+//     wider ones at int4 / int2 while a packed row fits twelve vectors per lane (F = 602: 5.7 / 5.5 -> 5.9 / 5.9 TB/s; at
+//     int8 the lane-group kernels are level or ahead: F = 301 5.9 against 5.5);
 //   - beyond 1024 floats every row a wavefront can hold (F = 2050: 3.7 -> 4.7 TB/s at int8 and int4).
-static bool stream_wanted(int F, int vec) {
+static bool stream_wanted(int F, int vec, int bits) {
     if (F > 1024) return true;
     if (vec == 4) return !(F % 64 == 0 && F <= 768);
-    return F <= 256;
+    return F <= 256 || (bits < 8 && (F + 3) / 4 * (8 / bits) <= 12 * 64);
 }
 
 static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp32_ptr, const void *u8_ptr,
@@ -2317,7 +2353,7 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
     SGNN_REQUIRE(aligned(a.params.p, a.params.bf16 ? 4 : 8), "params must be %d-byte aligned", a.params.bf16 ? 4 : 8);
     const int stream = env_flag("SGNN_QUANT_STREAM", -1);   // 1: every width the stream quantizer can take, 0: never
     bool taken = false;
-    if (a.quantize && !a.exact_division && (stream > 0 || (stream < 0 && stream_wanted(a.F, vec))))
+    if (a.quantize && !a.exact_division && (stream > 0 || (stream < 0 && stream_wanted(a.F, vec, bits))))
         taken = bits == 8 ? launch_quant_stream<8>(a, st) : bits == 4 ? launch_quant_stream<4>(a, st) : launch_quant_stream<2>(a, st);
     if (taken) {
     } else if (!a.quantize && vec == 4 && a.flat) {
