@@ -17,7 +17,7 @@ Output.  stdout carries ONE JSON line of at most LINE_LIMIT bytes: the headline 
 fields with a flat ``roofline`` and ``cpu_baseline``, and in ``extra`` one flat record per other
 workload (``extra["workloads"]``) plus the int2 quantize+pack rate and roofline fraction as scalars.
 Everything nested (per-kernel times, plans, step rooflines, every roofline object in full) goes to
-stderr as one ``[bench-detail]`` JSON line and to gpurun_out/bench_detail.json.
+stderr as one ``[bench-detail]`` JSON line and to the file bench_detail.json in the folder DETAIL_DIR.
 
 Roofline objects.  SpMM kernels: ``achieved`` is HBM-side bytes per step of the dominant kernel
 (rocprofv3 FETCH_SIZE + WRITE_SIZE, read from the ``traffic:`` lines of the summaries under
@@ -778,7 +778,40 @@ def wl_sage(args, ctx):
             "ms_per_step": ms, "dtype": "f32", "roofline": None, "cpu_baseline": None, "extra": {}}
 
 
-WORKLOADS = {"rmat": wl_rmat, "quant": wl_quant, "quant_widths": wl_quant_widths, "copy": wl_copy, "prepost": wl_prepost, "sbm": wl_sbm,
+def wl_gather_sets(args, ctx):
+    """What the memory system delivers to the row-stream SpMM kernel against the size of the set of dense rows it gathers
+    from: every one of --nodes rows has 12 edges to uniform columns among the first W rows of X (F = --feat), W from
+    --set-rows.  A set inside one L2, inside the Infinity Cache and far beyond it give the three ceilings the
+    headline's kernels are read against."""
+    import torch
+    from super_gnn_amd import supergnn_ops as ops
+    dev = ctx["dev"]
+    N, D, F = args.nodes, 12, args.feat
+    x = torch.randn(N, F, device=dev)
+    out = torch.zeros(N, F, device=dev)
+    rowptr = torch.arange(N + 1, device=dev, dtype=torch.int64) * D
+    rows = []
+    for W in [min(int(w), N) for w in args.set_rows.split(",")]:
+        g = torch.Generator(device=dev); g.manual_seed(W)
+        col = torch.randint(0, W, (N, D), generator=g, device=dev, dtype=torch.int64).sort(dim=1).values.reshape(-1).to(torch.int32)
+        plan = ops.SpmmPlan(rowptr, col, N)
+        ms, per_k, _ = profiled_steps(lambda: plan.run(None, x, out, accumulate=True), max(args.steps, 10), max(args.warmup, 3))
+        k_ms = sum(per_k.values())
+        nnz = N * D
+        gathers, rest = nnz * F * 4, 2 * N * F * 4 + nnz * 4 + N * 8   # dense rows gathered; out read and written, columns, rowptr
+        rows.append({"set_rows": W, "set_MiB": round(W * F * 4 / 2 ** 20, 1), "kernel_ms": round(k_ms, 4),
+                     "GEdges_per_s": round(nnz / k_ms / 1e6, 2), "gather_GBps": round(gathers / k_ms / 1e6),
+                     "other_GBps": round(rest / k_ms / 1e6), "total_GBps": round((gathers + rest) / k_ms / 1e6)})
+        log(f"[bench] gather set {W:8d} rows = {rows[-1]['set_MiB']:7.1f} MiB: {k_ms:.3f} ms, {rows[-1]['GEdges_per_s']:.2f} GEdges/s, "
+            f"gathers {rows[-1]['gather_GBps']} GB/s + out / edge streams {rows[-1]['other_GBps']} GB/s = {rows[-1]['total_GBps']} GB/s")
+        del plan
+    last = rows[-1]
+    return {"metric": "row-stream SpMM bytes/s against the size of the gathered set", "value": last["total_GBps"], "unit": "GB/s",
+            "config": {"workload": f"gather_sets_{N}n_{N * D}e_F{F}"}, "ms_per_step": last["kernel_ms"], "dtype": "f32",
+            "roofline": None, "cpu_baseline": None, "extra": {"sets": rows}}
+
+
+WORKLOADS = {"gather_sets": wl_gather_sets, "rmat": wl_rmat, "quant": wl_quant, "quant_widths": wl_quant_widths, "copy": wl_copy, "prepost": wl_prepost, "sbm": wl_sbm,
              "aggregate": wl_aggregate, "sage": wl_sage, "small": wl_small}
 
 
@@ -808,13 +841,14 @@ def quant_records(name, r):
     return out
 
 
+DETAIL_DIR = "gpurun_out"   # where the full record of a run is kept (relative to this file)
 LINE_LIMIT = 4000   # bytes; the harness that reads the line keeps only a bounded tail of stdout
 
 
 def build_line(result, others, steps, warmup):
     """The ONE JSON line of stdout, from the headline workload's result and the other workloads' results
     (name -> result dict).  Everything nested (per-kernel tables, plans, per-width rooflines) stays out of it:
-    main() writes that to stderr and to gpurun_out/bench_detail.json."""
+    main() writes that to stderr and to bench_detail.json in DETAIL_DIR."""
     rf = dict(result["roofline"] or {})
     for k in ("traffic_source", "algorithmic_bytes", "launches", "gather_GBps", "traffic_frac"):
         rf.pop(k, None)
@@ -862,7 +896,7 @@ def main():
     ap.add_argument("--workload", default="rmat", choices=sorted(WORKLOADS),
                     help="rmat: headline SpMM (default); quant: int2 quantize+pack as the step; copy: streaming copy; "
                          "prepost: one partition with packed remote rows, fused vs separate; sbm: dense-degree graph, F=602; "
-                         "small: the CPU-runnable case; aggregate / sage: the aggregation layer and a GraphSAGE epoch")
+                         "small: the CPU-runnable case; aggregate / sage: the aggregation layer and a GraphSAGE epoch; gather_sets: the row-stream kernel against the size of the gathered set")
     ap.add_argument("--local-nodes", type=int, default=8_000_000)
     ap.add_argument("--remote-nodes", type=int, default=2_000_000)
     ap.add_argument("--local-und-edges", type=int, default=160_000_000)
@@ -886,6 +920,8 @@ def main():
     ap.add_argument("--bits", type=int, default=2)
     ap.add_argument("--widths", default="32,64,100,123,128,200,256,300,500,600,602,640,1000,1024,1200,2050",
                     help="quant_widths: row widths of the sweep")
+    ap.add_argument("--set-rows", default="4096,16384,65536,131072,262144,524288,1048576,2450000",
+                    help="gather_sets: sizes (rows of X) of the sets the columns are drawn from")
     ap.add_argument("--segments", type=int, default=1, help="quant_widths: cut the rows into this many per-peer segments")
     ap.add_argument("--long-threshold", type=int, default=0, help="SpMM plan: rows longer than this are split (0 = default)")
     ap.add_argument("--piece-edges", type=int, default=0, help="SpMM plan: minimum edges per long-row piece (0 = default)")
@@ -935,8 +971,8 @@ def main():
     text = json.dumps(detail)
     log("[bench-detail] " + text)
     try:   # the same detail as a file, where the run has a results folder
-        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-        with open(os.path.join(ROOT, "gpurun_out", "bench_detail.json"), "w") as f:
+        os.makedirs(os.path.join(ROOT, DETAIL_DIR), exist_ok=True)
+        with open(os.path.join(ROOT, DETAIL_DIR, "bench_detail.json"), "w") as f:
             f.write(text + "\n")
     except OSError:
         pass
