@@ -361,12 +361,15 @@ def wl_copy(args, ctx):
             "cpu_baseline": None, "extra": {}}
 
 
-def quant_case(ops, x, bits, steps, warmup, segments=1):
+def quant_case(ops, x, bits, steps, warmup, segments=1, row_index=None):
     """Quantize+pack and unpack+dequantize of x at one width: times, rates, rooflines.  segments > 1: the rows
-    are cut at seeded random points into that many per-peer segments, each padded to whole packed rows."""
+    are cut at seeded random points into that many per-peer segments, each padded to whole packed rows.
+    row_index: the quantizer reads rows x[row_index] (the gather into the send buffer folded into it)."""
     import numpy as np
     import torch
     n, F = x.shape
+    if row_index is not None:
+        n = row_index.numel()
     epb = 8 // bits
     cuts = np.sort(np.random.default_rng(segments).integers(0, n, size=segments - 1)).tolist() if segments > 1 else []
     seg = torch.tensor([0] + cuts + [n], dtype=torch.int32)
@@ -376,7 +379,7 @@ def quant_case(ops, x, bits, steps, warmup, segments=1):
     d = torch.empty(n, F, device=x.device)
     wl = f"quant_pack_int{bits}_{n}x{F}"
     b = quant_bytes(n, F, bits)
-    ms_q, kq, _ = profiled_steps(lambda: ops.quantize_tensor_for_all_procs(x, q, p, seg, segments, bits), steps, warmup)
+    ms_q, kq, _ = profiled_steps(lambda: ops.quantize_tensor_for_all_procs(x, q, p, seg, segments, bits, row_index=row_index), steps, warmup)
     ms_d, kd, _ = profiled_steps(lambda: ops.dequantize_tensor_for_all_procs(q, d, p, seg, segments, bits), steps, warmup)
     kq_ms, kd_ms = kq["quant_pack_rows_kernel"], kd["unpack_dequant_rows_kernel"]
     return {"workload": wl, "bytes": b, "quant_ms": ms_q, "dequant_ms": ms_d,
@@ -624,10 +627,16 @@ def wl_quant_widths(args, ctx):
     table = {}
     for F in widths:
         n = 256_000_000 // F
-        x = synth.boundary_features(n, F, seed=5, device=ctx["dev"])
+        idx = None
+        if args.row_index != "none":   # two of three rows of a tensor half as large again, in ascending or random order
+            g = torch.Generator(device=ctx["dev"]); g.manual_seed(F)
+            idx = torch.randperm(n + n // 2, generator=g, device=ctx["dev"])[:n]
+            if args.row_index == "sorted":
+                idx = idx.sort().values
+        x = synth.boundary_features(n if idx is None else n + n // 2, F, seed=5, device=ctx["dev"])
         row = {}
         for bits in (8, 4, 2):
-            c = quant_case(ops, x, bits, max(args.steps, 5), max(args.warmup, 2), segments=args.segments)
+            c = quant_case(ops, x, bits, max(args.steps, 5), max(args.warmup, 2), segments=args.segments, row_index=idx)
             row[f"int{bits}"] = {"quant_us": round(c["quant_roofline"]["kernel_ms"] * 1e3, 1),
                                  "quant_GBps": c["quant_roofline"]["gather_GBps"],
                                  "dequant_us": round(c["dequant_roofline"]["kernel_ms"] * 1e3, 1),
@@ -922,6 +931,8 @@ def main():
                     help="quant_widths: row widths of the sweep")
     ap.add_argument("--set-rows", default="4096,16384,65536,131072,262144,524288,1048576,2450000",
                     help="gather_sets: sizes (rows of X) of the sets the columns are drawn from")
+    ap.add_argument("--row-index", default="none", choices=("none", "sorted", "random"),
+                    help="quant_widths: quantize rows picked by a row index (two of three rows of a larger tensor)")
     ap.add_argument("--segments", type=int, default=1, help="quant_widths: cut the rows into this many per-peer segments")
     ap.add_argument("--long-threshold", type=int, default=0, help="SpMM plan: rows longer than this are split (0 = default)")
     ap.add_argument("--piece-edges", type=int, default=0, help="SpMM plan: minimum edges per long-row piece (0 = default)")

@@ -675,7 +675,8 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
-// Fused quantize + pack over a run of consecutive rows: any row width from 16 floats, rows contiguous in memory.
+// Fused quantize + pack over a run of consecutive row slots: any row width from 16 floats; the rows themselves are
+// consecutive in memory (the fast case) or found through a table (a row index, a pitch, a chunk across two segments).
 //
 // A wavefront takes `gw` consecutive packed rows, i.e. gw * EPB fp32 rows (at most 64), which lie one after the
 // other in memory.  Each row is cut into VPR = ceil(F / 4) float4 vectors and the chunk's rows * VPR vectors are
@@ -726,18 +727,20 @@ __device__ __forceinline__ uint32_t lds_load_u32_unaligned(const uint8_t *p) {
 }
 __host__ __device__ constexpr int stream_wave_bytes(int nv) {
     // (min, max) pair per vector -- later the code bytes, which need half of it (+ 16 for the funnel reads) --, row
-    // table (float4, neutral entries past the last row), row ids, row flags
-    return nv * 512 + 16 + (kStreamRows + 4) * 16 + kStreamRows * (4 + 4);
+    // table (float4; empty row slots keep a neutral entry), row ids, row flags, source rows
+    return nv * 512 + 16 + kStreamRows * 16 + kStreamRows * (4 + 4 + 4);
 }
 
 // RAGGED: F % 4 != 0, or an output buffer that is not 4-byte aligned.
 template <int BITS, int NV, bool RAGGED, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
-    const float *__restrict__ x, uint8_t *__restrict__ q, const ParamBuf pb, const int32_t *__restrict__ seg,
-    const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F, int gw, int n_units, int n_rows,
+    const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb, const int32_t *__restrict__ seg,
+    const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F, int gw, int n_units,
     uint32_t vpr_magic) {
     constexpr int EPB = 8 / BITS;
     constexpr int kWaveBytes = stream_wave_bytes(NV);
+    const float *__restrict__ x = xs.x;
+    const int n_rows = (int)xs.n_src;   // rows of the source tensor (the launcher keeps them below 2^31)
     static_assert(kWaveBytes % 16 == 0, "wave pieces of LDS must keep 16-byte alignment");
     static_assert(WAVES * kWaveBytes <= 64 * 1024, "static LDS of a workgroup");
     __shared__ __align__(16) uint8_t lds_all[WAVES * kWaveBytes];
@@ -747,8 +750,9 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
     uint8_t *base = lds_all + wv * kWaveBytes;
     float2 *ent = reinterpret_cast<float2 *>(base);
     float4 *rowtab = reinterpret_cast<float4 *>(base + NV * 512 + 16);   // (zero_point, scale, 1 / scale, needs the exact division)
-    int *rowid = reinterpret_cast<int *>(rowtab + kStreamRows + 4);
+    int *rowid = reinterpret_cast<int *>(rowtab + kStreamRows);   // the row whose params a row slot writes, -1: empty slot
     int *rowflag = rowid + kStreamRows;
+    int *rowsrc = rowflag + kStreamRows;                                // the row of x it reads (the same without a row index)
     uint8_t *codes = base;   // the pairs are dead by the time the codes are written
 
     const int g0 = __builtin_amdgcn_readfirstlane(unit) * gw;
@@ -757,7 +761,7 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
     const int VPR = (F + 3) >> 2;      // vectors per row; npr * VPR <= NV * 64
 
     // ---- the chunk's rows: lane i looks up row slot i --------------------------------------------------------
-    int my_row = -1;
+    int my_row = -1, my_src = -1;
     {
         WaveSegment ws{0, 0, 0, 0, 0};
         if (single_rows < 0) ws = wave_find_segment(pseg, seg, P, g0);
@@ -767,16 +771,22 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
             const int64_t r = row0 + lane % EPB;
             if (r < rend) my_row = (int)r;
         }
+        my_src = my_row;
+        if (xs.index != nullptr && my_row >= 0) {
+            const int64_t r = xs.index[my_row];
+            my_src = (uint64_t)r < (uint64_t)xs.n_src ? (int)r : 0;   // (as row_ptr() treats an index out of range)
+        }
         rowid[lane] = my_row;
+        rowsrc[lane] = my_src;
         rowflag[lane] = 0;
         rowtab[lane] = make_float4(0.0f, 1.0f, 1.0f, 0.0f);
-        if (lane < 4) rowtab[kStreamRows + lane] = make_float4(0.0f, 1.0f, 1.0f, 0.0f);
     }
     const unsigned long long vb = __ballot(my_row >= 0);
     const int n_valid = __popcll(vb);
     const int r_first = __builtin_amdgcn_readfirstlane(my_row);
     // rows consecutive in memory, empty slots only at the end: row slot p holds row r_first + p for p < n_valid
-    const bool run = (vb & (vb + 1)) == 0 && (vb & 1) && __ballot(my_row >= 0 && my_row != r_first + lane) == 0;
+    const bool run = xs.index == nullptr && xs.ld == F && (vb & (vb + 1)) == 0 && (vb & 1) &&
+                     __ballot(my_row >= 0 && my_row != r_first + lane) == 0;
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 
     // ---- loads ------------------------------------------------------------------------------------------------
@@ -789,6 +799,7 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
     const int n_sv = run ? n_valid * VPR : 0;
     const int last = run ? n_sv - 1 : INT_MAX;
     const int n_full = run ? n_sv >> 6 : NV;   // the lane's vectors below this index are real in every lane (wave-uniform)
+    uint32_t dead_mask = 0;                    // table path: bit v = the lane's vector v belongs to no row
     if (run) {
         // The common case: one base address, 32-bit element offsets, every vector a 16-byte load -- a row's short last
         // vector too, which then reaches into the next row and is cut back after all loads are out; only the one that
@@ -836,23 +847,45 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
             }
         }
     } else {
-        // a chunk that spans the end of a segment: row by row through the chunk's row table
-        const int dpr = 64 / VPR, dcv = 64 % VPR;
-        int pr = lane / VPR, cv = lane - pr * VPR;
+        // Rows anywhere -- a row index, rows with a pitch, a chunk that spans the end of a segment: every vector finds
+        // its row in the chunk's table.  Slots of empty row slots and behind the chunk read the chunk's first row
+        // (their codes are cleared in C), so that here too no load needs a predicate.
+        const int src_any = __builtin_amdgcn_readlane(my_src, __builtin_ctzll(vb));   // some row of the chunk (vb != 0)
+        const int n_sl = npr * VPR;
+        const int pad = 4 * VPR - F;
+        int64_t eo[NV];
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
-            prv[v] = pr < kStreamRows ? pr : kStreamRows;   // (slots past the chunk: the neutral table entry)
-            const int r = pr < npr ? rowid[pr] : -1;
-            xv[v][0] = 0.0f; xv[v][1] = 0.0f; xv[v][2] = 0.0f; xv[v][3] = 0.0f;
-            if (r >= 0) {
-                const float *xp = x + (int64_t)r * F + 4 * cv;
-                const float first = __builtin_nontemporal_load(xp);
+            const int sl = v * 64 + lane < n_sl ? v * 64 + lane : n_sl - 1;
+            const int pr = (int)(__umul24((uint32_t)sl, vpr_magic) >> 21);
+            const int cv = sl - pr * VPR;
+            prv[v] = pr;
+            int src = rowsrc[pr];
+            if (src < 0 || v * 64 + lane >= n_sl) dead_mask |= 1u << v;
+            if (src < 0) src = src_any;
+            eo[v] = (int64_t)src * xs.ld + 4 * cv;
+            // the short last vector of the tensor's last row is loaded `pad` elements early (cut back below)
+            if (RAGGED && pad != 0 && cv == VPR - 1 && src == n_rows - 1) eo[v] -= pad;
+        }
 #pragma unroll
-                for (int t = 0; t < 4; ++t) xv[v][t] = (t == 0 || 4 * cv + t < F) ? __builtin_nontemporal_load(xp + t) : first;
+        for (int v = 0; v < NV; ++v) vec4_load_nt_unaligned(xv[v], x + eo[v]);
+        if constexpr (RAGGED) {
+            const int nt = F & 3;
+            if (nt != 0) {
+#pragma unroll
+                for (int v = 0; v < NV; ++v) {
+                    const int sl = v * 64 + lane < n_sl ? v * 64 + lane : n_sl - 1;
+                    const bool sh = sl - prv[v] * VPR == VPR - 1;
+                    if (sh && rowsrc[prv[v]] == n_rows - 1) {
+                        const float a1 = xv[v][1], a2 = xv[v][2], a3 = xv[v][3];
+                        xv[v][0] = pad == 1 ? a1 : pad == 2 ? a2 : a3;
+                        xv[v][1] = pad == 1 ? a2 : a3;
+                        xv[v][2] = a3;
+                    }
+#pragma unroll
+                    for (int t = 1; t < 4; ++t) xv[v][t] = (sh && t >= nt) ? xv[v][0] : xv[v][t];
+                }
             }
-            pr += dpr;
-            cv += dcv;
-            if (cv >= VPR) { cv -= VPR; ++pr; }
         }
     }
 
@@ -869,8 +902,7 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int sl = v * 64 + lane;
-            const int pr = run ? (int)(__umul24((uint32_t)(sl < last ? sl : last), vpr_magic) >> 21) : sl / VPR;
-            if (sl <= last && pr < npr && sl - pr * VPR == 0 && xv[v][0] != xv[v][0]) rowflag[pr] = 1;
+            if (sl <= last && !((dead_mask >> v) & 1u) && sl - prv[v] * VPR == 0 && xv[v][0] != xv[v][0]) rowflag[prv[v]] = 1;
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
@@ -973,7 +1005,7 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
     }
 #pragma unroll
     for (int v = 0; v < NV; ++v)   // slots behind the chunk's last vector hold copies of it: their codes are zero
-        if (v >= n_full && v * 64 + lane > last) words[v] = 0;
+        if ((v >= n_full && v * 64 + lane > last) || ((dead_mask >> v) & 1u)) words[v] = 0;
     if (EPB == 1 && !RAGGED) {   // code words are output words
         uint32_t *q32 = reinterpret_cast<uint32_t *>(out_run);
 #pragma unroll
@@ -2156,15 +2188,15 @@ static void launch_quant_stream_nv(const RowsArgs &a, int gw, hipStream_t st) {
     const int nb = (n_units + WAVES - 1) / WAVES;
     const uint32_t vpr = (uint32_t)(a.F + 3) / 4;   // (at most NV * 64 <= 1280: the kernel divides slots by it with one multiply)
     ProfScope prof(K_QUANT_PACK_ROWS, st);
-    hipLaunchKernelGGL((quant_pack_stream_kernel<BITS, NV, RAGGED, WAVES>), dim3(nb), dim3(64 * WAVES), 0, st, a.x_in.x, a.q_out,
-                       a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, gw, n_units, (int)a.x_in.n_src,
+    hipLaunchKernelGGL((quant_pack_stream_kernel<BITS, NV, RAGGED, WAVES>), dim3(nb), dim3(64 * WAVES), 0, st, a.x_in, a.q_out,
+                       a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F, gw, n_units,
                        (uint32_t)(((1u << 21) + vpr - 1) / vpr));
 }
 
 template <int BITS>
 static bool launch_quant_stream(const RowsArgs &a, hipStream_t st) {
     int nv = 0, gw = 0;
-    if (a.x_in.index != nullptr || a.x_in.ld != a.F || a.F < 16) return false;
+    if (a.x_in.ld < a.F || a.x_in.n_src >= ((int64_t)1 << 31) || a.F < 16) return false;
     const bool ragged = a.F % 4 != 0 || !aligned(a.q_out, 4);
     if (!stream_shape(a.F, 8 / BITS, ragged, &nv, &gw)) return false;
 #define SGNN_STREAM(NV_)                                                       \
@@ -2325,8 +2357,11 @@ static void dispatch_rows(int vec, const RowsArgs &a, hipStream_t st) {
 //     wider ones at int4 / int2 while a packed row fits twelve vectors per lane (F = 602: 5.7 / 5.5 -> 5.9 / 5.9 TB/s; at
 //     int8 the lane-group kernels are level or ahead: F = 301 5.9 against 5.5);
 //   - beyond 1024 floats every row a wavefront can hold (F = 2050: 3.7 -> 4.7 TB/s at int8 and int4).
-static bool stream_wanted(int F, int vec, int bits) {
+//   - rows picked by a row index, or with a pitch: the same up to 256 floats (F = 100 through a sorted index: 4.3-4.6 ->
+//     4.9-5.5 TB/s); wider ones keep the lane-group kernels (F = 602 through an index: 5.0-5.6 against 4.9-5.0).
+static bool stream_wanted(int F, int vec, int bits, bool rows_by_table) {
     if (F > 1024) return true;
+    if (rows_by_table && F > 256) return false;
     if (vec == 4) return !(F % 64 == 0 && F <= 768);
     return F <= 256 || (bits < 8 && (F + 3) / 4 * (8 / bits) <= 12 * 64);
 }
@@ -2353,7 +2388,7 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
     SGNN_REQUIRE(aligned(a.params.p, a.params.bf16 ? 4 : 8), "params must be %d-byte aligned", a.params.bf16 ? 4 : 8);
     const int stream = env_flag("SGNN_QUANT_STREAM", -1);   // 1: every width the stream quantizer can take, 0: never
     bool taken = false;
-    if (a.quantize && !a.exact_division && (stream > 0 || (stream < 0 && stream_wanted(a.F, vec, bits))))
+    if (a.quantize && !a.exact_division && (stream > 0 || (stream < 0 && stream_wanted(a.F, vec, bits, a.x_in.index != nullptr || a.x_in.ld != a.F))))
         taken = bits == 8 ? launch_quant_stream<8>(a, st) : bits == 4 ? launch_quant_stream<4>(a, st) : launch_quant_stream<2>(a, st);
     if (taken) {
     } else if (!a.quantize && vec == 4 && a.flat) {

@@ -640,3 +640,24 @@ def test_stream_and_lane_group_quantizers_write_the_oracles_bytes(stream, bits, 
         assert np.array_equal(np.isnan(params), nan_ref), seg
         assert np.array_equal(params[~nan_ref].view(np.uint32), p_ref[~nan_ref].view(np.uint32)), seg
         assert np.array_equal(q, q_ref), seg
+    # the same rows picked out of a wider tensor by a row index (repeats, the tensor's last row at several places,
+    # rows that start on odd 4-byte boundaries): the oracle on the gathered copy
+    from super_gnn_amd import supergnn_ops as ops
+    wide = np.zeros((n, F + 3), np.float32)
+    wide[:, 1:1 + F] = x
+    idx = rng.integers(0, n, size=613)
+    idx[[0, 100, 611, 612]] = n - 1
+    seg = [0, 5, 5, 300, 613]
+    q_ref, p_ref = orc.quant_rows(np.ascontiguousarray(x[idx]), seg, bits)
+    epb = 8 // bits
+    npk = sum(-(-(b - a) // epb) for a, b in zip(seg[:-1], seg[1:]))
+    view = torch.from_numpy(wide).cuda()[:, 1:1 + F]
+    q = torch.zeros(npk, F, dtype=torch.uint8, device="cuda")
+    params = torch.zeros(len(idx), 2, device="cuda")
+    ops.quantize_tensor_for_all_procs(view, q, params, torch.tensor(seg, dtype=torch.int32), len(seg) - 1, bits,
+                                      row_index=torch.from_numpy(idx).cuda())
+    params = params.cpu().numpy()
+    nan_ref = np.isnan(p_ref)
+    assert np.array_equal(np.isnan(params), nan_ref)
+    assert np.array_equal(params[~nan_ref].view(np.uint32), p_ref[~nan_ref].view(np.uint32))
+    assert np.array_equal(q.cpu().numpy(), q_ref)
