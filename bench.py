@@ -396,7 +396,9 @@ def wl_quant(args, ctx, rows=None, feat=None, headline=True):
     for bits in (8, 4, 2):
         if headline and args.no_extras and bits != args.bits:
             continue
-        c = quant_case(ops, xq, bits, args.steps if (headline and bits == args.bits) else 10, args.warmup if headline else 3)
+        # (the secondary shapes get as long a warm-up as the headline one: the first few dozen launches after the
+        # allocations before them run at lower clocks, which kernels close to their instruction-issue limit show)
+        c = quant_case(ops, xq, bits, args.steps if (headline and bits == args.bits) else 20, max(args.warmup, 10))
         cases[bits] = c
         log(f"[bench] {n}x{F} int{bits}: quantize+pack kernel {c['quant_roofline']['gather_GBps']:.0f} GB/s "
             f"({c['quant_roofline']['kernel_ms'] * 1e3:.1f} us), unpack+dequant kernel "

@@ -725,6 +725,10 @@ __device__ __forceinline__ uint32_t lds_load_u32_unaligned(const uint8_t *p) {
     typedef uint32_t u32u __attribute__((aligned(1)));
     return *reinterpret_cast<const u32u *>(p);
 }
+__device__ __forceinline__ void lds_store_u32_unaligned(uint8_t *p, uint32_t v) {
+    typedef uint32_t u32u __attribute__((aligned(1)));
+    *reinterpret_cast<u32u *>(p) = v;
+}
 __host__ __device__ constexpr int stream_wave_bytes(int nv) {
     // (min, max) pair per vector -- later the code bytes, which need half of it (+ 16 for the funnel reads) --, row
     // table (float4; empty row slots keep a neutral entry), row ids, row flags, source rows
@@ -1019,56 +1023,96 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
     __builtin_amdgcn_wave_barrier();
 
     // ---- D: pack and store ------------------------------------------------------------------------------------
-    // code byte of (row slot p, column j): codes[p * pitch + j]
-    const int pitch = 4 * VPR;
+    // code word w of row slot p: codes32[p * VPR + w]
     const int nbytes = ng * F;
     const int nw = (mis + nbytes + 3) >> 2;
     const uint32_t *codes32 = reinterpret_cast<const uint32_t *>(codes);
     uint32_t *q32 = reinterpret_cast<uint32_t *>(out_run - mis);
-    // (packed row, column) of the LAST byte of a lane's word (never negative): advanced by 256 bytes per round
-    const int dgr = 256 / F, djc = 256 % F;
-    int b0 = 4 * lane - mis;
-    int gr = (b0 + 3) / F, jc = b0 + 3 - gr * F;
-    for (int w = lane; w < nw; w += 64) {
-        if (!RAGGED) {
+    const int n_pw = ng * VPR;   // words of the packed rows, a row's last one short when F % 4 != 0
+    if constexpr (!RAGGED) {
+        // F % 4 == 0: packed word s of the chunk is output word s
+        for (int s = lane; s < n_pw; s += 64) {
+            const int g = (int)(__umul24((uint32_t)s, vpr_magic) >> 21);
+            const uint32_t *cw = codes32 + s * EPB - (s - g * VPR) * (EPB - 1);   // (g * EPB) * VPR + word in the row
             uint32_t word = 0;
 #pragma unroll
-            for (int k = 0; k < EPB; ++k) word |= codes32[((gr * EPB + k) * pitch + jc - 3) >> 2] << ((EPB - 1 - k) * BITS);
-            __builtin_nontemporal_store(word, q32 + w);
-        } else if (b0 >= 0 && b0 + 3 < nbytes) {
-            // jc >= 3: four bytes of packed row gr; else the first 3 - jc bytes are the end of packed row gr - 1
-            const int nA = jc >= 3 ? 0 : 3 - jc;
-            const uint32_t keep = 0xffffffffu << (8 * nA);
-            uint32_t word = 0;
-#pragma unroll
-            for (int k = 0; k < EPB; ++k) {
-                const uint32_t c = lds_load_u32_unaligned(codes + (gr * EPB + k) * pitch + jc - 3);
-                word |= (c & keep) << ((EPB - 1 - k) * BITS);
-            }
-            if (nA != 0) {
+            for (int k = 0; k < EPB; ++k) word |= cw[k * VPR] << ((EPB - 1 - k) * BITS);
+            __builtin_nontemporal_store(word, q32 + s);
+        }
+    } else if constexpr (EPB < 4) {
+        // The lanes walk the output run in aligned words; a word's bytes are gathered from the code words of its
+        // packed row -- or, where it straddles two, of both -- at their byte offsets.  (For int8 and int4 this is
+        // cheaper than the extra pass through LDS below: F = 123 int8 5.5 against 4.7 TB/s.)
+        const int pitch = 4 * VPR;
+        // (packed row, column) of the LAST byte of a lane's word (never negative): advanced by 256 bytes per round
+        const int dgr = 256 / F, djc = 256 % F;
+        int b0 = 4 * lane - mis;
+        int gr = (b0 + 3) / F, jc = b0 + 3 - gr * F;
+        for (int w = lane; w < nw; w += 64) {
+            if (b0 >= 0 && b0 + 3 < nbytes) {
+                // jc >= 3: four bytes of packed row gr; else the first 3 - jc bytes are the end of packed row gr - 1
+                const int nA = jc >= 3 ? 0 : 3 - jc;
+                const uint32_t keep = 0xffffffffu << (8 * nA);
+                uint32_t word = 0;
 #pragma unroll
                 for (int k = 0; k < EPB; ++k) {
-                    const uint32_t c = lds_load_u32_unaligned(codes + ((gr - 1) * EPB + k) * pitch + F + jc - 3);
-                    word |= (c & ~keep) << ((EPB - 1 - k) * BITS);
+                    const uint32_t c = lds_load_u32_unaligned(codes + (gr * EPB + k) * pitch + jc - 3);
+                    word |= (c & keep) << ((EPB - 1 - k) * BITS);
+                }
+                if (nA != 0) {
+#pragma unroll
+                    for (int k = 0; k < EPB; ++k) {
+                        const uint32_t c = lds_load_u32_unaligned(codes + ((gr - 1) * EPB + k) * pitch + F + jc - 3);
+                        word |= (c & ~keep) << ((EPB - 1 - k) * BITS);
+                    }
+                }
+                __builtin_nontemporal_store(word, q32 + w);
+            } else {   // the first or the last word of the run, partly outside it
+                for (int t = 0; t < 4; ++t) {
+                    const int b = b0 + t;
+                    if (b < 0 || b >= nbytes) continue;
+                    const int c = jc - 3 + t;
+                    const int g = c < 0 ? gr - 1 : gr, j = c < 0 ? c + F : c;
+                    uint32_t byte = 0;
+#pragma unroll
+                    for (int k = 0; k < EPB; ++k) byte |= (uint32_t)codes[(g * EPB + k) * pitch + j] << ((EPB - 1 - k) * BITS);
+                    out_run[b] = (uint8_t)byte;
                 }
             }
-            __builtin_nontemporal_store(word, q32 + w);
-        } else {   // the first or the last word of the run, partly outside it
-            for (int t = 0; t < 4; ++t) {
-                const int b = b0 + t;
-                if (b < 0 || b >= nbytes) continue;
-                const int c = jc - 3 + t;
-                const int g = c < 0 ? gr - 1 : gr, j = c < 0 ? c + F : c;
-                uint32_t byte = 0;
+            b0 += 256;
+            gr += dgr;
+            jc += djc;
+            if (jc >= F) { jc -= F; ++gr; }
+        }
+    } else {
+        // int2: the packed rows are first laid out byte after byte in LDS (behind the code words): a row's last word is
+        // written before the other words of the round, so that the bytes it spills into the next row are overwritten
+        // by that row's first word (same round, or a later one).  The run then goes out in aligned words.
+        uint8_t *packed = base + NV * 256;
+        for (int s0 = 0; s0 < n_pw; s0 += 64) {
+            const int s = s0 + lane < n_pw ? s0 + lane : n_pw - 1;
+            const int g = (int)(__umul24((uint32_t)s, vpr_magic) >> 21), wv = s - g * VPR;
+            const uint32_t *cw = codes32 + s * EPB - wv * (EPB - 1);
+            uint32_t word = 0;
 #pragma unroll
-                for (int k = 0; k < EPB; ++k) byte |= (uint32_t)codes[(g * EPB + k) * pitch + j] << ((EPB - 1 - k) * BITS);
-                out_run[b] = (uint8_t)byte;
+            for (int k = 0; k < EPB; ++k) word |= cw[k * VPR] << ((EPB - 1 - k) * BITS);
+            uint8_t *dst = packed + g * F + 4 * wv;
+            const bool live = s0 + lane < n_pw, tail = wv == VPR - 1;
+            if (live && tail) lds_store_u32_unaligned(dst, word);
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // (keeps the two stores apart and in this order)
+            if (live && !tail) lds_store_u32_unaligned(dst, word);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (int w = lane; w < nw; w += 64) {
+            const int b0 = 4 * w - mis;
+            if (b0 >= 0 && b0 + 3 < nbytes) {
+                __builtin_nontemporal_store(lds_load_u32_unaligned(packed + b0), q32 + w);
+            } else {   // the first or the last word of the run, partly outside it
+                for (int t = 0; t < 4; ++t)
+                    if (b0 + t >= 0 && b0 + t < nbytes) out_run[b0 + t] = packed[b0 + t];
             }
         }
-        b0 += 256;
-        gr += dgr;
-        jc += djc;
-        if (jc >= F) { jc -= F; ++gr; }
     }
 }
 
