@@ -857,7 +857,6 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
         const int src_any = __builtin_amdgcn_readlane(my_src, __builtin_ctzll(vb));   // some row of the chunk (vb != 0)
         const int n_sl = npr * VPR;
         const int pad = 4 * VPR - F;
-        int64_t eo[NV];
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int sl = v * 64 + lane < n_sl ? v * 64 + lane : n_sl - 1;
@@ -867,12 +866,11 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
             int src = rowsrc[pr];
             if (src < 0 || v * 64 + lane >= n_sl) dead_mask |= 1u << v;
             if (src < 0) src = src_any;
-            eo[v] = (int64_t)src * xs.ld + 4 * cv;
+            int64_t eo = (int64_t)src * xs.ld + 4 * cv;
             // the short last vector of the tensor's last row is loaded `pad` elements early (cut back below)
-            if (RAGGED && pad != 0 && cv == VPR - 1 && src == n_rows - 1) eo[v] -= pad;
+            if (RAGGED && pad != 0 && cv == VPR - 1 && src == n_rows - 1) eo -= pad;
+            vec4_load_nt_unaligned(xv[v], x + eo);
         }
-#pragma unroll
-        for (int v = 0; v < NV; ++v) vec4_load_nt_unaligned(xv[v], x + eo[v]);
         if constexpr (RAGGED) {
             const int nt = F & 3;
             if (nt != 0) {
@@ -2394,7 +2392,8 @@ static void dispatch_rows(int vec, const RowsArgs &a, hipStream_t st) {
 
 // Widths the stream quantizer takes by default (measured at 256 M elements per width, all three code widths):
 //   - rows of whole float4 in aligned buffers, except the multiples of 64 floats up to 768, which are whole passes of
-//     the sixteen-lane kernel (F = 128 / 256: level with it at int4 / int2, 3-6 % behind at int8).  It gains most where
+//     the sixteen-lane kernel (128 ... 768: level with it at int4 / int2 within +-4 %, 3-6 % behind at int8; F = 64 at
+//     int4 / int2 is the exception and takes the stream kernel: 6.16 / 5.95 -> 6.27 / 6.34 TB/s).  It gains most where
 //     a row leaves lane slots of that kernel idle: F = 20 / 36 / 72 / 100 / 160: 4.4-5.7 -> 5.9-6.3 TB/s;
 //   - rows of up to 256 floats that are not whole float4 or sit in unaligned buffers, where the lane-group kernels'
 //     per-row 16-byte pieces at 4-byte alignments cost most (F = 123: 4.4-4.8 -> 5.5-5.6 TB/s, F = 37: 3.4-3.9 -> 5.4-5.5);
@@ -2406,7 +2405,7 @@ static void dispatch_rows(int vec, const RowsArgs &a, hipStream_t st) {
 static bool stream_wanted(int F, int vec, int bits, bool rows_by_table) {
     if (F > 1024) return true;
     if (rows_by_table && F > 256) return false;
-    if (vec == 4) return !(F % 64 == 0 && F <= 768);
+    if (vec == 4) return !(F % 64 == 0 && F <= 768) || (F == 64 && bits < 8);
     return F <= 256 || (bits < 8 && (F + 3) / 4 * (8 / bits) <= 12 * 64);
 }
 
