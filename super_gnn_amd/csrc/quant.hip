@@ -1008,6 +1008,40 @@ __global__ __launch_bounds__(64 * WAVES) void quant_pack_stream_kernel(
 #pragma unroll
     for (int v = 0; v < NV; ++v)   // slots behind the chunk's last vector hold copies of it: their codes are zero
         if ((v >= n_full && v * 64 + lane > last) || ((dead_mask >> v) & 1u)) words[v] = 0;
+    if constexpr (EPB == 1 && RAGGED) {
+        // int8, rows that are not whole words or an output that is not word-aligned: code byte j of row slot p is
+        // output byte p * F + j, so every lane stores its words where they belong, at whatever alignment.  A row's
+        // short last word is filled up with the first bytes of the next row's first word (the next vector slot:
+        // the next lane, or lane 0's next vector), which that slot writes too -- the same bytes, so the order of
+        // the two stores does not matter; the chunk's last row has no next one and goes out byte by byte.
+        const int nt = F & 3;
+        const int n_sl = ng * VPR;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int sl = v * 64 + lane;
+            const int pr = prv[v];
+            const int cv = (sl < n_sl ? sl : n_sl - 1) - pr * VPR;
+            uint32_t w = words[v];
+            const bool sh = nt != 0 && cv == VPR - 1;
+            if (nt != 0) {
+                uint32_t nxt = (uint32_t)__shfl_down((int)words[v], 1, 64);
+                if (v + 1 < NV) {
+                    const uint32_t first_of_next = (uint32_t)__builtin_amdgcn_readfirstlane((int)words[v + 1]);
+                    if (lane == 63) nxt = first_of_next;
+                }
+                if (sh) w = (w & ((1u << (8 * nt)) - 1u)) | (nxt << (8 * nt));
+            }
+            if (sl < n_sl) {
+                uint8_t *dst = out_run + pr * F + 4 * cv;
+                if (sh && pr == ng - 1) {
+                    for (int t = 0; t < nt; ++t) dst[t] = (uint8_t)(w >> (8 * t));
+                } else {
+                    u32_store_nt_unaligned(dst, w);
+                }
+            }
+        }
+        return;
+    }
     if (EPB == 1 && !RAGGED) {   // code words are output words
         uint32_t *q32 = reinterpret_cast<uint32_t *>(out_run);
 #pragma unroll
