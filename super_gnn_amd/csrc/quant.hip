@@ -675,7 +675,7 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows16_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
-// Fused quantize + pack over a run of consecutive row slots: any row width from 16 floats; the rows themselves are
+// Fused quantize + pack over a run of consecutive row slots: any row width from 9 floats; the rows themselves are
 // consecutive in memory (the fast case) or found through a table (a row index, a pitch, a chunk across two segments).
 //
 // A wavefront takes `gw` consecutive packed rows, i.e. gw * EPB fp32 rows (at most 64), which lie one after the
@@ -2272,7 +2272,9 @@ static void launch_quant_stream_nv(const RowsArgs &a, int gw, hipStream_t st) {
 template <int BITS>
 static bool launch_quant_stream(const RowsArgs &a, hipStream_t st) {
     int nv = 0, gw = 0;
-    if (a.x_in.ld < a.F || a.x_in.n_src >= ((int64_t)1 << 31) || a.F < 16) return false;
+    // (from 9 floats: three vectors per row fill 3/4 of the slots of 64 rows x four vectors, and the tensor holds the four
+    //  floats the last load needs; narrower rows are faster with the lane-group kernels: F = 8 6.6 against 5.9 TB/s)
+    if (a.x_in.ld < a.F || a.x_in.n_src >= ((int64_t)1 << 31) || a.F < 9) return false;
     const bool ragged = a.F % 4 != 0 || !aligned(a.q_out, 4);
     if (!stream_shape(a.F, 8 / BITS, ragged, &nv, &gw)) return false;
 #define SGNN_STREAM(NV_)                                                       \
