@@ -92,6 +92,55 @@ def test_quant_random_shapes(case):
     assert np.all(np.abs(back.cpu().numpy() - want) <= tol), f"case {case}"
 
 
+@pytest.mark.parametrize("stream", ["default", "1", "0"])
+@pytest.mark.parametrize("case", range(40))
+def test_quant_rows_by_index_pitch_and_special_values(case, stream, monkeypatch):
+    """Quantizer input rows that are consecutive, picked by a row index (repeats, the source's last row), read with a
+    pitch out of a wider tensor, or both; rows with a NaN first / later, infinities, zeros of both signs, constants;
+    ragged per-peer segments; output at odd addresses -- under the default choice of kernel and with either
+    quantizer family forced (SGNN_QUANT_STREAM).  Bytes and params bit for bit against the oracle on the gathered copy."""
+    from super_gnn_amd import supergnn_ops as ops
+    if stream != "default":
+        monkeypatch.setenv("SGNN_QUANT_STREAM", stream)
+    rng = np.random.default_rng(7000 + case)
+    F = int(rng.choice([9, 10, 12, 13, 16, 17, 33, 37, 64, 100, 123, 128, 250, 256, 301, 602, 640, 1000, 1026, 1433, 2050]))
+    n = int(rng.integers(1, 2500)) if F < 1100 else int(rng.integers(1, 300))
+    bits = int(rng.choice([8, 4, 2]))
+    P = int(rng.choice([1, 1, 2, 5, 13, 64, 65]))
+    mode = case % 4                             # 0 consecutive, 1 index, 2 pitch, 3 index + pitch
+    n_src = n if mode in (0, 2) else int(rng.integers(1, 2 * n + 2))
+    pitch = F if mode in (0, 1) else F + int(rng.integers(1, 9))
+    col0 = 0 if pitch == F else int(rng.integers(0, pitch - F + 1))
+    src = (rng.standard_normal((n_src, pitch)) * np.exp(rng.uniform(-3, 3, size=(n_src, 1)))).astype(np.float32)
+    for r in rng.integers(0, n_src, size=max(1, n_src // 7)):
+        kind, c = int(rng.integers(0, 6)), col0 + int(rng.integers(0, F))
+        row = src[r, col0:col0 + F]
+        if kind == 0: row[0] = np.nan
+        elif kind == 1: src[r, c] = np.nan
+        elif kind == 2: src[r, c] = np.inf if rng.random() < 0.5 else -np.inf
+        elif kind == 3: row[:] = np.abs(row); src[r, c] = -0.0 if rng.random() < 0.5 else 0.0; row[int(rng.integers(0, F))] = 0.0
+        elif kind == 4: row[:] = np.float32(rng.standard_normal())
+        else: row[:] = -np.abs(row); src[r, c] = 0.0; row[int(rng.integers(0, F))] = -0.0
+    idx = rng.integers(0, n_src, size=n) if mode in (1, 3) else None
+    if idx is not None and n > 2:
+        idx[int(rng.integers(0, n))] = n_src - 1
+    x = np.ascontiguousarray((src[idx] if idx is not None else src)[:, col0:col0 + F])
+    seg = [0] + [int(c) for c in np.sort(rng.integers(0, n + 1, size=P - 1))] + [n]
+    q_ref, p_ref = orc.quant_rows(x, seg, bits)
+    npk, qoff = q_ref.shape[0], int(rng.integers(0, 4))
+    qb = torch.full((npk * F + 8,), 0xCD, dtype=torch.uint8, device="cuda")
+    prm = torch.zeros(n, 2, device="cuda")
+    ops.quantize_tensor_for_all_procs(torch.from_numpy(src).cuda()[:, col0:col0 + F], qb[qoff:qoff + npk * F].view(npk, F), prm,
+                                      torch.tensor(seg, dtype=torch.int32), P, bits,
+                                      row_index=None if idx is None else torch.from_numpy(idx).cuda())
+    got, pg, nan_ref = qb.cpu().numpy(), prm.cpu().numpy(), np.isnan(p_ref)
+    what = f"case {case}: n={n} F={F} bits={bits} P={P} mode={mode} pitch={pitch} col0={col0} qoff={qoff}"
+    assert np.array_equal(np.isnan(pg), nan_ref), what
+    assert np.array_equal(pg[~nan_ref].view(np.uint32), p_ref[~nan_ref].view(np.uint32)), what
+    assert np.array_equal(got[qoff:qoff + npk * F].reshape(npk, F), q_ref), what
+    assert (got[:qoff] == 0xCD).all() and (got[qoff + npk * F:] == 0xCD).all(), what + ": bytes outside the rows were written"
+
+
 @pytest.mark.parametrize("case", range(30))
 def test_fused_random_shapes(case):
     # random widths (every lane-group shape), ragged segments, hub rows, fp32 / bf16 params, all epilogues:
