@@ -103,7 +103,7 @@ def test_quant_rows_by_index_pitch_and_special_values(case, stream, monkeypatch)
     if stream != "default":
         monkeypatch.setenv("SGNN_QUANT_STREAM", stream)
     rng = np.random.default_rng(7000 + case)
-    F = int(rng.choice([9, 10, 12, 13, 16, 17, 33, 37, 64, 100, 123, 128, 250, 256, 301, 602, 640, 1000, 1026, 1433, 2050]))
+    F = int(rng.choice([9, 10, 12, 13, 16, 17, 33, 37, 64, 100, 123, 128, 250, 256, 301, 602, 640, 1000, 1026, 1433, 1538, 2050, 2562, 3703, 4100]))
     n = int(rng.integers(1, 2500)) if F < 1100 else int(rng.integers(1, 300))
     bits = int(rng.choice([8, 4, 2]))
     P = int(rng.choice([1, 1, 2, 5, 13, 64, 65]))
