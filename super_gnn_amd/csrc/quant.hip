@@ -2416,7 +2416,7 @@ static bool stream_shape(int F, int epb, bool ragged, int *nv_out, int *gw_out) 
     double best = 0.0;
     for (int k = 0; k < 6; ++k) {
         const int nv = nvs[k];
-        if (best > 0.0 && nv > 10) break;
+        if (best > 0.0 && (nv > 12 || (nv > 10 && best >= 0.8))) break;   // (twelve still competes with a poor fill)
         const int gw = std::min(nv * 64 / (epb * vpr), kStreamRows / epb);
         if (gw < 1) continue;
         const double fill = (double)gw * epb * vpr / (nv * 64);
