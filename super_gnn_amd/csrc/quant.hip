@@ -1623,19 +1623,19 @@ __global__ __launch_bounds__(kQBlock) void quant_pack_rows_wide_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
-// Rows too wide for a wavefront's registers, narrow enough for a workgroup's LDS (EPB rows of F floats in 64 KB:
-// F <= 4096 at int2, 8192 at int4, 16384 at int8): one workgroup per packed row.  The fp32 rows are read from
-// memory once, into LDS, with the min / max taken on the way; the codes are then made out of LDS.  (The two-pass
-// kernel above reads the rows twice, and at these widths the second read no longer finds them in a cache:
-// F = 3703 int2 2.7 TB/s.)
+// Rows too wide for a wavefront's registers: one workgroup per packed row, the row kept in the registers of its TB
+// threads.  Thread t holds vectors t, t + TB, ... (NVT of them) of each of the EPB rows, so the fp32 rows are read
+// once, the per-row min / max is a reduction over the workgroup (DPP inside a wavefront, a few words of LDS across
+// wavefronts), and a thread packs its own output words: the EPB code words it needs sit in its own registers.
+// F <= 4 * TB * NVT, i.e. up to 8192 floats.  (The two-pass kernel above reads the rows twice, and at these widths the
+// second read no longer finds them in a cache: F = 3703 int2 2.7 TB/s.)
 // ------------------------------------------------------------------------------------------------
-template <int BITS, int TB>
-__global__ __launch_bounds__(TB) void quant_pack_rows_lds_kernel(
+template <int BITS, int TB, int NVT>
+__global__ __launch_bounds__(TB) void quant_pack_rows_block_kernel(
     const RowSrc xs, uint8_t *__restrict__ q, const ParamBuf pb,
     const int32_t *__restrict__ seg, const int32_t *__restrict__ pseg, int P, int64_t single_rows, int n_packed, int F) {
     constexpr int EPB = 8 / BITS;
     constexpr int NW = TB / 64;
-    extern __shared__ __align__(16) float lds_rows[];   // [EPB][Fp]
     __shared__ float red_mn[NW][EPB], red_mx[NW][EPB];
     __shared__ int red_key[NW][EPB];
     __shared__ float4 rowpar[EPB];   // (zero_point, scale, 1 / scale, needs the exact division)
@@ -1643,72 +1643,52 @@ __global__ __launch_bounds__(TB) void quant_pack_rows_lds_kernel(
     const int gp = blockIdx.x;
     int64_t row0, rend;
     locate_packed_row(seg, pseg, P, single_rows, gp, gp, EPB, row0, rend);
-    const int nvf = F >> 2, n_tail = F & 3;
-    const int Fp = (F + 3) & ~3;
-    // eight loads in flight per thread: the EPB rows at the same vector index, times 8 / EPB indices
-    constexpr int UJ = 8 / EPB;
+    const int nvf = F >> 2, n_tail = F & 3;   // whole vectors of a row (1 <= nvf <= TB * NVT), elements behind them
     // (a row slot the segment's short last group leaves empty reads the group's first row again, so that no load
-    //  sits behind a condition; nothing of it is used)
+    //  sits behind a condition; nothing of it is used.  Vector slots behind the row repeat its last whole vector:
+    //  a repeat changes neither min nor max nor the first zero, and is not stored.)
     const float *xr[EPB];
-    float mn[EPB], mx[EPB];
-    int key[EPB];
+    float v[NVT][EPB][4], e_tail[EPB];
+#pragma unroll
+    for (int k = 0; k < EPB; ++k) xr[k] = row_ptr(xs, row0 + k < rend ? row0 + k : row0);
+#pragma unroll
+    for (int u = 0; u < NVT; ++u) {
+        const int j = u * TB + tid < nvf ? u * TB + tid : nvf - 1;
+#pragma unroll
+        for (int k = 0; k < EPB; ++k) vec4_load_nt_unaligned(v[u][k], xr[k] + 4 * j);
+    }
+#pragma unroll
+    for (int k = 0; k < EPB; ++k) e_tail[k] = tid < n_tail ? xr[k][4 * nvf + tid] : 0.0f;
 #pragma unroll
     for (int k = 0; k < EPB; ++k) {
-        xr[k] = row_ptr(xs, row0 + k < rend ? row0 + k : row0);
-        mn[k] = INFINITY;
-        mx[k] = -INFINITY;
-        key[k] = INT_MAX;
-    }
-    auto take = [&](const float (&v)[4], int k, int j) {   // vector j of row k: into LDS, into the row's min / max / first zero
-        *reinterpret_cast<float4 *>(lds_rows + k * Fp + 4 * j) = make_float4(v[0], v[1], v[2], v[3]);
+        float mn = INFINITY, mx = -INFINITY;
+        int key = INT_MAX;
 #pragma unroll
-        for (int t = 3; t >= 0; --t) {
-            mn[k] = fminf(mn[k], v[t]);
-            mx[k] = fmaxf(mx[k], v[t]);
+        for (int u = 0; u < NVT; ++u) {
+            const int j = u * TB + tid < nvf ? u * TB + tid : nvf - 1;
+#pragma unroll
+            for (int t = 3; t >= 0; --t) {
+                mn = fminf(mn, v[u][k][t]);
+                mx = fmaxf(mx, v[u][k][t]);
+            }
+            if (key == INT_MAX) {
+#pragma unroll
+                for (int t = 3; t >= 0; --t)
+                    if (v[u][k][t] == 0.0f) key = ((4 * j + t) << 1) | (int)(__float_as_uint(v[u][k][t]) >> 31);
+            }
         }
-        if (key[k] == INT_MAX) {
-#pragma unroll
-            for (int t = 3; t >= 0; --t)
-                if (v[t] == 0.0f) key[k] = ((4 * j + t) << 1) | (int)(__float_as_uint(v[t]) >> 31);
-        }
-    };
-    int jb = 0;   // first vector index of the round (uniform)
-    for (; jb + TB * UJ <= nvf; jb += TB * UJ) {   // whole rounds: UJ indices x EPB rows in flight per thread
-        float v[UJ][EPB][4];
-#pragma unroll
-        for (int u = 0; u < UJ; ++u) {
-#pragma unroll
-            for (int k = 0; k < EPB; ++k) vec4_load_nt_unaligned(v[u][k], xr[k] + 4 * (jb + TB * u + tid));
-        }
-#pragma unroll
-        for (int u = 0; u < UJ; ++u) {
-#pragma unroll
-            for (int k = 0; k < EPB; ++k) take(v[u][k], k, jb + TB * u + tid);
-        }
-    }
-    for (int j = jb + tid; j < nvf; j += TB) {   // the rest: one index x EPB rows
-        float v[EPB][4];
-#pragma unroll
-        for (int k = 0; k < EPB; ++k) vec4_load_nt_unaligned(v[k], xr[k] + 4 * j);
-#pragma unroll
-        for (int k = 0; k < EPB; ++k) take(v[k], k, j);
-    }
-#pragma unroll
-    for (int k = 0; k < EPB; ++k) {
         if (tid < n_tail) {
-            const float e = xr[k][4 * nvf + tid];
-            lds_rows[k * Fp + 4 * nvf + tid] = e;
-            mn[k] = fminf(mn[k], e);
-            mx[k] = fmaxf(mx[k], e);
-            if (e == 0.0f) key[k] = min(key[k], ((4 * nvf + tid) << 1) | (int)(__float_as_uint(e) >> 31));
+            mn = fminf(mn, e_tail[k]);
+            mx = fmaxf(mx, e_tail[k]);
+            if (e_tail[k] == 0.0f) key = min(key, ((4 * nvf + tid) << 1) | (int)(__float_as_uint(e_tail[k]) >> 31));
         }
-        const float wmn = group_allreduce_f<64, OpMinF>(mn[k]);
-        const float wmx = group_allreduce_f<64, OpMaxF>(mx[k]);
-        const int wkey = group_allmin_i<64>(key[k]);
+        mn = group_allreduce_f<64, OpMinF>(mn);
+        mx = group_allreduce_f<64, OpMaxF>(mx);
+        key = group_allmin_i<64>(key);
         if (lane == 0) {
-            red_mn[wave][k] = wmn;
-            red_mx[wave][k] = wmx;
-            red_key[wave][k] = wkey;
+            red_mn[wave][k] = mn;
+            red_mx[wave][k] = mx;
+            red_key[wave][k] = key;
         }
     }
     __syncthreads();
@@ -1725,7 +1705,7 @@ __global__ __launch_bounds__(TB) void quant_pack_rows_lds_kernel(
         const float z = (key & 1) ? -0.0f : 0.0f;
         if (mn == 0.0f) mn = z;
         if (mx == 0.0f) mx = z;
-        const float first = lds_rows[k * Fp];
+        const float first = row_ptr(xs, row0 + k)[0];
         if (first != first) { mn = first; mx = first; }
         float s = (mx - mn) / (float)((1 << BITS) - 1);
         if (s == 0.0f) s = 1.0f;
@@ -1734,20 +1714,22 @@ __global__ __launch_bounds__(TB) void quant_pack_rows_lds_kernel(
     }
     __syncthreads();
     constexpr float kGuard = BITS == 8 ? 0x1p-13f : BITS == 4 ? 0x1p-17f : 0x1p-19f;
+    float4 par[EPB];
+#pragma unroll
+    for (int k = 0; k < EPB; ++k) par[k] = rowpar[k];
     uint8_t *qr = q + (int64_t)gp * F;
-    for (int j = tid; j < nvf; j += TB) {
+#pragma unroll
+    for (int u = 0; u < NVT; ++u) {
+        const int j = u * TB + tid;
         uint32_t word = 0;
 #pragma unroll
         for (int k = 0; k < EPB; ++k) {
             if (row0 + k >= rend) continue;
-            const float4 par = rowpar[k];
-            const float4 v4 = *reinterpret_cast<const float4 *>(lds_rows + k * Fp + 4 * j);
-            const float v[4] = {v4.x, v4.y, v4.z, v4.w};
             uint32_t w = 0;
-            bool redo = par.w != 0.0f;
+            bool redo = par[k].w != 0.0f;
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                const float qf = (v[t] - par.x) * par.z;
+                const float qf = (v[u][k][t] - par[k].x) * par[k].z;
                 const float ri = rintf(qf);
                 if (!(fabsf(qf - ri) < 0.5f - kGuard)) redo = true;
                 w = __builtin_amdgcn_cvt_pk_u8_f32(ri, t, w);
@@ -1755,20 +1737,19 @@ __global__ __launch_bounds__(TB) void quant_pack_rows_lds_kernel(
             if (redo) {
                 w = 0;
 #pragma unroll
-                for (int t = 0; t < 4; ++t) w |= quant_code(v[t], par.x, par.y) << (8 * t);
+                for (int t = 0; t < 4; ++t) w |= quant_code(v[u][k][t], par[k].x, par[k].y) << (8 * t);
             }
             word |= w << ((EPB - 1 - k) * BITS);
         }
-        u32_store_nt_unaligned(qr + 4 * j, word);
+        if (j < nvf) u32_store_nt_unaligned(qr + 4 * j, word);
     }
     if (tid < n_tail) {
-        const int c = 4 * nvf + tid;
         uint32_t byte = 0;
 #pragma unroll
         for (int k = 0; k < EPB; ++k) {
-            if (row0 + k < rend) byte |= quant_code(lds_rows[k * Fp + c], rowpar[k].x, rowpar[k].y) << ((EPB - 1 - k) * BITS);
+            if (row0 + k < rend) byte |= quant_code(e_tail[k], par[k].x, par[k].y) << ((EPB - 1 - k) * BITS);
         }
-        qr[c] = (uint8_t)byte;
+        qr[4 * nvf + tid] = (uint8_t)byte;
     }
 }
 
@@ -2535,21 +2516,23 @@ static void launch_dequant_flat_ragged(const RowsArgs &a, int64_t n_rows, hipStr
     else launch_dequant_flat_ragged_r<BITS, VEC, 2>(a, n_rows, st);
 }
 
-// EPB rows of F floats (padded to whole float4) beside the kernel's few hundred static bytes in a workgroup's 64 KB.
-static bool rows_fit_lds(int F, int bits) {
-    return (size_t)(8 / bits) * (size_t)((F + 3) & ~3) * sizeof(float) <= 60 * 1024;
-}
+// Rows the workgroup-per-packed-row kernel holds in registers: at most 4 * 512 * 4 floats.
+static bool rows_fit_block(int F) { return F >= 4 && F / 4 <= 512 * 4; }
 template <int BITS>
-static void launch_quant_lds(const RowsArgs &a, hipStream_t st) {
-    const size_t lds_bytes = (size_t)(8 / BITS) * (size_t)((a.F + 3) & ~3) * sizeof(float);
+static void launch_quant_block(const RowsArgs &a, hipStream_t st) {
+    const int nvf = a.F / 4;
     ProfScope prof(K_QUANT_PACK_ROWS, st);
-    // rows that leave room for only two or three workgroups per CU get workgroups of eight wavefronts
-    if (lds_bytes > 32 * 1024)
-        hipLaunchKernelGGL((quant_pack_rows_lds_kernel<BITS, 512>), dim3(a.n_packed), dim3(512), lds_bytes, st, a.x_in, a.q_out,
-                           a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F);
-    else
-        hipLaunchKernelGGL((quant_pack_rows_lds_kernel<BITS, 256>), dim3(a.n_packed), dim3(256), lds_bytes, st, a.x_in, a.q_out,
-                           a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F);
+#define SGNN_BLOCKQ(TB_, NVT_)                                                                                              \
+    hipLaunchKernelGGL((quant_pack_rows_block_kernel<BITS, TB_, NVT_>), dim3(a.n_packed), dim3(TB_), 0, st, a.x_in, a.q_out, \
+                       a.params, a.seg, a.pseg, a.P, a.single_rows, a.n_packed, a.F)
+    // the fewest vectors per thread that hold the row, in the smaller workgroup where both do
+    if (nvf <= 256) SGNN_BLOCKQ(256, 1);
+    else if (nvf <= 512) SGNN_BLOCKQ(256, 2);
+    else if (nvf <= 768) SGNN_BLOCKQ(256, 3);
+    else if (nvf <= 1024) SGNN_BLOCKQ(512, 2);
+    else if (nvf <= 1536) SGNN_BLOCKQ(512, 3);
+    else SGNN_BLOCKQ(512, 4);
+#undef SGNN_BLOCKQ
 }
 
 template <int BITS>
@@ -2656,18 +2639,18 @@ static int run_rows(const RowsArgs &a, int bits, int64_t n_rows, const void *fp3
     SGNN_REQUIRE(aligned(a.params.p, a.params.bf16 ? 4 : 8), "params must be %d-byte aligned", a.params.bf16 ? 4 : 8);
     const int stream = env_flag("SGNN_QUANT_STREAM", -1);   // 1: every width the stream quantizer can take, 0: never
     bool taken = false;
-    const bool lds_rows_wanted = a.F > 1536 && rows_fit_lds(a.F, bits);
-    if (a.quantize && !a.exact_division && (stream > 0 || (stream < 0 && !lds_rows_wanted && stream_wanted(a.F, vec, bits, a.x_in.index != nullptr || a.x_in.ld != a.F))))
+    const bool block_rows_wanted = a.F > (bits == 2 ? 1280 : 1920) && rows_fit_block(a.F);
+    if (a.quantize && !a.exact_division && (stream > 0 || (stream < 0 && !block_rows_wanted && stream_wanted(a.F, vec, bits, a.x_in.index != nullptr || a.x_in.ld != a.F))))
         taken = bits == 8 ? launch_quant_stream<8>(a, st) : bits == 4 ? launch_quant_stream<4>(a, st) : launch_quant_stream<2>(a, st);
     if (taken) {
-    } else if (a.quantize && !a.exact_division && lds_rows_wanted) {
-        // rows a wavefront cannot hold, or holds only with few wavefronts per CU: a workgroup per packed row, the rows
-        // staged in LDS (F = 2050: 5.0 / 5.0 / 3.5 -> 5.2 / 5.6 / 4.7 TB/s at int8 / int4 / int2, F = 3703: 4.9 / 2.6 / 2.7 ->
-        // 5.8 / 5.3 / 4.4; up to 1536 floats the stream and lane-group kernels are ahead: F = 1433 5.0 / 5.4 / 4.7 against
-        // 4.1 / 4.8 / 4.4)
-        if (bits == 8) launch_quant_lds<8>(a, st);
-        else if (bits == 4) launch_quant_lds<4>(a, st);
-        else launch_quant_lds<2>(a, st);
+    } else if (a.quantize && !a.exact_division && block_rows_wanted) {
+        // rows a wavefront cannot hold (int2 beyond 1280 floats), or holds only with few wavefronts per CU: a workgroup
+        // per packed row, the rows in its registers (F = 2050: 5.0 / 5.0 / 3.5 -> 5.9 / 6.1 / 5.8 TB/s at int8 / int4 / int2,
+        // F = 3703: 4.9 / 2.6 / 2.7 -> 5.7 / 5.9 / 5.8, F = 1433 int2: 4.7 -> 5.6; at int8 / int4 the stream kernel is ahead up to
+        // about 1900 floats: F = 1700 6.3 / 6.2 against 5.6 / 6.0)
+        if (bits == 8) launch_quant_block<8>(a, st);
+        else if (bits == 4) launch_quant_block<4>(a, st);
+        else launch_quant_block<2>(a, st);
     } else if (!a.quantize && vec == 4 && a.flat) {
         if (bits == 8) launch_dequant_flat<8>(a, n_rows, st);
         else if (bits == 4) launch_dequant_flat<4>(a, n_rows, st);
